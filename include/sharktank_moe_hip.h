@@ -1,0 +1,179 @@
+/*
+ * C ABI of the MI355X (gfx950) quantized mixture-of-experts kernels.
+ *
+ * The library computes what sharktank's eager `MoeBlock` / `PreGatherFFNMOE`
+ * compute (sharktank/sharktank/layers/mixture_of_experts_block.py:64-90,
+ * sharktank/sharktank/layers/ffn_moe_block.py:60-74) and what its IREE custom
+ * ops `mmt_block_scaled_q8`, `mmt_block_scaled_offset_q4_unsigned` and
+ * `einsum_2args_q4` compute (sharktank/sharktank/kernels/ *.py), on device
+ * pointers, without any torch type in a signature.
+ *
+ * Conventions for every entry point:
+ *   - all pointers are device pointers unless the comment says "host";
+ *   - tensors are dense row-major; quantized planes are the planar planes of
+ *     the reference layouts (`d`, `qs`, `m`), made contiguous by the caller;
+ *   - the caller owns all memory, including the workspace; the library
+ *     allocates nothing, never synchronises and only enqueues on `stream`
+ *     (a hipStream_t passed as void*; NULL is the default stream);
+ *   - the return value is a stmoe_status; stmoe_last_error() returns a
+ *     thread-local, human-readable description of the last non-zero status.
+ */
+#ifndef SHARKTANK_MOE_HIP_H_
+#define SHARKTANK_MOE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* stmoe_stream_t;
+
+typedef enum {
+  STMOE_OK = 0,
+  STMOE_ERR_NULL = 1,        /* a required pointer is NULL */
+  STMOE_ERR_SHAPE = 2,       /* a size is negative, zero where it may not be, or not a multiple the kernel needs */
+  STMOE_ERR_DTYPE = 3,       /* dtype enum out of range or combination not implemented */
+  STMOE_ERR_ALIGN = 4,       /* a pointer is not aligned to 16 bytes */
+  STMOE_ERR_UNSUPPORTED = 5, /* layout / format combination not implemented */
+  STMOE_ERR_WORKSPACE = 6,   /* workspace smaller than *_workspace_bytes() */
+  STMOE_ERR_LAUNCH = 7       /* hipGetLastError() after a launch was not hipSuccess */
+} stmoe_status;
+
+typedef enum {
+  STMOE_F32 = 0,
+  STMOE_F16 = 1,
+  STMOE_BF16 = 2,
+  STMOE_F8E4M3FN = 3, /* OCP e4m3 (torch.float8_e4m3fn), the fp8 format of gfx950 MFMA */
+  STMOE_I8 = 4,
+  STMOE_U8 = 5
+} stmoe_dtype;
+
+typedef enum {
+  STMOE_ACT_SILU = 0,    /* torch.nn.functional.silu */
+  STMOE_ACT_GELU_ERF = 1 /* torch.nn.functional.gelu, exact erf form */
+} stmoe_act;
+
+typedef enum {
+  STMOE_W_DENSE = 0, /* DefaultPrimitiveTensor: qs = elements of `dtype` */
+  STMOE_W_Q8_0 = 1,  /* BlockScaledLayout, block 32: d fp16 [.,K/32], qs int8 [.,K/32,32] */
+  STMOE_W_Q4_1 = 2,  /* BlockScaledI4Layout, block 32, unsigned: d,m fp16 [.,K/32], qs u8 [.,K/32,16] */
+  STMOE_W_FP8 = 3    /* TensorScaledLayout: qs e4m3fn [.,K], d = d_count scales of `dtype` (f32 or f16) */
+} stmoe_wfmt;
+
+/* One stacked expert weight `[experts, rows, cols]`, used as x @ W[e]^T. */
+typedef struct stmoe_weight {
+  int32_t format;  /* stmoe_wfmt */
+  int32_t dtype;   /* DENSE: element dtype (F32/F16/BF16); FP8: dtype of d (F32/F16); else ignored */
+  int64_t experts; /* E; 1 for a plain matrix */
+  int64_t rows;    /* output features of the projection */
+  int64_t cols;    /* reduction length; multiple of 32 for the block formats */
+  const void* qs;
+  const void* d;   /* NULL for DENSE */
+  const void* m;   /* Q4_1 only */
+  int64_t d_count; /* FP8: 1 (one scale per tensor) or `experts` (one per expert) */
+} stmoe_weight;
+
+const char* stmoe_last_error(void);
+int stmoe_abi_version(void);
+
+/* ---- dequantization (bit-exact with the reference layouts' dequant()) ---------------------- */
+
+/* BlockScaledLayout.dequant (sharktank/sharktank/types/layouts.py:274-290):
+ * out[b,i] = D(d[b]) * D(qs[b,i]) (+ D(m[b])), every step rounded in out_dtype D. */
+int stmoe_dequant_block_scaled(const void* d, const void* m /*nullable*/, int dm_dtype,
+                               const int8_t* qs, int64_t n_blocks, int block_size,
+                               void* out, int out_dtype, stmoe_stream_t stream);
+
+/* BlockScaledI4Layout.dequant (layouts.py:302-357 + layout_utils.py:67-86): nibbles in linear
+ * little-endian order (element 2i = low nibble of byte i), unsigned or sign-extended. */
+int stmoe_dequant_block_scaled_i4(const void* d, const void* m /*nullable*/, int dm_dtype,
+                                  const uint8_t* qs_packed, int64_t n_blocks, int block_size,
+                                  int is_signed, void* out, int out_dtype, stmoe_stream_t stream);
+
+/* promote_linear_i4_block_to_i8 (layout_utils.py:67-86): n_bytes packed bytes -> 2*n_bytes (u)int8. */
+int stmoe_promote_i4(const uint8_t* qs_packed, int64_t n_bytes, int is_signed, void* out,
+                     stmoe_stream_t stream);
+
+/* TensorScaledLayout.dequant (layouts.py:163-181): out = ((D(qs) - m) * d).to(out_dtype) with
+ * D = d_dtype. `d`/`m` hold d_count values; value j applies to elements [j*n/d_count, (j+1)*n/d_count). */
+int stmoe_dequant_tensor_scaled(const void* qs, int qs_dtype, const void* d, const void* m /*nullable*/,
+                                int d_dtype, int64_t d_count, int64_t n, void* out, int out_dtype,
+                                stmoe_stream_t stream);
+
+/* StaticScaledQuantizer per-tensor quantize to fp8 (sharktank/sharktank/types/quantizers.py:153-183 with
+ * saturate_cast, layout_utils.py:150-176): out = e4m3fn(clamp(x / rscale, -448, 448)); the quotient is
+ * computed in fp32 and rounded to x's dtype before the clamp.  `rscale` points to one device float. */
+int stmoe_quantize_fp8(const void* x, int x_dtype, const float* rscale, int64_t n, void* out_fp8,
+                       stmoe_stream_t stream);
+
+/* ---- layer pieces ----------------------------------------------------------------------------- */
+
+/* RMSNormLayer.forward (sharktank/sharktank/layers/norm.py:34-41) with rms_norm_default
+ * (sharktank/sharktank/ops/default_impls.py:402-408): fp32 statistics, weight `w` of w_dtype, result
+ * rounded to the dtype of x.  x, out: [T, K]. */
+int stmoe_rms_norm(const void* x, int dtype, const void* w, int w_dtype, int64_t T, int64_t K, float eps,
+                   void* out, stmoe_stream_t stream);
+
+/* Router of MoeBlock.forward (mixture_of_experts_block.py:70-83): logits = x @ Wr^T rounded to `dtype`,
+ * fp32 softmax over E, top-k (descending; equal logits -> lower expert index first), gates renormalised
+ * in fp32 then rounded to `dtype`.  Wr [E,K] is given in `dtype`.  K % 8 == 0, E <= 64, k <= E.
+ * logits_out ([T,E], `dtype`) and idx64_out ([T,k], int64) may be NULL. */
+int stmoe_router_topk(const void* x, const void* w_router, int dtype, int64_t T, int64_t K, int E, int k,
+                      void* logits_out, int32_t* idx_out, int64_t* idx64_out, void* gate_out,
+                      stmoe_stream_t stream);
+
+/* Token-to-expert dispatch: a stable counting sort of the n_pairs = T*k (token, slot) pairs
+ * p = t*k + j by expert id.  counts[E]; offsets[E+1] = exclusive scan; perm[offsets[e]+r] = the r-th
+ * pair of expert e in increasing p; inv[perm[i]] = i.  The reference has no such step (it gathers
+ * weights per token instead, ffn_moe_block.py:37-41); this is what replaces it. */
+int stmoe_dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets,
+                         int32_t* perm, int32_t* inv, stmoe_stream_t stream);
+
+/* Workspace for stmoe_grouped_ffn / stmoe_moe_forward (bytes; depends on sizes only). */
+size_t stmoe_grouped_ffn_workspace_bytes(int64_t T, int k, int64_t K, int64_t N, int dtype);
+size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int64_t K, int64_t N, int dtype);
+
+/* Gated expert FFN of PreGatherFFNMOE.forward (ffn_moe_block.py:60-72) over rows grouped by expert:
+ * for sorted position i (pair p = perm[i], token t = p / k, expert e with offsets[e] <= i < offsets[e+1])
+ *   y[i,:] = Wd[e] . ( act(Wg[e] . x[t]) * (Wu[e] . x[t]) )
+ * with each intermediate rounded to `dtype` where the reference materialises a tensor.  x [T,K];
+ * y [T*k, K] in `dtype`.  `x_scale` (nullable, device float) is the reciprocal scale of fp8-quantised
+ * activations: when given with FP8 weights, x is taken as e4m3fn [T,K] and results are scaled by it.
+ * `variant` 0 picks the kernel by shape; other values force one (see the kernel list in ffn.hip). */
+int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                      const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
+                      int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
+                      void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
+                      stmoe_stream_t stream);
+
+/* Weighted combine (ffn_moe_block.py:73-74) and the layer tail (mixture_of_experts_block.py:86-90):
+ *   o[t,:] = sum_j round(gate[t,j] * y[inv[t*k+j],:])   (slot order, fp32 sum, rounded to `dtype`)
+ *   o = rms_norm(o; out_norm_w, eps) if out_norm_w != NULL     (layer_output_norm)
+ *   out[t,:] = residual[t,:] + o[t,:] if residual != NULL      (h + moe_output)   */
+int stmoe_combine(const void* y_sorted, const void* gate, const int32_t* inv, int dtype, int64_t T, int k,
+                  int64_t K, const void* out_norm_w /*nullable*/, int w_dtype, float eps,
+                  const void* residual /*nullable*/, void* out, stmoe_stream_t stream);
+
+/* Whole MoeBlock.forward (mixture_of_experts_block.py:64-90) on h [T,K] -> out [T,K]:
+ * ffn_norm -> router -> dispatch -> grouped FFN -> combine (+ layer_output_norm) + residual.
+ * ffn_norm_w / out_norm_w are of w_dtype; out_norm_w may be NULL.  idx_out/gate_out ([T,k]) may be NULL. */
+int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                      const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
+                      const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
+                      const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
+                      void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream);
+
+/* x @ W^T for one quantised (or dense) matrix W [rows, cols]: the operand set of the reference's
+ * `mmt_block_scaled_q8(a,d,qs)` (sharktank/sharktank/kernels/mmt_block_scaled_q8.py:30) and
+ * `mmt_block_scaled_offset_q4_unsigned(a,d,qs,m)` (mmt_block_scaled_offset_q4.py:31), reached from
+ * ops.matmul(Tensor, QuantizedTensor, transpose_rhs=True) (sharktank/sharktank/ops/custom_impls.py:66-103).
+ * a [M,K], out [M,rows], both `dtype`; fp32 accumulation. */
+int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight* w, void* out, int variant,
+              stmoe_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SHARKTANK_MOE_HIP_H_ */

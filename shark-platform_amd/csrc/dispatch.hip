@@ -1,0 +1,153 @@
+// Token-to-expert dispatch (histogram, exclusive scan, stable permutation) and the weighted combine.
+//
+// The reference has no dispatch step: it gathers expert weights per token
+// (sharktank/sharktank/layers/ffn_moe_block.py:37-41).  Grouping rows by expert instead needs a
+// permutation; it is defined as the stable counting sort of the pairs p = t*k + j by expert id, so it
+// is a pure function of the routing indices and can be checked bit for bit.
+#include "stmoe_common.h"
+
+namespace stmoe {
+
+static constexpr int kDispatchThreads = 1024;
+static constexpr int kDispatchWaves = kDispatchThreads / 64;
+
+// One workgroup walks the pairs in chunks of 1024, in order.  LDS: base[E] (next free position of each
+// expert) and wcnt[16][E] (per-wave counts of the current chunk).
+__global__ void __launch_bounds__(kDispatchThreads)
+dispatch_build_kernel(const int32_t* __restrict__ idx, int64_t n, int E, int32_t* __restrict__ counts,
+                      int32_t* __restrict__ offsets, int32_t* __restrict__ perm, int32_t* __restrict__ inv) {
+  extern __shared__ int32_t sm[];
+  int32_t* base = sm;
+  int32_t* wcnt = sm + E;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  for (int e = tid; e < E; e += kDispatchThreads) base[e] = 0;
+  __syncthreads();
+  for (int64_t i = tid; i < n; i += kDispatchThreads) {
+    int e = idx[i];
+    e = e < 0 ? 0 : (e >= E ? E - 1 : e);  // out-of-range ids are a caller error; clamp to stay in bounds
+    atomicAdd(&base[e], 1);                // integer LDS atomics: the counts do not depend on their order
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int32_t run = 0;
+    for (int e = 0; e < E; ++e) {
+      const int32_t c = base[e];
+      counts[e] = c;
+      offsets[e] = run;
+      base[e] = run;
+      run += c;
+    }
+    offsets[E] = run;
+  }
+  __syncthreads();
+
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int64_t c0 = 0; c0 < n; c0 += kDispatchThreads) {
+    const int64_t i = c0 + tid;
+    int e = -1;
+    if (i < n) {
+      e = idx[i];
+      e = e < 0 ? 0 : (e >= E ? E - 1 : e);
+    }
+    int my_rank = 0;
+    for (int ee = 0; ee < E; ++ee) {
+      const uint64_t mask = __ballot(e == ee);
+      if (e == ee) my_rank = __popcll(mask & lt_mask);
+      if (lane == 0) wcnt[wave * E + ee] = __popcll(mask);
+    }
+    __syncthreads();
+    if (i < n) {
+      int32_t pos = base[e] + my_rank;
+      for (int w = 0; w < wave; ++w) pos += wcnt[w * E + e];
+      perm[pos] = (int32_t)i;
+      inv[i] = pos;
+    }
+    __syncthreads();
+    for (int ee = tid; ee < E; ee += kDispatchThreads) {
+      int32_t s = 0;
+      for (int w = 0; w < kDispatchWaves; ++w) s += wcnt[w * E + ee];
+      base[ee] += s;
+    }
+    __syncthreads();
+  }
+}
+
+// One workgroup per token.  o = sum over slots of round(gate * y) (fp32 sum in slot order, rounded to T);
+// optional RMS norm of o; optional residual add.
+template <typename T, typename W>
+__global__ void __launch_bounds__(256)
+combine_kernel(const T* __restrict__ y, const T* __restrict__ gate, const int32_t* __restrict__ inv, int k,
+               int64_t K, const W* __restrict__ norm_w, float eps, const T* __restrict__ residual,
+               T* __restrict__ out) {
+  __shared__ float partial[4];
+  const int64_t t = blockIdx.x;
+  T* orow = out + t * K;
+  float ss = 0.0f;
+  for (int64_t i = threadIdx.x; i < K; i += 256) {
+    float acc = 0.0f;
+    for (int j = 0; j < k; ++j) {
+      const int64_t r = inv[t * k + j];
+      const float g = Cvt<T>::to_f32(gate[t * k + j]);
+      acc += round_to<T>(__fmul_rn(g, Cvt<T>::to_f32(y[r * K + i])));
+    }
+    const float o = round_to<T>(acc);
+    if (norm_w) {
+      ss = fmaf(o, o, ss);
+      orow[i] = Cvt<T>::from_f32(o);
+    } else {
+      const float r = residual ? round_to<T>(Cvt<T>::to_f32(residual[t * K + i]) + o) : o;
+      orow[i] = Cvt<T>::from_f32(r);
+    }
+  }
+  if (!norm_w) return;
+  ss = wave_xor_sum(ss);
+  if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float total = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+  const float rs = 1.0f / sqrtf(total / (float)K + eps);
+  for (int64_t i = threadIdx.x; i < K; i += 256) {  // each thread re-reads only what it wrote itself
+    float o = round_to<W>(Cvt<T>::to_f32(orow[i]) * rs);
+    o = round_to<T>(round_to<W>(Cvt<W>::to_f32(norm_w[i]) * o));
+    if (residual) o = round_to<T>(Cvt<T>::to_f32(residual[t * K + i]) + o);
+    orow[i] = Cvt<T>::from_f32(o);
+  }
+}
+
+}  // namespace stmoe
+
+using namespace stmoe;
+
+extern "C" int stmoe_dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets,
+                                    int32_t* perm, int32_t* inv, stmoe_stream_t stream) {
+  STMOE_REQUIRE(n_pairs >= 0 && n_pairs < 0x7fffffffLL, STMOE_ERR_SHAPE, "dispatch_build: n_pairs=%lld", (long long)n_pairs);
+  STMOE_REQUIRE(E >= 1 && E <= 1024, STMOE_ERR_SHAPE, "dispatch_build: expert count %d outside 1..1024", E);
+  STMOE_REQUIRE(counts && offsets, STMOE_ERR_NULL, "dispatch_build: counts/offsets NULL");
+  STMOE_REQUIRE(n_pairs == 0 || (idx && perm && inv), STMOE_ERR_NULL, "dispatch_build: idx/perm/inv NULL");
+  const size_t lds = sizeof(int32_t) * (size_t)E * (1 + kDispatchWaves);
+  dispatch_build_kernel<<<1, kDispatchThreads, lds, as_stream(stream)>>>(idx, n_pairs, E, counts, offsets, perm, inv);
+  return check_launch("dispatch_build");
+}
+
+extern "C" int stmoe_combine(const void* y_sorted, const void* gate, const int32_t* inv, int dtype, int64_t T, int k,
+                             int64_t K, const void* out_norm_w, int w_dtype, float eps, const void* residual,
+                             void* out, stmoe_stream_t stream) {
+  STMOE_REQUIRE(T >= 0 && K > 0 && k >= 1, STMOE_ERR_SHAPE, "combine: T=%lld K=%lld k=%d", (long long)T, (long long)K, k);
+  if (T == 0) return STMOE_OK;
+  STMOE_REQUIRE(y_sorted && gate && inv && out, STMOE_ERR_NULL, "combine: NULL pointer");
+  STMOE_REQUIRE(T < 0x7fffffffLL, STMOE_ERR_SHAPE, "combine: T too large");
+  hipStream_t st = as_stream(stream);
+  dim3 g((unsigned)T);
+  const int wd = out_norm_w ? w_dtype : STMOE_F32;
+#define STMOE_COMBINE(TT, WW)                                                                               \
+  combine_kernel<TT, WW><<<g, 256, 0, st>>>((const TT*)y_sorted, (const TT*)gate, inv, k, K, (const WW*)out_norm_w, \
+                                            eps, (const TT*)residual, (TT*)out)
+  if (dtype == STMOE_F32 && wd == STMOE_F32) STMOE_COMBINE(float, float);
+  else if (dtype == STMOE_F16 && wd == STMOE_F32) STMOE_COMBINE(f16_t, float);
+  else if (dtype == STMOE_BF16 && wd == STMOE_F32) STMOE_COMBINE(bf16_t, float);
+  else if (dtype == STMOE_F16 && wd == STMOE_F16) STMOE_COMBINE(f16_t, f16_t);
+  else if (dtype == STMOE_BF16 && wd == STMOE_BF16) STMOE_COMBINE(bf16_t, bf16_t);
+  else return set_error(STMOE_ERR_DTYPE, "combine: dtype %d with norm weight dtype %d not implemented", dtype, w_dtype);
+#undef STMOE_COMBINE
+  return check_launch("combine");
+}

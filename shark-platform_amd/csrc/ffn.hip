@@ -1,0 +1,184 @@
+// C-ABI entry points of the grouped expert FFN, the fused layer forward and the single-matrix mmt.
+#include "ffn_kernels.h"
+
+namespace stmoe {
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64_t rows, int64_t cols) {
+  STMOE_REQUIRE(w, STMOE_ERR_NULL, "%s: weight descriptor is NULL", who);
+  STMOE_REQUIRE(w->qs, STMOE_ERR_NULL, "%s: qs plane is NULL", who);
+  STMOE_REQUIRE(w->experts == E && w->rows == rows && w->cols == cols, STMOE_ERR_SHAPE,
+                "%s: weight is [%lld,%lld,%lld], expected [%lld,%lld,%lld]", who, (long long)w->experts,
+                (long long)w->rows, (long long)w->cols, (long long)E, (long long)rows, (long long)cols);
+  STMOE_REQUIRE(aligned16(w->qs), STMOE_ERR_ALIGN, "%s: qs plane must be 16-byte aligned", who);
+  switch (w->format) {
+    case STMOE_W_Q8_0:
+      STMOE_REQUIRE(w->d, STMOE_ERR_NULL, "%s: Q8_0 needs d", who);
+      STMOE_REQUIRE(w->m == nullptr, STMOE_ERR_UNSUPPORTED, "%s: Q8 block scaled with offset is not implemented", who);
+      STMOE_REQUIRE(cols % 32 == 0, STMOE_ERR_SHAPE, "%s: Q8_0 needs cols %% 32 == 0", who);
+      break;
+    case STMOE_W_Q4_1:
+      STMOE_REQUIRE(w->d && w->m, STMOE_ERR_NULL, "%s: Q4_1 needs d and m", who);
+      STMOE_REQUIRE(cols % 32 == 0, STMOE_ERR_SHAPE, "%s: Q4_1 needs cols %% 32 == 0", who);
+      break;
+    case STMOE_W_FP8:
+      STMOE_REQUIRE(w->d, STMOE_ERR_NULL, "%s: FP8 needs d", who);
+      STMOE_REQUIRE(w->d_count == 1 || w->d_count == E, STMOE_ERR_SHAPE, "%s: FP8 d_count must be 1 or experts", who);
+      STMOE_REQUIRE(cols % 16 == 0, STMOE_ERR_SHAPE, "%s: FP8 needs cols %% 16 == 0", who);
+      break;
+    case STMOE_W_DENSE:
+      STMOE_REQUIRE(cols % 16 == 0, STMOE_ERR_SHAPE, "%s: dense weights need cols %% 16 == 0", who);
+      break;
+    default:
+      return set_error(STMOE_ERR_UNSUPPORTED, "%s: unknown weight format %d", who, w->format);
+  }
+  STMOE_REQUIRE(weight_tag(w) >= 0, STMOE_ERR_DTYPE, "%s: dtype %d not valid for format %d", who, w->dtype, w->format);
+  return STMOE_OK;
+}
+
+// variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile
+static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
+  if (variant == 0) variant = (dtype == STMOE_F32) ? 1 : 2;
+  if (variant == 2) {
+    int rc = launch_mfma_tile(dtype, wtag, mode, p, max_rows, st);
+    if (rc != STMOE_ERR_UNSUPPORTED) return rc;
+    variant = 1;  // combination without a matrix-core instantiation: the vector-ALU kernel covers it
+  }
+  if (variant == 1) return launch_generic(dtype, wtag, mode, p, max_rows, st);
+  return set_error(STMOE_ERR_UNSUPPORTED, "grouped_ffn: unknown kernel variant %d", variant);
+}
+
+}  // namespace stmoe
+
+using namespace stmoe;
+
+extern "C" size_t stmoe_grouped_ffn_workspace_bytes(int64_t T, int k, int64_t K, int64_t N, int dtype) {
+  (void)K;
+  if (T <= 0 || k <= 0 || N <= 0) return 0;
+  return align_up((size_t)T * k * N * dtype_size(dtype), 256);
+}
+
+extern "C" int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                                 const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
+                                 int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
+                                 void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
+                                 stmoe_stream_t stream) {
+  STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1, STMOE_ERR_SHAPE, "grouped_ffn: T=%lld K=%lld N=%lld E=%d k=%d",
+                (long long)T, (long long)K, (long long)N, E, k);
+  STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
+                "grouped_ffn: activation dtype %d is not f32/f16/bf16", dtype);
+  STMOE_REQUIRE(act == STMOE_ACT_SILU || act == STMOE_ACT_GELU_ERF, STMOE_ERR_UNSUPPORTED, "grouped_ffn: activation %d", act);
+  STMOE_REQUIRE(x_scale == nullptr, STMOE_ERR_UNSUPPORTED, "grouped_ffn: quantised activations are not implemented");
+  int rc;
+  if ((rc = check_weight(w_gate, "grouped_ffn(ffn_gate_exps)", E, N, K))) return rc;
+  if ((rc = check_weight(w_up, "grouped_ffn(ffn_up_exps)", E, N, K))) return rc;
+  if ((rc = check_weight(w_down, "grouped_ffn(ffn_down_exps)", E, K, N))) return rc;
+  STMOE_REQUIRE(weight_tag(w_gate) == weight_tag(w_up), STMOE_ERR_UNSUPPORTED,
+                "grouped_ffn: gate and up weights must share one format");
+  if (T == 0) return STMOE_OK;
+  STMOE_REQUIRE(x && offsets && perm && y_sorted, STMOE_ERR_NULL, "grouped_ffn: NULL pointer");
+  STMOE_REQUIRE(aligned16(x) && aligned16(y_sorted) && aligned16(workspace), STMOE_ERR_ALIGN,
+                "grouped_ffn: x, y_sorted and workspace must be 16-byte aligned");
+  STMOE_REQUIRE((K * dtype_size(dtype)) % 16 == 0 && (N * dtype_size(dtype)) % 16 == 0, STMOE_ERR_SHAPE,
+                "grouped_ffn: rows of x and of the intermediate must be multiples of 16 bytes");
+  const size_t need = stmoe_grouped_ffn_workspace_bytes(T, k, K, N, dtype);
+  STMOE_REQUIRE(workspace && workspace_bytes >= need, STMOE_ERR_WORKSPACE, "grouped_ffn: workspace %zu < %zu bytes",
+                workspace_bytes, need);
+  hipStream_t st = as_stream(stream);
+  const int64_t rows = T * k;
+
+  GemmParams p{};
+  p.a = x; p.lda = K; p.perm = perm; p.k_top = k; p.offsets = offsets; p.E = E; p.fixed_rows = 0;
+  p.w0 = make_view(w_gate); p.w1 = make_view(w_up);
+  p.out = workspace; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr;
+  if ((rc = run_projection(variant, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st))) return rc;
+
+  GemmParams q{};
+  q.a = workspace; q.lda = N; q.perm = nullptr; q.k_top = 1; q.offsets = offsets; q.E = E; q.fixed_rows = 0;
+  q.w0 = make_view(w_down); q.w1 = q.w0;
+  q.out = y_sorted; q.ldo = K; q.n_out = K; q.kred = N; q.act = act; q.x_scale = nullptr;
+  return run_projection(variant, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
+}
+
+extern "C" int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight* w, void* out, int variant,
+                         stmoe_stream_t stream) {
+  STMOE_REQUIRE(w, STMOE_ERR_NULL, "mmt: weight descriptor is NULL");
+  STMOE_REQUIRE(M >= 0, STMOE_ERR_SHAPE, "mmt: M=%lld", (long long)M);
+  STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
+                "mmt: activation dtype %d is not f32/f16/bf16", dtype);
+  int rc;
+  if ((rc = check_weight(w, "mmt", 1, w->rows, w->cols))) return rc;
+  if (M == 0) return STMOE_OK;
+  STMOE_REQUIRE(a && out, STMOE_ERR_NULL, "mmt: NULL pointer");
+  STMOE_REQUIRE(aligned16(a) && aligned16(out), STMOE_ERR_ALIGN, "mmt: a and out must be 16-byte aligned");
+  STMOE_REQUIRE((w->cols * dtype_size(dtype)) % 16 == 0 && (w->rows * dtype_size(dtype)) % 8 == 0, STMOE_ERR_SHAPE,
+                "mmt: row sizes must keep 16-byte (input) and 8-byte (output) alignment");
+  GemmParams p{};
+  p.a = a; p.lda = w->cols; p.perm = nullptr; p.k_top = 1; p.offsets = nullptr; p.E = 1; p.fixed_rows = M;
+  p.w0 = make_view(w); p.w1 = p.w0;
+  p.out = out; p.ldo = w->rows; p.n_out = w->rows; p.kred = w->cols; p.act = 0; p.x_scale = nullptr;
+  return run_projection(variant, dtype, weight_tag(w), MODE_DOWN, p, M, as_stream(stream));
+}
+
+// ---- whole layer ----------------------------------------------------------------------------------
+// Workspace carve-up (each piece 256-byte aligned):
+//   xn [T,K] T | logits-free | idx i32 [T,k] | gate T [T,k] | counts i32 [E] | offsets i32 [E+1] |
+//   perm i32 [T*k] | inv i32 [T*k] | y [T*k, K] T | ffn workspace
+struct LayerWs {
+  size_t xn, idx, gate, counts, offsets, perm, inv, y, ffn, total;
+};
+static LayerWs carve(int64_t T, int k, int E, int64_t K, int64_t N, int dtype) {
+  LayerWs w{};
+  const size_t es = dtype_size(dtype);
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes ? bytes : 1, 256); return o; };
+  w.xn = take((size_t)T * K * es);
+  w.idx = take((size_t)T * k * 4);
+  w.gate = take((size_t)T * k * es);
+  w.counts = take((size_t)E * 4);
+  w.offsets = take((size_t)(E + 1) * 4);
+  w.perm = take((size_t)T * k * 4);
+  w.inv = take((size_t)T * k * 4);
+  w.y = take((size_t)T * k * K * es);
+  w.ffn = take(stmoe_grouped_ffn_workspace_bytes(T, k, K, N, dtype));
+  w.total = off;
+  return w;
+}
+
+extern "C" size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int64_t K, int64_t N, int dtype) {
+  if (T <= 0 || k <= 0 || E <= 0 || K <= 0 || N <= 0) return 0;
+  return carve(T, k, E, K, N, dtype).total;
+}
+
+extern "C" int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                                 const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
+                                 const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
+                                 const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
+                                 void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream) {
+  STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1 && k <= E, STMOE_ERR_SHAPE,
+                "moe_forward: T=%lld K=%lld N=%lld E=%d k=%d", (long long)T, (long long)K, (long long)N, E, k);
+  if (T == 0) return STMOE_OK;
+  STMOE_REQUIRE(h && ffn_norm_w && w_router && out, STMOE_ERR_NULL, "moe_forward: NULL pointer");
+  const LayerWs ws = carve(T, k, E, K, N, dtype);
+  STMOE_REQUIRE(workspace && workspace_bytes >= ws.total, STMOE_ERR_WORKSPACE, "moe_forward: workspace %zu < %zu bytes",
+                workspace_bytes, ws.total);
+  STMOE_REQUIRE(aligned16(workspace), STMOE_ERR_ALIGN, "moe_forward: workspace must be 16-byte aligned");
+  char* base = (char*)workspace;
+  void* xn = base + ws.xn;
+  int32_t* idx = idx_out ? idx_out : (int32_t*)(base + ws.idx);
+  void* gate = gate_out ? gate_out : (void*)(base + ws.gate);
+  int32_t* counts = (int32_t*)(base + ws.counts);
+  int32_t* offsets = (int32_t*)(base + ws.offsets);
+  int32_t* perm = (int32_t*)(base + ws.perm);
+  int32_t* inv = (int32_t*)(base + ws.inv);
+  void* y = base + ws.y;
+  int rc;
+  if ((rc = stmoe_rms_norm(h, dtype, ffn_norm_w, w_dtype, T, K, eps, xn, stream))) return rc;
+  if ((rc = stmoe_router_topk(xn, w_router, dtype, T, K, E, k, nullptr, idx, nullptr, gate, stream))) return rc;
+  if ((rc = stmoe_dispatch_build(idx, T * k, E, counts, offsets, perm, inv, stream))) return rc;
+  if ((rc = stmoe_grouped_ffn(xn, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, nullptr, y,
+                              base + ws.ffn, workspace_bytes - ws.ffn, variant, stream)))
+    return rc;
+  return stmoe_combine(y, gate, inv, dtype, T, k, K, out_norm_w, w_dtype, eps, h, out, stream);
+}

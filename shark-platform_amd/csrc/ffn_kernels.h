@@ -1,0 +1,73 @@
+// Grouped expert projections over rows sorted by expert.
+//
+// Two projection shapes cover PreGatherFFNMOE.forward (sharktank/sharktank/layers/ffn_moe_block.py:60-72):
+//   GATEUP: z[i, n] = T( T(act(T(x[t] . Wg[e][n]))) * T(x[t] . Wu[e][n]) )   ("mk,menk->men" twice + act + mul)
+//   DOWN:   y[i, c] = T( z[i] . Wd[e][c] )                                    ("mek,menk->men")
+// where i is a sorted position, t = perm[i] / k its token and e its expert; dot products accumulate in
+// fp32 and T(.) is a rounding to the activation dtype where the reference materialises a tensor.
+#pragma once
+#include "weights.h"
+
+namespace stmoe {
+
+enum : int { MODE_GATEUP = 0, MODE_DOWN = 1 };
+
+struct GemmParams {
+  const void* a;          // activations: x [T, lda] (GATEUP) or z [rows, lda] (DOWN)
+  int64_t lda;
+  const int32_t* perm;    // sorted position -> pair id; source row = perm[i] / k_top.  NULL: source row = i
+  int32_t k_top;
+  const int32_t* offsets; // [E+1] row ranges per expert; NULL: one expert with `fixed_rows` rows
+  int32_t E;
+  int64_t fixed_rows;
+  WeightView w0, w1;      // GATEUP: gate, up.  DOWN: w0 only
+  void* out;
+  int64_t ldo;
+  int64_t n_out;          // rows of the weight matrices
+  int64_t kred;           // reduction length
+  int32_t act;
+  const float* x_scale;   // optional scale applied to the fp32 dot products (fp8 activations)
+};
+
+// (expert, first row, end row) of m-tile `slot` when every expert's rows are cut into tiles of BM.
+__device__ __forceinline__ bool find_tile(const GemmParams& p, int slot, int BM, int& e, int& row_begin, int& row_end) {
+  if (!p.offsets) {
+    e = 0;
+    row_begin = slot * BM;
+    row_end = (int)(p.fixed_rows < (int64_t)row_begin + BM ? p.fixed_rows : (int64_t)row_begin + BM);
+    return row_begin < p.fixed_rows;
+  }
+  int acc = 0;
+  for (e = 0; e < p.E; ++e) {
+    const int b = p.offsets[e], en = p.offsets[e + 1];
+    const int tiles = (en - b + BM - 1) / BM;
+    if (slot < acc + tiles) {
+      row_begin = b + (slot - acc) * BM;
+      row_end = en < row_begin + BM ? en : row_begin + BM;
+      return true;
+    }
+    acc += tiles;
+  }
+  return false;
+}
+
+__device__ __forceinline__ float act_rt(int act, float v) {
+  return act == STMOE_ACT_SILU ? act_silu(v) : act_gelu_erf(v);
+}
+
+template <typename T> __device__ __forceinline__ float gateup_epilogue(int act, float g, float u, float scale) {
+  const float gr = round_to<T>(g * scale);
+  const float a = round_to<T>(act_rt(act, gr));
+  const float ur = round_to<T>(u * scale);
+  return round_to<T>(__fmul_rn(a, ur));
+}
+
+}  // namespace stmoe
+
+namespace stmoe {
+// Launchers (one per kernel family).  `act_dtype` is the activation dtype enum, `wtag` a WF_* tag,
+// `max_rows` an upper bound of the sorted row count known on the host (T*k).  Each returns
+// STMOE_ERR_UNSUPPORTED when the family has no instantiation for the combination.
+int launch_generic(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
+int launch_mfma_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
+}  // namespace stmoe

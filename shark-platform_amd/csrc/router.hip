@@ -1,0 +1,218 @@
+// RMS norm and the router (logits, softmax, top-k, gate renormalisation) of MoeBlock.forward
+// (sharktank/sharktank/layers/mixture_of_experts_block.py:68-83, norm.py:34-41,
+//  sharktank/sharktank/ops/default_impls.py:328-359,402-408).
+#include "stmoe_common.h"
+
+namespace stmoe {
+
+// ---------------------------------------------------------------------------------------------------
+// rms_norm: one workgroup per row.  x32 = float(x); o = x32 * rsqrt(mean(x32^2) + eps);
+// o = w * W(o) in W = dtype of w; result rounded to T.
+template <typename T, typename W>
+__global__ void __launch_bounds__(256)
+rms_norm_kernel(const T* __restrict__ x, const W* __restrict__ w, int64_t K, float eps, T* __restrict__ out) {
+  __shared__ float partial[4];
+  const T* row = x + (int64_t)blockIdx.x * K;
+  T* orow = out + (int64_t)blockIdx.x * K;
+  float ss = 0.0f;
+  for (int64_t i = threadIdx.x; i < K; i += 256) {
+    const float v = Cvt<T>::to_f32(row[i]);
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_xor_sum(ss);
+  if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float total = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+  const float rs = 1.0f / sqrtf(total / (float)K + eps);
+  for (int64_t i = threadIdx.x; i < K; i += 256) {
+    float o = round_to<W>(Cvt<T>::to_f32(row[i]) * rs);
+    o = round_to<W>(Cvt<W>::to_f32(w[i]) * o);
+    orow[i] = Cvt<T>::from_f32(o);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// router: one wavefront per token.
+//
+// Summation order of a logit (part of the contract, restated by the parity oracle): with c = chunk,
+// l = lane, lane l owns the 8 consecutive elements k = (c*64 + l)*8 + j, j = 0..7, of every chunk
+// c = 0..ceil(K/512)-1 that lies inside K; it adds their products x[k]*w[e][k] to an fp32 accumulator
+// in increasing (c, j) order (multiply and add rounded separately, no FMA contraction), and the 64
+// lane sums are then combined by the xor butterfly 32,16,8,4,2,1.  The logit is that fp32 sum rounded
+// to the activation dtype, as `torch.matmul` on T tensors returns T.
+template <typename T> struct Vec8;
+template <> struct Vec8<float> {
+  float v[8];
+  __device__ __forceinline__ void load(const float* p) {
+    const float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+};
+template <> struct Vec8<f16_t> {
+  float v[8];
+  __device__ __forceinline__ void load(const f16_t* p) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+    const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      union { uint16_t u; f16_t h; } lo, hi;
+      lo.u = (uint16_t)(r[i] & 0xffffu);
+      hi.u = (uint16_t)(r[i] >> 16);
+      v[2 * i] = (float)lo.h;
+      v[2 * i + 1] = (float)hi.h;
+    }
+  }
+};
+template <> struct Vec8<bf16_t> {
+  float v[8];
+  __device__ __forceinline__ void load(const bf16_t* p) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+    const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(r[i] << 16);
+      v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+    }
+  }
+};
+
+template <typename T, int EP>
+__global__ void __launch_bounds__(256)
+router_topk_kernel(const T* __restrict__ x, const T* __restrict__ wr, int64_t T_tokens, int64_t K, int E, int k,
+                   T* __restrict__ logits_out, int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out,
+                   T* __restrict__ gate_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T_tokens) return;
+  const T* xr = x + t * K;
+
+  float acc[EP];
+#pragma unroll
+  for (int e = 0; e < EP; ++e) acc[e] = 0.0f;
+
+  for (int64_t k0 = (int64_t)lane * 8; k0 < K; k0 += 512) {
+    Vec8<T> xv;
+    xv.load(xr + k0);
+#pragma unroll
+    for (int e = 0; e < EP; ++e) {
+      if (e < E) {
+        Vec8<T> wv;
+        wv.load(wr + (int64_t)e * K + k0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[e] = __fadd_rn(acc[e], __fmul_rn(xv.v[j], wv.v[j]));
+      }
+    }
+  }
+
+  float lg[EP];
+#pragma unroll
+  for (int e = 0; e < EP; ++e) lg[e] = (e < E) ? round_to<T>(wave_xor_sum(acc[e])) : -INFINITY;
+
+  if (logits_out) {
+#pragma unroll
+    for (int e = 0; e < EP; ++e)
+      if (e < E && lane == (e & 63)) logits_out[t * E + e] = Cvt<T>::from_f32(lg[e]);
+  }
+
+  // fp32 softmax over the E logits (F.softmax(dim=1, dtype=float)).
+  float mx = lg[0];
+#pragma unroll
+  for (int e = 1; e < EP; ++e) mx = fmaxf(mx, lg[e]);
+  float denom = 0.0f;
+#pragma unroll
+  for (int e = 0; e < EP; ++e)
+    if (e < E) denom += expf(lg[e] - mx);
+
+  // top-k by (logit descending, expert index ascending).  exp is monotone, so this is the order of the
+  // probabilities with ties resolved toward the lower index.
+  uint64_t taken = 0;
+  float vsum = 0.0f;
+  float pv[EP];  // selected probabilities in slot order (only the first k are used)
+  int pi[EP];
+#pragma unroll
+  for (int j = 0; j < EP; ++j) {
+    if (j < k) {
+      int best = -1;
+      float bestv = 0.0f;
+#pragma unroll
+      for (int e = 0; e < EP; ++e) {
+        if (e < E && !((taken >> e) & 1ull) && (best < 0 || lg[e] > bestv)) {
+          best = e;
+          bestv = lg[e];
+        }
+      }
+      taken |= 1ull << best;
+      const float p = expf(bestv - mx) / denom;
+      pv[j] = p;
+      pi[j] = best;
+      vsum += p;
+    }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int j = 0; j < EP; ++j) {
+      if (j < k) {
+        idx_out[t * k + j] = pi[j];
+        if (idx64_out) idx64_out[t * k + j] = pi[j];
+        gate_out[t * k + j] = Cvt<T>::from_f32(pv[j] / vsum);
+      }
+    }
+  }
+}
+
+template <typename T>
+static int launch_router(const void* x, const void* wr, int64_t T_tokens, int64_t K, int E, int k, void* logits,
+                         int32_t* idx, int64_t* idx64, void* gate, hipStream_t st) {
+  dim3 grid((unsigned)((T_tokens + 3) / 4));
+#define STMOE_ROUTER_CASE(EP)                                                                               \
+  router_topk_kernel<T, EP><<<grid, 256, 0, st>>>((const T*)x, (const T*)wr, T_tokens, K, E, k, (T*)logits, \
+                                                  idx, idx64, (T*)gate)
+  if (E <= 8) STMOE_ROUTER_CASE(8);
+  else if (E <= 16) STMOE_ROUTER_CASE(16);
+  else if (E <= 32) STMOE_ROUTER_CASE(32);
+  else STMOE_ROUTER_CASE(64);
+#undef STMOE_ROUTER_CASE
+  return check_launch("router_topk");
+}
+
+}  // namespace stmoe
+
+using namespace stmoe;
+
+extern "C" int stmoe_rms_norm(const void* x, int dtype, const void* w, int w_dtype, int64_t T, int64_t K, float eps,
+                              void* out, stmoe_stream_t stream) {
+  STMOE_REQUIRE(T >= 0 && K > 0, STMOE_ERR_SHAPE, "rms_norm: T=%lld K=%lld", (long long)T, (long long)K);
+  if (T == 0) return STMOE_OK;
+  STMOE_REQUIRE(x && w && out, STMOE_ERR_NULL, "rms_norm: NULL pointer");
+  STMOE_REQUIRE(T < 0x7fffffffLL, STMOE_ERR_SHAPE, "rms_norm: T too large");
+  hipStream_t st = as_stream(stream);
+  dim3 g((unsigned)T);
+#define STMOE_RMS(TT, WW) rms_norm_kernel<TT, WW><<<g, 256, 0, st>>>((const TT*)x, (const WW*)w, K, eps, (TT*)out)
+  if (dtype == STMOE_F32 && w_dtype == STMOE_F32) STMOE_RMS(float, float);
+  else if (dtype == STMOE_F16 && w_dtype == STMOE_F32) STMOE_RMS(f16_t, float);
+  else if (dtype == STMOE_BF16 && w_dtype == STMOE_F32) STMOE_RMS(bf16_t, float);
+  else if (dtype == STMOE_F16 && w_dtype == STMOE_F16) STMOE_RMS(f16_t, f16_t);
+  else if (dtype == STMOE_BF16 && w_dtype == STMOE_BF16) STMOE_RMS(bf16_t, bf16_t);
+  else return set_error(STMOE_ERR_DTYPE, "rms_norm: dtype %d with weight dtype %d not implemented", dtype, w_dtype);
+#undef STMOE_RMS
+  return check_launch("rms_norm");
+}
+
+extern "C" int stmoe_router_topk(const void* x, const void* w_router, int dtype, int64_t T, int64_t K, int E, int k,
+                                 void* logits_out, int32_t* idx_out, int64_t* idx64_out, void* gate_out,
+                                 stmoe_stream_t stream) {
+  STMOE_REQUIRE(T >= 0 && K > 0 && K % 8 == 0, STMOE_ERR_SHAPE, "router_topk: T=%lld, K=%lld (K must be a positive multiple of 8)",
+                (long long)T, (long long)K);
+  STMOE_REQUIRE(E >= 1 && E <= 64, STMOE_ERR_SHAPE, "router_topk: expert count %d outside 1..64", E);
+  STMOE_REQUIRE(k >= 1 && k <= E, STMOE_ERR_SHAPE, "router_topk: top-k %d outside 1..%d", k, E);
+  if (T == 0) return STMOE_OK;
+  STMOE_REQUIRE(x && w_router && idx_out && gate_out, STMOE_ERR_NULL, "router_topk: NULL pointer");
+  STMOE_REQUIRE(aligned16(x) && aligned16(w_router), STMOE_ERR_ALIGN, "router_topk: x and w_router must be 16-byte aligned");
+  hipStream_t st = as_stream(stream);
+  switch (dtype) {
+    case STMOE_F32: return launch_router<float>(x, w_router, T, K, E, k, logits_out, idx_out, idx64_out, gate_out, st);
+    case STMOE_F16: return launch_router<f16_t>(x, w_router, T, K, E, k, logits_out, idx_out, idx64_out, gate_out, st);
+    case STMOE_BF16: return launch_router<bf16_t>(x, w_router, T, K, E, k, logits_out, idx_out, idx64_out, gate_out, st);
+    default: return set_error(STMOE_ERR_DTYPE, "router_topk: dtype %d is not f32/f16/bf16", dtype);
+  }
+}

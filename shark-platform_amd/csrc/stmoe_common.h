@@ -1,0 +1,126 @@
+// Shared device/host helpers for the gfx950 MoE kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/sharktank_moe_hip.h"
+
+namespace stmoe {
+
+// ---- status plumbing --------------------------------------------------------------------------
+int set_error(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+#define STMOE_REQUIRE(cond, code, ...)            \
+  do {                                            \
+    if (!(cond)) return ::stmoe::set_error((code), __VA_ARGS__); \
+  } while (0)
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline hipStream_t as_stream(stmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+static inline int dtype_size(int dt) {
+  switch (dt) {
+    case STMOE_F32: return 4;
+    case STMOE_F16: case STMOE_BF16: return 2;
+    case STMOE_F8E4M3FN: case STMOE_I8: case STMOE_U8: return 1;
+    default: return 0;
+  }
+}
+
+// ---- 16-bit float types as raw bits -------------------------------------------------------------
+// bf16 is handled as a 16-bit pattern with explicit round-to-nearest-even conversions so that every
+// rounding point is spelled out; fp16 uses the native _Float16 type.
+typedef _Float16 f16_t;
+struct bf16_t { uint16_t bits; };
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  bf16_t r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {  // NaN: keep it quiet
+    r.bits = (uint16_t)((u >> 16) | 0x40u);
+    return r;
+  }
+  u += 0x7fffu + ((u >> 16) & 1u);
+  r.bits = (uint16_t)(u >> 16);
+  return r;
+}
+
+template <typename T> struct Cvt;
+template <> struct Cvt<float> {
+  static __device__ __forceinline__ float to_f32(float v) { return v; }
+  static __device__ __forceinline__ float from_f32(float v) { return v; }
+};
+template <> struct Cvt<f16_t> {
+  static __device__ __forceinline__ float to_f32(f16_t v) { return (float)v; }
+  static __device__ __forceinline__ f16_t from_f32(float v) { return (f16_t)v; }
+};
+template <> struct Cvt<bf16_t> {
+  static __device__ __forceinline__ float to_f32(bf16_t v) { return bf16_to_f32(v); }
+  static __device__ __forceinline__ bf16_t from_f32(float v) { return f32_to_bf16(v); }
+};
+
+// Round an fp32 value to T and widen it again: the value a tensor of dtype T would hold.
+template <typename T> __device__ __forceinline__ float round_to(float v) {
+  return Cvt<T>::to_f32(Cvt<T>::from_f32(v));
+}
+
+// ---- fp8 e4m3fn (OCP) ---------------------------------------------------------------------------
+__device__ __forceinline__ float fp8_e4m3fn_to_f32(uint8_t b) {
+  const uint32_t sign = (uint32_t)(b & 0x80u) << 24;
+  const uint32_t e = (b >> 3) & 0xfu;
+  const uint32_t mnt = b & 0x7u;
+  if (e == 0) {  // subnormal: mnt * 2^-9
+    float v = (float)mnt * 0.001953125f;
+    return __uint_as_float(__float_as_uint(v) | sign);
+  }
+  if (e == 0xf && mnt == 0x7) return __uint_as_float(0x7fc00000u | sign);  // NaN (no inf in e4m3fn)
+  return __uint_as_float(sign | ((e + 120u) << 23) | (mnt << 20));
+}
+
+// Round-to-nearest-even fp32 -> e4m3fn; magnitudes above 448 that round past it become NaN (0x7f),
+// as torch's cast does; callers that want saturation clamp first.
+__device__ __forceinline__ uint8_t f32_to_fp8_e4m3fn(float f) {
+  uint32_t u = __float_as_uint(f);
+  const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+  u &= 0x7fffffffu;
+  if (u > 0x7f800000u) return sign | 0x7f;       // NaN
+  if (u >= 0x43f00000u) return sign | 0x7f;      // >= 480 rounds beyond 448 -> NaN; (464 handled below)
+  if (u < 0x3c800000u) {                         // < 2^-6: subnormal result, step 2^-9
+    float a = __uint_as_float(u);
+    // a * 512 rounded to nearest even integer in [0, 8]
+    float r = rintf(a * 512.0f);
+    return sign | (uint8_t)r;                    // r == 8 gives 0x08 = 2^-6, the smallest normal: correct
+  }
+  // normal: keep 3 mantissa bits
+  uint32_t rounded = u + 0x7ffffu + ((u >> 20) & 1u);
+  uint32_t e = (rounded >> 23) - 120u;
+  uint32_t mnt = (rounded >> 20) & 0x7u;
+  uint32_t enc = (e << 3) | mnt;
+  if (enc > 0x7eu) return sign | 0x7f;           // rounded above 448
+  return sign | (uint8_t)enc;
+}
+
+// ---- activations ---------------------------------------------------------------------------------
+__device__ __forceinline__ float act_silu(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float act_gelu_erf(float v) { return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f)); }
+template <int ACT> __device__ __forceinline__ float apply_act(float v) {
+  return ACT == STMOE_ACT_SILU ? act_silu(v) : act_gelu_erf(v);
+}
+
+// ---- wavefront helpers -----------------------------------------------------------------------------
+static constexpr int kWave = 64;
+
+__device__ __forceinline__ float wave_xor_sum(float v) {
+  // Fixed butterfly: partner distance 32, 16, 8, 4, 2, 1.  Each step adds a value and its partner's,
+  // which is commutative, so every lane ends with the same bits.
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, kWave);
+  return v;
+}
+
+}  // namespace stmoe

@@ -1,0 +1,260 @@
+// Weight-format accessors: turn 16 consecutive reduction elements of one weight row into values of the
+// activation type T, with the roundings of the reference's dequantize-then-cast
+// (`unbox_tensor` -> layout.dequant() -> `.to(lhs.dtype)`, sharktank/sharktank/ops/default_impls.py:345-351):
+//   Q8_0   w = T( f16(d * q) )                  sharktank/sharktank/types/layouts.py:274-290
+//   Q4_1   w = T( f16( f16(d * q) + m ) )       layouts.py:302-357, layout_utils.py:67-86
+//   FP8    w = T( DD( DD(q) * d ) ), DD = dtype of d   layouts.py:163-181
+//   DENSE  w = T( element )
+#pragma once
+#include "stmoe_common.h"
+
+namespace stmoe {
+
+struct WeightView {
+  const uint8_t* qs;
+  const uint8_t* d;
+  const uint8_t* m;
+  int64_t rows;     // per expert
+  int64_t cols;     // reduction length
+  int64_t d_count;  // FP8: number of scales (1 or experts)
+  int32_t dtype;    // DENSE element dtype / FP8 scale dtype
+  int32_t experts;
+};
+
+static inline WeightView make_view(const stmoe_weight* w) {
+  WeightView v;
+  v.qs = (const uint8_t*)w->qs;
+  v.d = (const uint8_t*)w->d;
+  v.m = (const uint8_t*)w->m;
+  v.rows = w->rows;
+  v.cols = w->cols;
+  v.d_count = w->d_count;
+  v.dtype = w->dtype;
+  v.experts = (int32_t)w->experts;
+  return v;
+}
+
+// Formats as compile-time tags.  Dense weights are split by element type.
+enum : int { WF_Q8_0 = 0, WF_Q4_1 = 1, WF_FP8_F32D = 2, WF_FP8_F16D = 3, WF_DENSE_F32 = 4, WF_DENSE_F16 = 5, WF_DENSE_BF16 = 6 };
+
+// pack two fp32 values, already rounded to T, into one dword of T bits
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi) {
+  union { f16_t h[2]; uint32_t u; } c;
+  c.h[0] = (f16_t)lo;
+  c.h[1] = (f16_t)hi;
+  return c.u;
+}
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo).bits | ((uint32_t)f32_to_bf16(hi).bits << 16);
+}
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ half2_t as_half2(uint32_t u) {
+  union { uint32_t u; half2_t h; } c;
+  c.u = u;
+  return c.h;
+}
+__device__ __forceinline__ uint32_t as_u32(half2_t h) {
+  union { uint32_t u; half2_t h; } c;
+  c.h = h;
+  return c.u;
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
+  union { uint16_t u; f16_t h; } c;
+  c.u = (uint16_t)b;
+  return (float)c.h;
+}
+
+// Raw bytes of a 16-element chunk and its conversion.  `load` only issues the global loads (so a caller
+// can keep a chunk in flight across a compute phase); `to_f32` produces the 16 values as fp32 numbers
+// equal to the dequantised weight in the layout dtype (the caller rounds to T).
+template <int WF> struct Chunk16;
+
+template <> struct Chunk16<WF_Q8_0> {
+  uint4 q;
+  uint16_t dbits;
+  __device__ __forceinline__ void load(const WeightView& w, int64_t e, int64_t n, int64_t k0) {
+    const int64_t row = e * w.rows + n;
+    q = *reinterpret_cast<const uint4*>(w.qs + row * w.cols + k0);
+    dbits = reinterpret_cast<const uint16_t*>(w.d)[row * (w.cols >> 5) + (k0 >> 5)];
+  }
+  __device__ __forceinline__ void zero() { q = make_uint4(0, 0, 0, 0); dbits = 0; }
+  // 16 fp16 values as 8 dwords: (q + 1152) built by byte permutation as 0x6400|u8, minus 1152, times d.
+  // Products of an fp16 scale and an integer of magnitude <= 128 are exact in the multiplier, so the
+  // single rounding of the fp16 multiply equals the reference's f16(d * q).
+  __device__ __forceinline__ void to_f16x16(uint32_t out[8]) const {
+    const uint32_t r[4] = {q.x, q.y, q.z, q.w};
+    const half2_t bias = {(f16_t)1152.0f, (f16_t)1152.0f};
+    union { uint16_t u; f16_t h; } dc;
+    dc.u = dbits;
+    const half2_t dd = {dc.h, dc.h};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t u = r[i] ^ 0x80808080u;
+      const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
+      const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+      out[2 * i] = as_u32((as_half2(lo) - bias) * dd);
+      out[2 * i + 1] = as_u32((as_half2(hi) - bias) * dd);
+    }
+  }
+  __device__ __forceinline__ void to_f32(float out[16]) const {
+    uint32_t h[8];
+    to_f16x16(h);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      out[2 * i] = f16_bits_to_f32(h[i] & 0xffffu);
+      out[2 * i + 1] = f16_bits_to_f32(h[i] >> 16);
+    }
+  }
+};
+
+template <> struct Chunk16<WF_Q4_1> {
+  uint2 q;
+  uint16_t dbits, mbits;
+  __device__ __forceinline__ void load(const WeightView& w, int64_t e, int64_t n, int64_t k0) {
+    const int64_t row = e * w.rows + n;
+    q = *reinterpret_cast<const uint2*>(w.qs + ((row * w.cols + k0) >> 1));
+    const int64_t b = row * (w.cols >> 5) + (k0 >> 5);
+    dbits = reinterpret_cast<const uint16_t*>(w.d)[b];
+    mbits = reinterpret_cast<const uint16_t*>(w.m)[b];
+  }
+  __device__ __forceinline__ void zero() { q = make_uint2(0, 0); dbits = 0; mbits = 0; }
+  // element 2i = low nibble of byte i, element 2i+1 = high nibble.  f16(f16(d*q) + m): two roundings.
+  __device__ __forceinline__ void to_f16x16(uint32_t out[8]) const {
+    const uint32_t r[2] = {q.x, q.y};
+    union { uint16_t u; f16_t h; } dc, mc;
+    dc.u = dbits;
+    mc.u = mbits;
+    const half2_t dd = {dc.h, dc.h}, mm = {mc.h, mc.h};
+    const half2_t bias = {(f16_t)1024.0f, (f16_t)1024.0f};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const uint32_t byte = (r[i] >> (8 * b)) & 0xffu;
+        const uint32_t pair = 0x64006400u | (byte & 0xfu) | ((byte >> 4) << 16);
+        half2_t v = (as_half2(pair) - bias) * dd;
+        v = v + mm;
+        out[4 * i + b] = as_u32(v);
+      }
+    }
+  }
+  __device__ __forceinline__ void to_f32(float out[16]) const {
+    uint32_t h[8];
+    to_f16x16(h);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      out[2 * i] = f16_bits_to_f32(h[i] & 0xffffu);
+      out[2 * i + 1] = f16_bits_to_f32(h[i] >> 16);
+    }
+  }
+};
+
+template <bool F16D> struct Chunk16Fp8 {
+  uint4 q;
+  float dv;
+  __device__ __forceinline__ void load(const WeightView& w, int64_t e, int64_t n, int64_t k0) {
+    const int64_t row = e * w.rows + n;
+    q = *reinterpret_cast<const uint4*>(w.qs + row * w.cols + k0);
+    const int64_t j = w.d_count > 1 ? e : 0;
+    dv = F16D ? (float)reinterpret_cast<const f16_t*>(w.d)[j] : reinterpret_cast<const float*>(w.d)[j];
+  }
+  __device__ __forceinline__ void zero() { q = make_uint4(0, 0, 0, 0); dv = 0.0f; }
+  __device__ __forceinline__ void to_f32(float out[16]) const {
+    const uint32_t r[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float v = fp8_e4m3fn_to_f32((uint8_t)(r[i >> 2] >> (8 * (i & 3))));
+      const float p = __fmul_rn(v, dv);
+      out[i] = F16D ? round_to<f16_t>(p) : p;
+    }
+  }
+};
+template <> struct Chunk16<WF_FP8_F32D> : Chunk16Fp8<false> {};
+template <> struct Chunk16<WF_FP8_F16D> : Chunk16Fp8<true> {};
+
+template <> struct Chunk16<WF_DENSE_F32> {
+  float4 v[4];
+  __device__ __forceinline__ void load(const WeightView& w, int64_t e, int64_t n, int64_t k0) {
+    const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(w.qs) + (e * w.rows + n) * w.cols + k0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = p[i];
+  }
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = make_float4(0, 0, 0, 0);
+  }
+  __device__ __forceinline__ void to_f32(float out[16]) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      out[4 * i] = v[i].x; out[4 * i + 1] = v[i].y; out[4 * i + 2] = v[i].z; out[4 * i + 3] = v[i].w;
+    }
+  }
+};
+
+template <bool BF> struct Chunk16Dense16 {
+  uint32_t r[8];
+  __device__ __forceinline__ void load(const WeightView& w, int64_t e, int64_t n, int64_t k0) {
+    const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(w.qs) + (e * w.rows + n) * w.cols + k0);
+    const uint4 a = p[0], b = p[1];
+    r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w;
+    r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+  }
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = 0;
+  }
+  __device__ __forceinline__ void to_f32(float out[16]) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (BF) {
+        out[2 * i] = __uint_as_float(r[i] << 16);
+        out[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+      } else {
+        out[2 * i] = f16_bits_to_f32(r[i] & 0xffffu);
+        out[2 * i + 1] = f16_bits_to_f32(r[i] >> 16);
+      }
+    }
+  }
+  __device__ __forceinline__ void raw(uint32_t out[8]) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = r[i];
+  }
+};
+template <> struct Chunk16<WF_DENSE_F16> : Chunk16Dense16<false> {};
+template <> struct Chunk16<WF_DENSE_BF16> : Chunk16Dense16<true> {};
+
+// 16 values of T as 8 dwords, ready for LDS / MFMA operands.
+template <typename T, int WF>
+__device__ __forceinline__ void chunk_to_T(const Chunk16<WF>& c, uint32_t out[8]) {
+  if constexpr (WF == WF_Q8_0 || WF == WF_Q4_1) {
+    if constexpr (__is_same(T, f16_t)) {
+      c.to_f16x16(out);
+      return;
+    }
+  }
+  if constexpr ((WF == WF_DENSE_F16 && __is_same(T, f16_t)) || (WF == WF_DENSE_BF16 && __is_same(T, bf16_t))) {
+    c.raw(out);
+    return;
+  }
+  float f[16];
+  c.to_f32(f);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) out[i] = pack2<T>(f[2 * i], f[2 * i + 1]);
+}
+
+// Host-side: compile-time tag of a weight descriptor, or -1.
+static inline int weight_tag(const stmoe_weight* w) {
+  switch (w->format) {
+    case STMOE_W_Q8_0: return WF_Q8_0;
+    case STMOE_W_Q4_1: return WF_Q4_1;
+    case STMOE_W_FP8: return w->dtype == STMOE_F32 ? WF_FP8_F32D : (w->dtype == STMOE_F16 ? WF_FP8_F16D : -1);
+    case STMOE_W_DENSE:
+      return w->dtype == STMOE_F32 ? WF_DENSE_F32 : (w->dtype == STMOE_F16 ? WF_DENSE_F16 : (w->dtype == STMOE_BF16 ? WF_DENSE_BF16 : -1));
+    default: return -1;
+  }
+}
+
+}  // namespace stmoe

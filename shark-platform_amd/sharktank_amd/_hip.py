@@ -1,0 +1,389 @@
+"""ctypes binding of libsharktank_moe_hip.so (the C ABI in include/sharktank_moe_hip.h).
+
+torch is used for device memory and the current HIP stream only.  Every wrapper refuses host tensors and
+raises if the shared library is missing: there is no CPU or eager-torch arithmetic path in this package.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
+from typing import Optional
+
+import torch
+
+_LIB_NAME = "libsharktank_moe_hip.so"
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+
+# enum stmoe_dtype
+F32, F16, BF16, F8E4M3FN, I8, U8 = 0, 1, 2, 3, 4, 5
+# enum stmoe_act
+ACT_SILU, ACT_GELU_ERF = 0, 1
+# enum stmoe_wfmt
+W_DENSE, W_Q8_0, W_Q4_1, W_FP8 = 0, 1, 2, 3
+# grouped_ffn variants
+VARIANT_AUTO, VARIANT_GENERIC, VARIANT_MFMA_TILE = 0, 1, 2
+
+_DTYPE_ENUM = {
+    torch.float32: F32,
+    torch.float16: F16,
+    torch.bfloat16: BF16,
+    torch.float8_e4m3fn: F8E4M3FN,
+    torch.int8: I8,
+    torch.uint8: U8,
+}
+
+STATUS_NAMES = {
+    0: "OK",
+    1: "NULL pointer",
+    2: "bad shape",
+    3: "bad dtype",
+    4: "misaligned pointer",
+    5: "unsupported combination",
+    6: "workspace too small",
+    7: "kernel launch failed",
+}
+
+
+class StmoeWeight(Structure):
+    _fields_ = [
+        ("format", c_int32),
+        ("dtype", c_int32),
+        ("experts", c_int64),
+        ("rows", c_int64),
+        ("cols", c_int64),
+        ("qs", c_void_p),
+        ("d", c_void_p),
+        ("m", c_void_p),
+        ("d_count", c_int64),
+    ]
+
+
+# name -> (restype, argtypes); kept in one table so a test can check that the library exports them all.
+SIGNATURES = {
+    "stmoe_last_error": (c_char_p, []),
+    "stmoe_abi_version": (c_int, []),
+    "stmoe_dequant_block_scaled": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_void_p, c_int, c_void_p]),
+    "stmoe_dequant_block_scaled_i4": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p, c_int, c_void_p]),
+    "stmoe_promote_i4": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
+    "stmoe_dequant_tensor_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p]),
+    "stmoe_quantize_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
+    "stmoe_rms_norm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_float, c_void_p, c_void_p]),
+    "stmoe_router_topk": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "stmoe_dispatch_build": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "stmoe_grouped_ffn_workspace_bytes": (c_size_t, [c_int64, c_int, c_int64, c_int64, c_int]),
+    "stmoe_moe_forward_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int64, c_int64, c_int]),
+    "stmoe_grouped_ffn": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, POINTER(StmoeWeight), POINTER(StmoeWeight),
+                                  POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    "stmoe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int64, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p]),
+    "stmoe_moe_forward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
+                                  POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_size_t, c_int, c_void_p]),
+    "stmoe_mmt": (c_int, [c_void_p, c_int, c_int64, POINTER(StmoeWeight), c_void_p, c_int, c_void_p]),
+}
+
+_lib = None
+
+
+class StmoeError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"sharktank_moe_hip: {STATUS_NAMES.get(status, status)}: {message}")
+        self.status = status
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def load_library() -> ctypes.CDLL:
+    """Loads the shared library; raises (never falls back) when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise RuntimeError(
+            f"{_LIB_PATH} is missing: build it with `make -C shark-platform_amd/csrc` "
+            "(or __graft_entry__.build()). sharktank_amd has no other compute path."
+        )
+    lib = ctypes.CDLL(_LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def _check(status: int):
+    if status != 0:
+        msg = load_library().stmoe_last_error()
+        err = StmoeError(status, msg.decode() if msg else "")
+        # The reference signals a missing kernel for a type combination with NotImplementedError.
+        if status == 5:
+            raise NotImplementedError(str(err))
+        raise err
+
+
+def dtype_enum(dt: torch.dtype) -> int:
+    try:
+        return _DTYPE_ENUM[dt]
+    except KeyError:
+        raise TypeError(f"sharktank_amd: dtype {dt} has no kernel support") from None
+
+
+def _dev(*tensors: Optional[torch.Tensor]) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "sharktank_amd computes on the GPU only: got a host tensor "
+                f"({tuple(t.shape)}, {t.dtype}); move the parameters and inputs to the device first"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _contig(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    return None if t is None else t.contiguous()
+
+
+# ---- dequantisation -------------------------------------------------------------------------------
+
+
+def dequant_block_scaled(d, qs, m, dtype: Optional[torch.dtype]) -> torch.Tensor:
+    """BlockScaledLayout.dequant_blocked: returns a tensor shaped like `qs`."""
+    dev = _dev(d, qs, m)
+    lib = load_library()
+    out_dtype = d.dtype if dtype is None else dtype
+    d_c, qs_c, m_c = _contig(d), _contig(qs), _contig(m)
+    if qs_c.dtype != torch.int8:
+        raise TypeError(f"BlockScaledLayout qs must be int8, got {qs_c.dtype}")
+    block = qs_c.shape[-1]
+    n_blocks = qs_c.numel() // block if block else 0
+    out = torch.empty(qs_c.shape, dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_dequant_block_scaled(_ptr(d_c), _ptr(m_c), dtype_enum(d_c.dtype), _ptr(qs_c), n_blocks, block,
+                                              _ptr(out), dtype_enum(out_dtype), _stream(dev)))
+    return out
+
+
+def dequant_block_scaled_i4(d, qs_packed, m, signed: bool, dtype: Optional[torch.dtype]) -> torch.Tensor:
+    dev = _dev(d, qs_packed, m)
+    lib = load_library()
+    out_dtype = d.dtype if dtype is None else dtype
+    d_c, qs_c, m_c = _contig(d), _contig(qs_packed), _contig(m)
+    if qs_c.dtype not in (torch.uint8, torch.int8):
+        raise AssertionError(f"Expected tensor to by uint8 or int8. Got: {qs_c.dtype}")
+    block = qs_c.shape[-1] * 2
+    n_blocks = qs_c.numel() * 2 // block if block else 0
+    out = torch.empty(tuple(qs_c.shape[:-1]) + (block,), dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_dequant_block_scaled_i4(_ptr(d_c), _ptr(m_c), dtype_enum(d_c.dtype), _ptr(qs_c), n_blocks, block,
+                                                 int(bool(signed)), _ptr(out), dtype_enum(out_dtype), _stream(dev)))
+    return out
+
+
+def promote_i4_block(qs_packed, signed: bool) -> torch.Tensor:
+    dev = _dev(qs_packed)
+    lib = load_library()
+    qs_c = _contig(qs_packed)
+    if qs_c.dtype not in (torch.uint8, torch.int8):
+        raise AssertionError(f"Expected tensor to by uint8 or int8. Got: {qs_c.dtype}")
+    out = torch.empty(tuple(qs_c.shape[:-1]) + (qs_c.shape[-1] * 2,), dtype=torch.int8 if signed else torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_promote_i4(_ptr(qs_c), qs_c.numel(), int(bool(signed)), _ptr(out), _stream(dev)))
+    return out
+
+
+def dequant_tensor_scaled(qs, d, m, dtype: torch.dtype) -> torch.Tensor:
+    dev = _dev(qs, d, m)
+    lib = load_library()
+    qs_c, d_c = _contig(qs), _contig(d)
+    m_c = None if m is None else _contig(m).to(d_c.dtype)
+    n = qs_c.numel()
+    d_count = d_c.numel()
+    if d_count != 1:
+        # per-axis scales broadcast along one axis: only a leading-axis broadcast maps to contiguous runs
+        lead = qs_c.shape[0] if qs_c.dim() else 1
+        if d_count != lead or tuple(d_c.shape) not in ((lead,), (lead,) + (1,) * (qs_c.dim() - 1)):
+            raise NotImplementedError(f"TensorScaledLayout dequant: scale shape {tuple(d.shape)} for qs {tuple(qs.shape)}")
+    if m_c is not None and m_c.numel() != d_count:
+        raise NotImplementedError("TensorScaledLayout dequant: offset and scale must have the same shape")
+    out = torch.empty(qs_c.shape, dtype=dtype, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_dequant_tensor_scaled(_ptr(qs_c), dtype_enum(qs_c.dtype), _ptr(d_c), _ptr(m_c), dtype_enum(d_c.dtype),
+                                               d_count, n, _ptr(out), dtype_enum(dtype), _stream(dev)))
+    return out
+
+
+def quantize_fp8(x: torch.Tensor, rscale: torch.Tensor) -> torch.Tensor:
+    dev = _dev(x, rscale)
+    lib = load_library()
+    x_c = _contig(x)
+    rs = rscale.to(torch.float32).reshape(1)
+    out = torch.empty(x_c.shape, dtype=torch.float8_e4m3fn, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_quantize_fp8(_ptr(x_c), dtype_enum(x_c.dtype), _ptr(rs), x_c.numel(), _ptr(out), _stream(dev)))
+    return out
+
+
+# ---- layer pieces -----------------------------------------------------------------------------------
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, epsilon: float) -> torch.Tensor:
+    dev = _dev(x, weight)
+    lib = load_library()
+    x_c, w_c = _contig(x), _contig(weight)
+    K = x_c.shape[-1]
+    T = x_c.numel() // K if K else 0
+    out = torch.empty_like(x_c)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_rms_norm(_ptr(x_c), dtype_enum(x_c.dtype), _ptr(w_c), dtype_enum(w_c.dtype), T, K, float(epsilon),
+                                  _ptr(out), _stream(dev)))
+    return out
+
+
+def router_topk(x: torch.Tensor, w_router: torch.Tensor, k: int, *, want_logits: bool = False, index_dtype=torch.int32):
+    """x [T,K], w_router [E,K] (same dtype) -> (idx [T,k], gate [T,k], logits [T,E] | None)."""
+    dev = _dev(x, w_router)
+    lib = load_library()
+    x_c, w_c = _contig(x), _contig(w_router)
+    if w_c.dtype != x_c.dtype:
+        raise TypeError("router weight must already be cast to the activation dtype")
+    T, K = x_c.shape
+    E = w_c.shape[0]
+    idx = torch.empty((T, k), dtype=torch.int32, device=dev)
+    idx64 = torch.empty((T, k), dtype=torch.int64, device=dev) if index_dtype == torch.int64 else None
+    gate = torch.empty((T, k), dtype=x_c.dtype, device=dev)
+    logits = torch.empty((T, E), dtype=x_c.dtype, device=dev) if want_logits else None
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_router_topk(_ptr(x_c), _ptr(w_c), dtype_enum(x_c.dtype), T, K, E, k, _ptr(logits), _ptr(idx), _ptr(idx64),
+                                     _ptr(gate), _stream(dev)))
+    return (idx64 if idx64 is not None else idx), gate, logits
+
+
+def dispatch_build(idx: torch.Tensor, E: int):
+    """idx [T,k] int32 -> (counts [E], offsets [E+1], perm [T*k], inv [T*k]) int32."""
+    dev = _dev(idx)
+    lib = load_library()
+    idx_c = _contig(idx.to(torch.int32))
+    n = idx_c.numel()
+    counts = torch.empty(E, dtype=torch.int32, device=dev)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    perm = torch.empty(n, dtype=torch.int32, device=dev)
+    inv = torch.empty(n, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_dispatch_build(_ptr(idx_c), n, E, _ptr(counts), _ptr(offsets), _ptr(perm), _ptr(inv), _stream(dev)))
+    return counts, offsets, perm, inv
+
+
+class DeviceWeight:
+    """An expert-stacked weight `[E, rows, cols]` as the C ABI sees it; keeps its planes alive."""
+
+    def __init__(self, fmt: int, experts: int, rows: int, cols: int, qs, d=None, m=None, dtype_tag: int = 0):
+        self.keep = (qs, d, m)
+        self.device = _dev(qs, d, m)
+        self.desc = StmoeWeight(
+            format=fmt, dtype=dtype_tag, experts=experts, rows=rows, cols=cols,
+            qs=_ptr(qs), d=_ptr(d), m=_ptr(m), d_count=(d.numel() if (d is not None and fmt == W_FP8) else 1),
+        )
+        self.format = fmt
+        self.experts, self.rows, self.cols = experts, rows, cols
+
+    @property
+    def ref(self):
+        return ctypes.byref(self.desc)
+
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.keep if t is not None)
+
+
+def grouped_ffn_workspace_bytes(T: int, k: int, K: int, N: int, dtype: torch.dtype) -> int:
+    return int(load_library().stmoe_grouped_ffn_workspace_bytes(T, k, K, N, dtype_enum(dtype)))
+
+
+def grouped_ffn(x, w_gate: DeviceWeight, w_up: DeviceWeight, w_down: DeviceWeight, act: int, offsets, perm, k: int,
+                *, variant: int = VARIANT_AUTO, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [T,K] -> y_sorted [T*k, K] (rows in dispatch order)."""
+    dev = _dev(x, offsets, perm)
+    lib = load_library()
+    x_c = _contig(x)
+    T, K = x_c.shape
+    N, E = w_gate.rows, w_gate.experts
+    need = grouped_ffn_workspace_bytes(T, k, K, N, x_c.dtype)
+    if workspace is None:
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    y = torch.empty((T * k, K), dtype=x_c.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_grouped_ffn(_ptr(x_c), dtype_enum(x_c.dtype), T, K, N, E, k, w_gate.ref, w_up.ref, w_down.ref, act,
+                                     _ptr(offsets), _ptr(perm), None, _ptr(y), _ptr(workspace), workspace.numel(), variant,
+                                     _stream(dev)))
+    return y
+
+
+def combine(y_sorted, gate, inv, T: int, k: int, *, out_norm_w=None, eps: float = 0.0, residual=None) -> torch.Tensor:
+    dev = _dev(y_sorted, gate, inv, out_norm_w, residual)
+    lib = load_library()
+    K = y_sorted.shape[-1]
+    y_c, g_c = _contig(y_sorted), _contig(gate)
+    res_c = None if residual is None else _contig(residual)
+    w_c = None if out_norm_w is None else _contig(out_norm_w)
+    out = torch.empty((T, K), dtype=y_c.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_combine(_ptr(y_c), _ptr(g_c), _ptr(inv), dtype_enum(y_c.dtype), T, k, K, _ptr(w_c),
+                                 dtype_enum(w_c.dtype) if w_c is not None else F32, float(eps), _ptr(res_c), _ptr(out), _stream(dev)))
+    return out
+
+
+def moe_forward_workspace_bytes(T: int, k: int, E: int, K: int, N: int, dtype: torch.dtype) -> int:
+    return int(load_library().stmoe_moe_forward_workspace_bytes(T, k, E, K, N, dtype_enum(dtype)))
+
+
+def moe_forward(h, ffn_norm_w, out_norm_w, eps: float, w_router, w_gate: DeviceWeight, w_up: DeviceWeight, w_down: DeviceWeight,
+                act: int, k: int, *, variant: int = VARIANT_AUTO, workspace: Optional[torch.Tensor] = None, want_routing: bool = False):
+    """h [T,K] -> out [T,K] (and, if asked, idx int32 [T,k] and gate [T,k])."""
+    dev = _dev(h, ffn_norm_w, out_norm_w, w_router)
+    lib = load_library()
+    h_c = _contig(h)
+    T, K = h_c.shape
+    N, E = w_gate.rows, w_gate.experts
+    need = moe_forward_workspace_bytes(T, k, E, K, N, h_c.dtype)
+    if workspace is None or workspace.numel() < need:
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    out = torch.empty_like(h_c)
+    idx = torch.empty((T, k), dtype=torch.int32, device=dev) if want_routing else None
+    gate = torch.empty((T, k), dtype=h_c.dtype, device=dev) if want_routing else None
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_moe_forward(_ptr(h_c), dtype_enum(h_c.dtype), T, K, N, E, k, _ptr(ffn_norm_w), _ptr(out_norm_w),
+                                     dtype_enum(ffn_norm_w.dtype), float(eps), _ptr(w_router), w_gate.ref, w_up.ref, w_down.ref, act,
+                                     _ptr(out), _ptr(idx), _ptr(gate), _ptr(workspace), workspace.numel(), variant, _stream(dev)))
+    if want_routing:
+        return out, idx, gate
+    return out
+
+
+def mmt(a: torch.Tensor, w: DeviceWeight, *, variant: int = VARIANT_AUTO) -> torch.Tensor:
+    """a [..., K] @ W[rows, K]^T -> [..., rows] in a's dtype."""
+    dev = _dev(a)
+    lib = load_library()
+    a_c = _contig(a)
+    K = a_c.shape[-1]
+    M = a_c.numel() // K if K else 0
+    out = torch.empty(tuple(a_c.shape[:-1]) + (w.rows,), dtype=a_c.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_mmt(_ptr(a_c), dtype_enum(a_c.dtype), M, w.ref, _ptr(out), variant, _stream(dev)))
+    return out

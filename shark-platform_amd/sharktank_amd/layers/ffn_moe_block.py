@@ -1,0 +1,62 @@
+"""Drop-in for sharktank's PreGatherFFNMOE (sharktank/sharktank/layers/ffn_moe_block.py:23-74).
+
+Same constructor, attributes and `forward(h, experts, expert_gate)` contract.  Instead of gathering a
+[T,k,N,K] copy of the expert weights per token and running T batched M=1 products, the rows are grouped by
+expert (stable counting sort of the (token, slot) pairs) and the three projections run as grouped kernels over
+the stacked, still-quantized weights; the slot-weighted sum is the combine kernel.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+from .. import _hip
+from ..ops import device_weight
+from ..types import Theta
+from .base import ThetaLayer
+
+__all__ = ["PreGatherFFNMOE", "activation_enum"]
+
+
+def activation_enum(activation) -> int:
+    """Maps the reference's activation callables to kernel enums: F.silu (default, ffn_moe_block.py:27) and
+    F.gelu in its exact erf form (Grok, sharktank/sharktank/models/grok/grok.py:108)."""
+    if activation is F.silu or isinstance(activation, torch.nn.SiLU):
+        return _hip.ACT_SILU
+    if activation is F.gelu or (isinstance(activation, torch.nn.GELU) and activation.approximate == "none"):
+        return _hip.ACT_GELU_ERF
+    raise NotImplementedError(f"PreGatherFFNMOE: no kernel epilogue for activation {activation!r} (have F.silu, F.gelu)")
+
+
+class PreGatherFFNMOE(ThetaLayer):
+    def __init__(self, theta: Theta, activation=F.silu):
+        super().__init__(theta)
+        self.ffn_gate = theta.tensor("ffn_gate_exps", "weight")
+        self.ffn_up = theta.tensor("ffn_up_exps", "weight")
+        self.ffn_down = theta.tensor("ffn_down_exps", "weight")
+        self.activation = activation
+        self._act = activation_enum(activation)
+        self._dw = None
+        self.kernel_variant = _hip.VARIANT_AUTO
+
+    def device_weights(self):
+        """C-ABI descriptors of the three stacked weights, built once (planes made contiguous once)."""
+        if self._dw is None:
+            self._dw = (
+                device_weight(self.ffn_gate, stacked=True),
+                device_weight(self.ffn_up, stacked=True),
+                device_weight(self.ffn_down, stacked=True),
+            )
+        return self._dw
+
+    @property
+    def expert_count(self) -> int:
+        return int(self.ffn_gate.shape[0])
+
+    def forward(self, h: torch.Tensor, experts: torch.Tensor, expert_gate: torch.Tensor):
+        wg, wu, wd = self.device_weights()
+        T, k = experts.shape
+        _, offsets, perm, inv = _hip.dispatch_build(experts, wg.experts)
+        y = _hip.grouped_ffn(h, wg, wu, wd, self._act, offsets, perm, k, variant=self.kernel_variant)
+        return _hip.combine(y, expert_gate.to(h.dtype), inv, T, k)

@@ -1,0 +1,72 @@
+"""Drop-in for sharktank's MoeBlock (sharktank/sharktank/layers/mixture_of_experts_block.py:23-90): same
+constructor arguments, sub-module names and `forward(h [B,S,K]) -> [B,S,K]`.
+
+forward = ffn_norm -> router (logits, fp32 softmax, top-k, renormalise) -> PreGatherFFNMOE ->
+layer_output_norm -> residual, run as one C-ABI call that enqueues the HIP kernels back to back on the current
+stream with one caller-owned workspace.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+from .. import _hip
+from ..types import Theta, unbox_tensor
+from .base import ThetaLayer
+from .ffn_moe_block import PreGatherFFNMOE
+from .linear import LinearLayer
+from .norm import RMSNormLayer
+
+__all__ = ["MoeBlock"]
+
+
+class MoeBlock(ThetaLayer):
+    def __init__(self, theta: Theta, expert_count: int, expert_used_count: int, rms_epsilon: float, moe_activation=F.silu):
+        super().__init__(theta)
+        self.expert_count = expert_count
+        self.expert_used_count = expert_used_count
+        self.rms_epsilon = rms_epsilon
+
+        self.add_module("ffn_gate_inp", LinearLayer(theta("ffn_gate_inp")))
+        self.add_module("ffn_norm", RMSNormLayer(theta("ffn_norm"), epsilon=rms_epsilon))
+        if theta.optional_tensor("layer_output_norm") is not None:
+            self.add_module("layer_output_norm", RMSNormLayer(theta("layer_output_norm"), epsilon=rms_epsilon))
+        else:
+            self.add_module("layer_output_norm", torch.nn.Identity())
+        self.experts = PreGatherFFNMOE(theta, activation=moe_activation)
+
+        self._router_w = {}  # activation dtype -> router matrix cast to it (the reference casts on every call)
+        self._workspace: Optional[torch.Tensor] = None
+        self.last_routing = None
+
+    def _router_weight(self, dtype: torch.dtype) -> torch.Tensor:
+        w = self._router_w.get(dtype)
+        if w is None:
+            w = unbox_tensor(self.ffn_gate_inp.weight).to(dtype).contiguous()
+            self._router_w[dtype] = w
+        return w
+
+    def forward(self, h: torch.Tensor, *, return_routing: bool = False):
+        batch_size, sequence_length, feature_dim = h.shape
+        x = h.reshape(-1, feature_dim)
+        T = x.shape[0]
+        wg, wu, wd = self.experts.device_weights()
+        if wg.experts != self.expert_count:
+            raise ValueError(f"expert_count {self.expert_count} != stacked weight experts {wg.experts}")
+        out_norm = self.layer_output_norm
+        out_norm_w = unbox_tensor(out_norm.weight) if isinstance(out_norm, RMSNormLayer) else None
+        need = _hip.moe_forward_workspace_bytes(T, self.expert_used_count, self.expert_count, feature_dim, wg.rows, h.dtype)
+        if self._workspace is None or self._workspace.numel() < need or self._workspace.device != h.device:
+            self._workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=h.device)
+        res = _hip.moe_forward(
+            x, unbox_tensor(self.ffn_norm.weight), out_norm_w, self.rms_epsilon, self._router_weight(h.dtype),
+            wg, wu, wd, self.experts._act, self.expert_used_count,
+            variant=self.experts.kernel_variant, workspace=self._workspace, want_routing=return_routing,
+        )
+        if return_routing:
+            out, idx, gate = res
+            return out.reshape(batch_size, sequence_length, feature_dim), idx, gate
+        return res.reshape(batch_size, sequence_length, feature_dim)

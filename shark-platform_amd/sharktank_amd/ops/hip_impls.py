@@ -1,0 +1,142 @@
+"""GPU implementations of the `sharktank.ops` operators on the MoE path, registered through the same
+`@op.override(...)` protocol the reference uses for its own kernels
+(sharktank/sharktank/ops/custom_impls.py:54-103, default_impls.py:108-128,204-218,328-359,402-408).
+Arithmetic runs in the HIP library; torch is used for allocation, views and dtype/device moves.
+Anything not implemented returns `NotImplemented`, which surfaces as the reference's NotImplementedError.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from .. import _hip
+from ..types.layouts import BlockScaledI4Layout, BlockScaledLayout, TensorScaledLayout
+from ..types.tensors import InferenceTensor, PrimitiveTensor, QuantizedTensor, unbox_tensor
+from ._registry import AllOfType
+from .signatures import *
+
+__all__ = ["device_weight"]
+
+_FLOAT_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
+
+
+def device_weight(w, *, stacked: bool) -> _hip.DeviceWeight:
+    """C-ABI descriptor of a weight tensor.  `stacked`: [E, rows, cols]; otherwise a single [rows, cols] matrix.
+    Planes are made contiguous once here (GGUF-derived planes are strided views of the raw blocks)."""
+    shape = list(w.shape)
+    if stacked:
+        assert len(shape) == 3, f"expert-stacked weight must be [E, rows, cols], got {shape}"
+        experts, rows, cols = shape
+    else:
+        assert len(shape) == 2, f"weight must be [rows, cols], got {shape}"
+        experts, (rows, cols) = 1, shape
+    if isinstance(w, QuantizedTensor):
+        layout = w.unpack()
+        if type(layout) is BlockScaledLayout:
+            assert layout.m is None, "NYI: Q8 block scaled with offset"
+            if layout.qs.shape[-1] != 32 or layout.d.dtype != torch.float16:
+                raise NotImplementedError("BlockScaledLayout kernels exist for block 32 with fp16 scales (Q8_0) only")
+            return _hip.DeviceWeight(_hip.W_Q8_0, experts, rows, cols, layout.qs.contiguous(), layout.d.contiguous())
+        if type(layout) is BlockScaledI4Layout:
+            assert layout.m is not None, "NYI: Q4 without offset not"
+            assert not layout.signed, "NYI: Q4 signed"
+            if layout.qs_bit_packed.shape[-1] != 16 or layout.d.dtype != torch.float16:
+                raise NotImplementedError("BlockScaledI4Layout kernels exist for block 32 with fp16 d/m (Q4_1) only")
+            return _hip.DeviceWeight(_hip.W_Q4_1, experts, rows, cols, layout.qs_bit_packed.contiguous(),
+                                     layout.d.contiguous(), layout.m.contiguous())
+        if type(layout) is TensorScaledLayout:
+            if layout.m is not None or layout.qs.dtype != torch.float8_e4m3fn:
+                raise NotImplementedError("TensorScaledLayout kernels exist for offset-free float8_e4m3fn samples only")
+            d = layout.d.contiguous().reshape(-1)
+            if d.numel() not in (1, experts) or d.dtype not in (torch.float32, torch.float16):
+                raise NotImplementedError("TensorScaledLayout kernels take one f32/f16 scale per tensor or per expert")
+            if layout.dtype != d.dtype:
+                raise NotImplementedError("TensorScaledLayout kernels produce the scale's dtype before the activation cast")
+            return _hip.DeviceWeight(_hip.W_FP8, experts, rows, cols, layout.qs.contiguous(), d, None, _hip.dtype_enum(d.dtype))
+        raise NotImplementedError(f"no kernel for layout {type(layout).__name__}")
+    t = unbox_tensor(w).contiguous()
+    if t.dtype not in _FLOAT_DTYPES:
+        raise NotImplementedError(f"no kernel for dense weights of dtype {t.dtype}")
+    return _hip.DeviceWeight(_hip.W_DENSE, experts, rows, cols, t, None, None, _hip.dtype_enum(t.dtype))
+
+
+# ---- plumbing ops ---------------------------------------------------------------------------------------
+
+
+@to.override(Tensor)
+def to_default(tensor, *args, **kwargs):
+    return unbox_tensor(tensor).to(*args, **kwargs)
+
+
+@view.override(Tensor)
+def view_default(tensor, shape):
+    return unbox_tensor(tensor).view(*shape)
+
+
+@elementwise.override(Tensor)
+def elementwise_unary(operator, x, *args, **kwargs):
+    return operator(unbox_tensor(x), *args, **kwargs)
+
+
+@elementwise.override(Tensor, Tensor)
+def elementwise_binary(operator, x, y, *args, **kwargs):
+    return operator(unbox_tensor(x), unbox_tensor(y), *args, **kwargs)
+
+
+# ---- arithmetic ops -------------------------------------------------------------------------------------
+
+
+@rms_norm.override(AllOfType(Tensor, InferenceTensor))
+def rms_norm_hip(x, weight, *, epsilon: float):
+    x = unbox_tensor(x)
+    weight = unbox_tensor(weight)
+    if x.dtype not in _FLOAT_DTYPES:
+        return NotImplemented
+    # the reference multiplies by the weight in the weight's dtype and returns that dtype
+    # (sharktank/sharktank/ops/default_impls.py:402-408); RMSNormLayer casts x to fp32 before and back after.
+    if x.dtype == torch.float32 and weight.dtype == torch.float32:
+        return _hip.rms_norm(x, weight, epsilon)
+    return NotImplemented
+
+
+def _mmt_2d(lhs: torch.Tensor, dw: _hip.DeviceWeight):
+    return _hip.mmt(lhs, dw)
+
+
+@matmul.override(Tensor, QuantizedTensor)
+def matmul_tensor_quantized(lhs, rhs: QuantizedTensor, *, transpose_rhs: bool):
+    lhs = unbox_tensor(lhs)
+    if not transpose_rhs or len(rhs.shape) != 2 or lhs.dtype not in _FLOAT_DTYPES:
+        return NotImplemented
+    return _mmt_2d(lhs, device_weight(rhs, stacked=False))
+
+
+@matmul.override(Tensor, Tensor)
+def matmul_tensor_tensor(lhs, rhs, *, transpose_rhs: bool):
+    lhs = unbox_tensor(lhs)
+    rhs = unbox_tensor(rhs)
+    if not transpose_rhs or rhs.dim() != 2 or lhs.dtype not in _FLOAT_DTYPES:
+        return NotImplemented
+    return _mmt_2d(lhs, device_weight(rhs.to(lhs.dtype), stacked=False))
+
+
+def _linear(input, weight, bias, *, accum_dtype=None):
+    if bias is not None:
+        return NotImplemented
+    input = unbox_tensor(input)
+    if isinstance(weight, QuantizedTensor):
+        return matmul(input, weight, transpose_rhs=True)
+    weight = unbox_tensor(weight)
+    if weight.dtype != input.dtype:
+        weight = weight.to(dtype=input.dtype)
+    return matmul(input, weight, transpose_rhs=True)
+
+
+linear.override(Tensor, Tensor)(_linear)
+linear.override(Tensor, QuantizedTensor)(_linear)
+
+
+@get_index.override(AllOfType(Tensor, PrimitiveTensor))
+def get_index_default(tensor, key):
+    return unbox_tensor(tensor)[key]

@@ -1,0 +1,75 @@
+"""Activation quantizers that produce `TensorScaledLayout` tensors (mirror of
+sharktank/sharktank/types/quantizers.py:87-183 StaticScaledQuantizer, per-tensor fp8 case, which is the one the
+fp8 MoE configuration uses).  The cast runs in a HIP kernel."""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .layouts import TensorScaledLayout
+from .tensors import InferenceTensor, PlanarQuantizedTensor, QuantizedTensor, UnnamedTensorName, unbox_tensor
+
+__all__ = ["QuantizerTensor", "StaticScaledQuantizer"]
+
+
+class QuantizerTensor(InferenceTensor):
+    def quantize(self, t, *, name: str = UnnamedTensorName) -> QuantizedTensor:
+        return self._quantize_raw_tensor(unbox_tensor(t), name=name)
+
+    def _quantize_raw_tensor(self, t: torch.Tensor, *, name: str) -> QuantizedTensor:
+        raise NotImplementedError
+
+
+class StaticScaledQuantizer(QuantizerTensor):
+    def __init__(self, *, scale: torch.Tensor, dtype: torch.dtype, axis: Optional[int] = None,
+                 reciprocal_scale: Optional[torch.Tensor] = None, offset: Optional[torch.Tensor] = None,
+                 disable_saturate: bool = False, name: str = UnnamedTensorName):
+        super().__init__(shape=scale.shape, name=name)
+        if axis is not None or offset is not None or disable_saturate:
+            raise NotImplementedError("StaticScaledQuantizer: only the per-tensor, offset-free, saturating form has a kernel")
+        if dtype != torch.float8_e4m3fn:
+            raise NotImplementedError(f"StaticScaledQuantizer: target dtype {dtype} has no kernel (gfx950 MFMA consumes float8_e4m3fn)")
+        assert len(scale.shape) == 0, "Expected per-tensor scale to be 0D"
+        self._scale = scale
+        self._reciprocal_scale = reciprocal_scale if reciprocal_scale is not None else 1.0 / scale
+        self._dtype = dtype
+
+    @property
+    def axis(self):
+        return None
+
+    @property
+    def offset(self):
+        return None
+
+    @property
+    def scale(self):
+        return self._scale
+
+    @property
+    def reciprocal_scale(self):
+        return self._reciprocal_scale
+
+    @property
+    def dtype(self):
+        return self._dtype
+
+    @property
+    def globals(self):
+        return {f"{self.name}:d": self._scale, f"{self.name}:rscale": self._reciprocal_scale}
+
+    def _clone_with_globals(self, new_globals):
+        return StaticScaledQuantizer(name=self.name, scale=new_globals[f"{self.name}:d"],
+                                     reciprocal_scale=new_globals[f"{self.name}:rscale"], dtype=self._dtype)
+
+    def _quantize_raw_tensor(self, t: torch.Tensor, *, name: str) -> QuantizedTensor:
+        from .. import _hip
+
+        qs = _hip.quantize_fp8(t, self._reciprocal_scale)
+        shape = list(t.shape)
+        return PlanarQuantizedTensor(
+            shape=shape, name=name,
+            layout=TensorScaledLayout(shape=shape, d=self._reciprocal_scale, qs=qs, m=None, dtype=t.dtype),
+        )

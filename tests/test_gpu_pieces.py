@@ -1,0 +1,210 @@
+"""Parity of each HIP entry point against the CPU oracle (through the C ABI via the ctypes binding)."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import moe_oracle as O
+import moe_cases as MC
+
+pytestmark = pytest.mark.gpu
+
+
+def _hip():
+    from sharktank_amd import _hip
+
+    return _hip
+
+
+@pytest.mark.parametrize("out_dtype", [None, torch.float32, torch.bfloat16])
+def test_dequant_q8_0_bit_exact(device, out_dtype):
+    g = torch.Generator().manual_seed(1)
+    w = torch.randn(64, 256, generator=g) * 0.02
+    w[0, :32] = 0.0  # an all-zero block (d = 0)
+    w[1, :32] *= 1e-4  # subnormal fp16 products
+    d, qs = O.quantize_q8_0(w)
+    want = O.dequant_block_scaled(d, qs, dtype=out_dtype)
+    got = _hip().dequant_block_scaled(d.to(device), qs.to(device), None, out_dtype).cpu()
+    assert got.dtype == want.dtype
+    assert torch.equal(got.view(torch.int16 if got.element_size() == 2 else torch.int32),
+                       want.view(torch.int16 if want.element_size() == 2 else torch.int32))
+
+
+@pytest.mark.parametrize("out_dtype", [None, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("signed", [False, True])
+def test_dequant_q4_1_bit_exact(device, out_dtype, signed):
+    g = torch.Generator().manual_seed(2)
+    w = torch.randn(48, 128, generator=g) * 0.02
+    d, m, qs = O.quantize_q4_1(w)
+    want = O.dequant_block_scaled_i4(d, qs, m, signed=signed, dtype=out_dtype)
+    got = _hip().dequant_block_scaled_i4(d.to(device), qs.to(device), m.to(device), signed, out_dtype).cpu()
+    assert got.dtype == want.dtype
+    view = torch.int16 if got.element_size() == 2 else torch.int32
+    assert torch.equal(got.view(view), want.view(view))
+
+
+def test_promote_i4_known_answer(device):
+    packed = torch.tensor([[0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]], dtype=torch.uint8)
+    u = _hip().promote_i4_block(packed.to(device), False).cpu()
+    s = _hip().promote_i4_block(packed.to(device), True).cpu()
+    assert u.dtype == torch.uint8 and s.dtype == torch.int8
+    assert u.tolist() == [list(range(16))]
+    assert s.tolist() == [[0, 1, 2, 3, 4, 5, 6, 7, -8, -7, -6, -5, -4, -3, -2, -1]]
+
+
+def test_dequant_tensor_scaled_known_answer(device):
+    # the reference's own vector: sharktank/tests/types/layouts_test.py:107-125
+    got = _hip().dequant_tensor_scaled(
+        torch.tensor([2.0, 3.0, 4.0], dtype=torch.float16, device=device),
+        torch.tensor(2.0, dtype=torch.float32, device=device),
+        torch.tensor(5.0, dtype=torch.float32, device=device), torch.float32).cpu()
+    assert got.tolist() == [-6.0, -4.0, -2.0]
+
+
+def test_dequant_fp8_bit_exact(device):
+    qs = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).repeat(4)
+    d = torch.tensor(0.0118, dtype=torch.float32)
+    for out_dtype in (torch.float32, torch.float16, torch.bfloat16):
+        want = O.dequant_tensor_scaled(d, qs, dtype=out_dtype)
+        got = _hip().dequant_tensor_scaled(qs.to(device), d.to(device), None, out_dtype).cpu()
+        ok = (got == want) | (got.isnan() & want.isnan())
+        assert bool(ok.all()), out_dtype
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_quantize_fp8_bit_exact(device, dtype):
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(4096, generator=g) * 3).to(dtype)
+    x[:4] = torch.tensor([1000.0, -1000.0, 0.0, 448.0]).to(dtype)
+    rscale = torch.tensor(0.0118, dtype=torch.float32)
+    want, _, _ = O.static_quantize_per_tensor(x, rscale, torch.float8_e4m3fn)
+    got = _hip().quantize_fp8(x.to(device), rscale.to(device)).cpu()
+    assert torch.equal(got.view(torch.uint8), want.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_rms_norm(device, dtype):
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(37, 1024, generator=g).to(dtype)
+    w = torch.ones(1024) + 0.1 * torch.randn(1024, generator=g)
+    want = O.rms_norm(x, w, 1e-5)
+    got = _hip().rms_norm(x.to(device), w.to(device), 1e-5).cpu()
+    assert O.rel_l2(got, want) < (1e-6 if dtype == torch.float32 else 1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T,K,E,k", [(64, 512, 8, 2), (33, 4096, 8, 2), (5, 1000 * 8, 16, 4), (1, 64, 3, 3)])
+def test_router_bit_exact(device, dtype, T, K, E, k):
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(T, K, generator=g).to(dtype)
+    wr = (torch.randn(E, K, generator=g) * 0.02)
+    idx, gate, logits = _hip().router_topk(x.to(device), wr.to(dtype).to(device), k, want_logits=True, index_dtype=torch.int64)
+    want_logits = O.router_logits_ordered(x, wr)
+    view = torch.int16 if dtype != torch.float32 else torch.int32
+    assert torch.equal(logits.cpu().view(view), want_logits.view(view)), "logit bits differ from the documented order"
+    want_idx, want_gate, _ = O.route(want_logits, k)
+    assert idx.dtype == torch.int64
+    assert torch.equal(idx.cpu(), want_idx)
+    assert O.rel_l2(gate.cpu(), want_gate) < (1e-6 if dtype == torch.float32 else 2e-3)
+    # against torch's own summation order: indices agree except where a logit sits on a rounding boundary
+    ref_idx, _, _ = O.route(O.router_logits(x, wr), k)
+    mism = int((ref_idx != want_idx).any(dim=1).sum())
+    assert mism <= max(1, T // 100), f"{mism} of {T} tokens route differently from torch.matmul logits"
+
+
+def test_router_ties_lower_index_first(device):
+    # identical router rows give identical logits: ties must resolve toward the lower expert index
+    x = torch.randn(16, 64, generator=torch.Generator().manual_seed(6)).to(torch.float16)
+    row = torch.randn(64, generator=torch.Generator().manual_seed(7)) * 0.02
+    wr = torch.stack([row, row * 0.5, row, row * 0.5, row, -row, row * 0.25, row]).to(torch.float16)
+    idx, gate, logits = _hip().router_topk(x.to(device), wr.to(device), 3, want_logits=True)
+    want_idx, want_gate, _ = O.route(O.router_logits_ordered(x, wr), 3)
+    assert torch.equal(idx.cpu().long(), want_idx)
+    lg = logits.cpu().float()
+    pos = lg[:, 0] > 0
+    assert torch.equal(idx.cpu()[pos].long(), torch.tensor([[0, 2, 4]]).expand(int(pos.sum()), 3))
+
+
+@pytest.mark.parametrize("T,k,E", [(1, 2, 8), (32, 2, 8), (2048, 2, 8), (3000, 4, 64), (7, 1, 1)])
+def test_dispatch_bit_exact(device, T, k, E):
+    g = torch.Generator().manual_seed(8)
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    counts, offsets, perm, inv = _hip().dispatch_build(idx.to(device), E)
+    wc, wo, wp, wi = O.dispatch_permutation(idx, E)
+    assert torch.equal(counts.cpu(), wc) and torch.equal(offsets.cpu(), wo)
+    assert torch.equal(perm.cpu(), wp) and torch.equal(inv.cpu(), wi)
+
+
+def test_dispatch_skewed_and_empty_experts(device):
+    idx = torch.zeros(500, 2, dtype=torch.int32)
+    idx[:, 1] = 5  # experts 1-4, 6, 7 receive nothing
+    counts, offsets, perm, inv = _hip().dispatch_build(idx.to(device), 8)
+    wc, wo, wp, wi = O.dispatch_permutation(idx, 8)
+    assert torch.equal(counts.cpu(), wc) and torch.equal(offsets.cpu(), wo)
+    assert torch.equal(perm.cpu(), wp) and torch.equal(inv.cpu(), wi)
+
+
+def _ffn_parity(device, case, variant, tol):
+    hip = _hip()
+    from sharktank_amd.ops import device_weight
+
+    case = MC.build(case)
+    x = case.planes["h"]
+    g = torch.Generator().manual_seed(case.seed + 100)
+    idx = torch.stack([torch.randperm(case.E, generator=g)[: case.k] for _ in range(case.T)])
+    gate = torch.rand(case.T, case.k, generator=g)
+    gate = (gate / gate.sum(-1, keepdim=True)).to(case.dtype)
+    wg, wu, wd = MC.dense_weights(case)
+    want = O.grouped_ffn_moe(x, idx, gate, wg, wu, wd, case.activation)
+    E, N, K = case.E, case.N, case.K
+    dws = [device_weight(MC.to_inference_tensor(case.fmt, case.planes[n], shp, n, device), stacked=True)
+           for n, shp in (("gate", [E, N, K]), ("up", [E, N, K]), ("down", [E, K, N]))]
+    _, offsets, perm, inv = hip.dispatch_build(idx.to(torch.int32).to(device), E)
+    act = hip.ACT_SILU if case.act == "silu" else hip.ACT_GELU_ERF
+    y = hip.grouped_ffn(x.to(device), dws[0], dws[1], dws[2], act, offsets, perm, case.k, variant=variant)
+    got = hip.combine(y, gate.to(device), inv, case.T, case.k).cpu()
+    err = O.rel_l2(got, want)
+    assert err < tol, f"rel-L2 {err:.3e} >= {tol}"
+    return got
+
+
+@pytest.mark.parametrize("fmt", ["dense", "q8_0", "q4_1", "fp8"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_ffn_generic_kernel(device, fmt, dtype):
+    tol = 1e-5 if dtype == torch.float32 else (1e-3 if dtype == torch.float16 else 8e-3)
+    _ffn_parity(device, MC.Case(T=24, K=128, N=256, fmt=fmt, dtype=dtype, seed=11), 1, tol)
+
+
+@pytest.mark.parametrize("fmt", ["dense", "q8_0", "q4_1", "fp8"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_ffn_mfma_tile_kernel(device, fmt, dtype, act):
+    tol = 1e-3 if dtype == torch.float16 else 8e-3
+    got = _ffn_parity(device, MC.Case(T=200, K=256, N=384, fmt=fmt, dtype=dtype, act=act, seed=12), 2, tol)
+    # and against the independent vector-ALU kernel
+    got2 = _ffn_parity(device, MC.Case(T=200, K=256, N=384, fmt=fmt, dtype=dtype, act=act, seed=12), 1, tol)
+    assert O.rel_l2(got, got2) < tol
+
+
+def test_combine_with_output_norm_and_residual(device):
+    hip = _hip()
+    g = torch.Generator().manual_seed(13)
+    T, k, K = 19, 2, 512
+    for dtype in (torch.float16, torch.bfloat16, torch.float32):
+        y = torch.randn(T * k, K, generator=g).to(dtype)
+        gate = torch.rand(T, k, generator=g).to(dtype)
+        inv = torch.randperm(T * k, generator=g).to(torch.int32)
+        h = torch.randn(T, K, generator=g).to(dtype)
+        w = torch.ones(K) + 0.1 * torch.randn(K, generator=g)
+        down = y[inv.long()].reshape(T, k, K)
+        o = torch.sum(gate.unsqueeze(-1) * down, dim=1)
+        want_plain = o
+        want_full = h + O.rms_norm(o, w, 1e-5)
+        got_plain = hip.combine(y.to(device), gate.to(device), inv.to(device), T, k).cpu()
+        got_full = hip.combine(y.to(device), gate.to(device), inv.to(device), T, k, out_norm_w=w.to(device), eps=1e-5,
+                               residual=h.to(device)).cpu()
+        tol = 1e-6 if dtype == torch.float32 else 2e-3
+        if dtype == torch.float16:
+            assert torch.equal(got_plain, want_plain)  # products and the fp32 slot sum are exact: one rounding each
+        assert O.rel_l2(got_plain, want_plain) < tol
+        assert O.rel_l2(got_full, want_full) < tol
