@@ -165,6 +165,18 @@ int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K, int64_t N,
                       const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
                       void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream);
 
+/* stmoe_moe_forward with per-stage timing for benchmarks: `events` is a host array of 12 hipEvent_t created by
+ * the caller (entries may be NULL); stage s is bracketed on `stream` by events[2s] and events[2s+1], with
+ * s = 0 ffn_norm, 1 router, 2 dispatch, 3 gate/up projection, 4 down projection, 5 combine.  No counterpart in
+ * the reference; it exists so a benchmark can time each kernel inside its timed region. */
+#define STMOE_FORWARD_STAGES 6
+int stmoe_moe_forward_timed(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                            const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
+                            const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
+                            const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
+                            void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream,
+                            void** events);
+
 /* x @ W^T for one quantised (or dense) matrix W [rows, cols]: the operand set of the reference's
  * `mmt_block_scaled_q8(a,d,qs)` (sharktank/sharktank/kernels/mmt_block_scaled_q8.py:30) and
  * `mmt_block_scaled_offset_q4_unsigned(a,d,qs,m)` (mmt_block_scaled_offset_q4.py:31), reached from

@@ -59,11 +59,15 @@ extern "C" size_t stmoe_grouped_ffn_workspace_bytes(int64_t T, int k, int64_t K,
   return align_up((size_t)T * k * N * dtype_size(dtype), 256);
 }
 
-extern "C" int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
-                                 const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
-                                 int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
-                                 void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
-                                 stmoe_stream_t stream) {
+static inline void mark(void** events, int i, hipStream_t st) {
+  if (events && events[i]) (void)hipEventRecord(reinterpret_cast<hipEvent_t>(events[i]), st);
+}
+
+static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                            const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
+                            int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
+                            void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
+                            stmoe_stream_t stream, void** events) {
   STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1, STMOE_ERR_SHAPE, "grouped_ffn: T=%lld K=%lld N=%lld E=%d k=%d",
                 (long long)T, (long long)K, (long long)N, E, k);
   STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
@@ -92,13 +96,27 @@ extern "C" int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K,
   p.a = x; p.lda = K; p.perm = perm; p.k_top = k; p.offsets = offsets; p.E = E; p.fixed_rows = 0;
   p.w0 = make_view(w_gate); p.w1 = make_view(w_up);
   p.out = workspace; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr;
+  mark(events, 0, st);
   if ((rc = run_projection(variant, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st))) return rc;
+  mark(events, 1, st);
 
   GemmParams q{};
   q.a = workspace; q.lda = N; q.perm = nullptr; q.k_top = 1; q.offsets = offsets; q.E = E; q.fixed_rows = 0;
   q.w0 = make_view(w_down); q.w1 = q.w0;
   q.out = y_sorted; q.ldo = K; q.n_out = K; q.kred = N; q.act = act; q.x_scale = nullptr;
-  return run_projection(variant, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
+  mark(events, 2, st);
+  rc = run_projection(variant, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
+  mark(events, 3, st);
+  return rc;
+}
+
+extern "C" int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                                 const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
+                                 int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
+                                 void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
+                                 stmoe_stream_t stream) {
+  return grouped_ffn_impl(x, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, y_sorted,
+                          workspace, workspace_bytes, variant, stream, nullptr);
 }
 
 extern "C" int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight* w, void* out, int variant,
@@ -151,11 +169,12 @@ extern "C" size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int
   return carve(T, k, E, K, N, dtype).total;
 }
 
-extern "C" int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
-                                 const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
-                                 const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
-                                 const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
-                                 void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream) {
+static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                            const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
+                            const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
+                            const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
+                            void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream,
+                            void** events) {
   STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1 && k <= E, STMOE_ERR_SHAPE,
                 "moe_forward: T=%lld K=%lld N=%lld E=%d k=%d", (long long)T, (long long)K, (long long)N, E, k);
   if (T == 0) return STMOE_OK;
@@ -174,11 +193,42 @@ extern "C" int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K,
   int32_t* inv = (int32_t*)(base + ws.inv);
   void* y = base + ws.y;
   int rc;
+  hipStream_t st = as_stream(stream);
+  // stages: 0 rms_norm, 1 router, 2 dispatch, 3 gate/up projection, 4 down projection, 5 combine;
+  // stage s is bracketed by events[2s] and events[2s+1]
+  mark(events, 0, st);
   if ((rc = stmoe_rms_norm(h, dtype, ffn_norm_w, w_dtype, T, K, eps, xn, stream))) return rc;
+  mark(events, 1, st);
+  mark(events, 2, st);
   if ((rc = stmoe_router_topk(xn, w_router, dtype, T, K, E, k, nullptr, idx, nullptr, gate, stream))) return rc;
+  mark(events, 3, st);
+  mark(events, 4, st);
   if ((rc = stmoe_dispatch_build(idx, T * k, E, counts, offsets, perm, inv, stream))) return rc;
-  if ((rc = stmoe_grouped_ffn(xn, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, nullptr, y,
-                              base + ws.ffn, workspace_bytes - ws.ffn, variant, stream)))
+  mark(events, 5, st);
+  if ((rc = grouped_ffn_impl(xn, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, nullptr, y,
+                             base + ws.ffn, workspace_bytes - ws.ffn, variant, stream, events ? events + 6 : nullptr)))
     return rc;
-  return stmoe_combine(y, gate, inv, dtype, T, k, K, out_norm_w, w_dtype, eps, h, out, stream);
+  mark(events, 10, st);
+  rc = stmoe_combine(y, gate, inv, dtype, T, k, K, out_norm_w, w_dtype, eps, h, out, stream);
+  mark(events, 11, st);
+  return rc;
+}
+
+extern "C" int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                                 const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
+                                 const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
+                                 const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
+                                 void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream) {
+  return moe_forward_impl(h, dtype, T, K, N, E, k, ffn_norm_w, out_norm_w, w_dtype, eps, w_router, w_gate, w_up, w_down,
+                          act, out, idx_out, gate_out, workspace, workspace_bytes, variant, stream, nullptr);
+}
+
+extern "C" int stmoe_moe_forward_timed(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                                       const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
+                                       const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
+                                       const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
+                                       void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream,
+                                       void** events) {
+  return moe_forward_impl(h, dtype, T, K, N, E, k, ffn_norm_w, out_norm_w, w_dtype, eps, w_router, w_gate, w_up, w_down,
+                          act, out, idx_out, gate_out, workspace, workspace_bytes, variant, stream, events);
 }

@@ -80,6 +80,9 @@ SIGNATURES = {
     "stmoe_moe_forward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
                                   POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_size_t, c_int, c_void_p]),
+    "stmoe_moe_forward_timed": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
+                                        POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_size_t, c_int, c_void_p, POINTER(c_void_p)]),
     "stmoe_mmt": (c_int, [c_void_p, c_int, c_int64, POINTER(StmoeWeight), c_void_p, c_int, c_void_p]),
 }
 
@@ -354,8 +357,10 @@ def moe_forward_workspace_bytes(T: int, k: int, E: int, K: int, N: int, dtype: t
 
 
 def moe_forward(h, ffn_norm_w, out_norm_w, eps: float, w_router, w_gate: DeviceWeight, w_up: DeviceWeight, w_down: DeviceWeight,
-                act: int, k: int, *, variant: int = VARIANT_AUTO, workspace: Optional[torch.Tensor] = None, want_routing: bool = False):
-    """h [T,K] -> out [T,K] (and, if asked, idx int32 [T,k] and gate [T,k])."""
+                act: int, k: int, *, variant: int = VARIANT_AUTO, workspace: Optional[torch.Tensor] = None, want_routing: bool = False,
+                out: Optional[torch.Tensor] = None, events=None):
+    """h [T,K] -> out [T,K] (and, if asked, idx int32 [T,k] and gate [T,k]).  `events`: optional ctypes array of
+    12 hipEvent_t handles that bracket the six stages (see stmoe_moe_forward_timed)."""
     dev = _dev(h, ffn_norm_w, out_norm_w, w_router)
     lib = load_library()
     h_c = _contig(h)
@@ -364,13 +369,18 @@ def moe_forward(h, ffn_norm_w, out_norm_w, eps: float, w_router, w_gate: DeviceW
     need = moe_forward_workspace_bytes(T, k, E, K, N, h_c.dtype)
     if workspace is None or workspace.numel() < need:
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
-    out = torch.empty_like(h_c)
+    if out is None:
+        out = torch.empty_like(h_c)
     idx = torch.empty((T, k), dtype=torch.int32, device=dev) if want_routing else None
     gate = torch.empty((T, k), dtype=h_c.dtype, device=dev) if want_routing else None
+    args = (_ptr(h_c), dtype_enum(h_c.dtype), T, K, N, E, k, _ptr(ffn_norm_w), _ptr(out_norm_w),
+            dtype_enum(ffn_norm_w.dtype), float(eps), _ptr(w_router), w_gate.ref, w_up.ref, w_down.ref, act,
+            _ptr(out), _ptr(idx), _ptr(gate), _ptr(workspace), workspace.numel(), variant, _stream(dev))
     with torch.cuda.device(dev):
-        _check(lib.stmoe_moe_forward(_ptr(h_c), dtype_enum(h_c.dtype), T, K, N, E, k, _ptr(ffn_norm_w), _ptr(out_norm_w),
-                                     dtype_enum(ffn_norm_w.dtype), float(eps), _ptr(w_router), w_gate.ref, w_up.ref, w_down.ref, act,
-                                     _ptr(out), _ptr(idx), _ptr(gate), _ptr(workspace), workspace.numel(), variant, _stream(dev)))
+        if events is None:
+            _check(lib.stmoe_moe_forward(*args))
+        else:
+            _check(lib.stmoe_moe_forward_timed(*args, events))
     if want_routing:
         return out, idx, gate
     return out

@@ -1,0 +1,66 @@
+"""The C-ABI library loads without a GPU and exports every symbol the public header declares."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "sharktank_moe_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(stmoe_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for name in ("stmoe_router_topk", "stmoe_dispatch_build", "stmoe_grouped_ffn", "stmoe_combine", "stmoe_moe_forward",
+                 "stmoe_dequant_block_scaled", "stmoe_dequant_block_scaled_i4", "stmoe_dequant_tensor_scaled", "stmoe_mmt"):
+        assert name in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from sharktank_amd import _hip
+
+    lib = ctypes.CDLL(_hip.library_path())
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+
+
+def test_binding_table_matches_header():
+    from sharktank_amd import _hip
+
+    assert sorted(_hip.SIGNATURES) == declared_symbols()
+
+
+def test_argument_validation_without_a_gpu():
+    """Status codes come back before any launch, so these calls are safe on a host without a GPU."""
+    from sharktank_amd import _hip
+
+    lib = _hip.load_library()
+    assert lib.stmoe_abi_version() == 1
+    assert lib.stmoe_router_topk(None, None, _hip.F16, 4, 30, 8, 2, None, None, None, None, None) == 2  # K % 8
+    assert b"multiple of 8" in lib.stmoe_last_error()
+    assert lib.stmoe_router_topk(None, None, _hip.F16, 4, 64, 8, 9, None, None, None, None, None) == 2  # k > E
+    assert lib.stmoe_router_topk(None, None, _hip.F16, 4, 64, 8, 2, None, None, None, None, None) == 1  # NULL
+    assert lib.stmoe_router_topk(None, None, _hip.F16, 0, 64, 8, 2, None, None, None, None, None) == 0  # zero tokens
+    assert lib.stmoe_dispatch_build(None, 0, 0, None, None, None, None, None) == 2
+    assert lib.stmoe_dequant_block_scaled(None, None, _hip.F16, None, 0, 32, None, _hip.F16, None) == 0
+    assert lib.stmoe_grouped_ffn_workspace_bytes(32, 2, 4096, 14336, _hip.F16) == 32 * 2 * 14336 * 2
+    w = _hip.StmoeWeight(format=_hip.W_Q8_0, dtype=0, experts=8, rows=64, cols=48, qs=16, d=16, m=None, d_count=1)
+    rc = lib.stmoe_grouped_ffn(None, _hip.F16, 4, 48, 64, 8, 2, ctypes.byref(w), ctypes.byref(w), ctypes.byref(w), 0,
+                               None, None, None, None, None, 0, 0, None)
+    assert rc == 2 and b"32" in lib.stmoe_last_error()  # Q8_0 needs cols % 32 == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from sharktank_amd import _hip
+
+    monkeypatch.setattr(_hip, "_lib", None)
+    monkeypatch.setattr(_hip, "_LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="is missing"):
+        _hip.load_library()

@@ -1,0 +1,115 @@
+"""Host-side mirror of the reference interfaces: dispatch protocol, Theta, tensor wrappers (no GPU needed)."""
+
+import pytest
+import torch
+
+from sharktank_amd import ops
+from sharktank_amd import types as ST
+from sharktank_amd.ops._registry import AllOfType, AnyOfType, overridable
+
+
+def test_override_protocol_and_failure_message():
+    @overridable
+    def myop(a, b):
+        ...
+
+    @myop.trampoline
+    def _t(d, a, b):
+        for o in d.find_overrides((a, b)):
+            r = o(a, b)
+            if r is not NotImplemented:
+                return o, r
+        d.fail((a, b))
+
+    calls = []
+
+    @myop.override(torch.Tensor, torch.Tensor)
+    def first(a, b):
+        calls.append("first")
+        return "first"
+
+    @myop.override(torch.Tensor, torch.Tensor)
+    def second(a, b):
+        calls.append("second")
+        return NotImplemented
+
+    t = torch.zeros(1)
+    assert myop(t, t) == "first" and calls == ["second", "first"]  # later registration is tried first
+    # PrimitiveTensor auto-unboxes to Tensor; QuantizedTensor does not unless auto_dequant
+    assert myop(ST.DefaultPrimitiveTensor(data=t), t) == "first"
+    q = ST.PlanarQuantizedTensor(shape=[1, 32], layout=ST.BlockScaledLayout([1, 32], torch.zeros(1, 1, 1), torch.zeros(1, 1, 32, dtype=torch.int8)))
+    # message format pinned by the reference's test (sharktank/tests/ops/ops_test.py:109-116)
+    with pytest.raises(NotImplementedError, match=r"Overridable operator.+does not have an implementation for argument types:.+"):
+        myop(t, q)
+
+    @myop.override(AllOfType(torch.Tensor, ST.QuantizedTensor), salience=5)
+    def high(a, b):
+        return "high"
+
+    assert myop(t, q) == "high" and myop(t, t) == "high"
+    assert AnyOfType(int)(str, int) and not AnyOfType(int)(str, str)
+
+
+def test_last_op_dispatch_hook():
+    ops._test_enable_last_op_dispatch(True)
+    try:
+        t = ST.DefaultPrimitiveTensor(data=torch.zeros(2, 3))
+        ops.view(t, (3, 2))
+        assert ops._test_get_last_op_dispatch().__name__ == "view_default"
+    finally:
+        ops._test_enable_last_op_dispatch(False)
+
+
+def test_quantized_matmul_without_kernel_raises_not_implemented():
+    # matmul(Tensor, QuantizedTensor) with transpose_rhs=False has no kernel: every override declines
+    q = ST.PlanarQuantizedTensor(shape=[4, 32], layout=ST.BlockScaledLayout([4, 32], torch.zeros(4, 1, 1, dtype=torch.float16), torch.zeros(4, 1, 32, dtype=torch.int8)))
+    with pytest.raises(NotImplementedError, match="does not have an implementation"):
+        ops.matmul(torch.zeros(2, 32), q, transpose_rhs=False)
+
+
+def test_theta_accessors():
+    a = ST.DefaultPrimitiveTensor(name="ffn_norm.weight", data=torch.ones(4))
+    b = ST.DefaultPrimitiveTensor(name="ffn_gate_exps.weight", data=torch.ones(2, 3, 4))
+    theta = ST.Theta([a, b])
+    assert set(theta.keys) == {"ffn_norm", "ffn_gate_exps"}
+    assert theta.tensor("ffn_gate_exps", "weight") is b
+    assert theta("ffn_norm").tensor("weight") is a
+    assert theta.optional_tensor("layer_output_norm") is None
+    with pytest.raises(KeyError):
+        theta.tensor("nope")
+    assert set(theta.flatten()) == {"ffn_norm.weight", "ffn_gate_exps.weight"}
+
+
+def test_planar_globals_and_clone():
+    d = torch.ones(2, 1, 1, dtype=torch.float16)
+    m = torch.zeros(2, 1, 1, dtype=torch.float16)
+    qs = torch.zeros(2, 1, 16, dtype=torch.uint8)
+    q = ST.PlanarQuantizedTensor(name="w", shape=[2, 32], layout=ST.BlockScaledI4Layout([2, 32], d, qs, m=m, signed=False))
+    assert set(q.globals) == {"w:d", "w:m", "w:qs"}
+    moved = q.to(device="cpu")
+    assert isinstance(moved.unpack(), ST.BlockScaledI4Layout) and moved.unpack().signed is False
+    assert moved.layout_type is ST.BlockScaledI4Layout
+
+
+def test_gguf_raw_views_carry_no_arithmetic():
+    raw = torch.zeros(2 * 34, dtype=torch.uint8)
+    lay = ST.Q8_0(raw=raw, shape=[2, 32]).unpack()
+    assert lay.d.shape == (2, 1, 1) and lay.qs.shape == (2, 1, 32) and lay.d.dtype == torch.float16
+    raw4 = torch.zeros(2 * 20, dtype=torch.uint8)
+    lay4 = ST.Q4_1(raw=raw4, shape=[2, 32]).unpack()
+    assert lay4.qs_bit_packed.shape == (2, 1, 16) and lay4.m.shape == (2, 1, 1)
+
+
+def test_layers_refuse_host_tensors():
+    from sharktank_amd.layers import RMSNormLayer
+
+    theta = ST.Theta([ST.DefaultPrimitiveTensor(name="weight", data=torch.ones(8))])
+    with pytest.raises(RuntimeError, match="GPU only"):
+        RMSNormLayer(theta)(torch.zeros(2, 8))
+
+
+def test_unknown_activation_is_rejected():
+    from sharktank_amd.layers.ffn_moe_block import activation_enum
+
+    with pytest.raises(NotImplementedError):
+        activation_enum(torch.tanh)
