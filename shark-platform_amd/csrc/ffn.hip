@@ -37,9 +37,18 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
   return STMOE_OK;
 }
 
-// variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile
+// variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile, 3 skinny streaming kernel (decode)
+static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
-  if (variant == 0) variant = (dtype == STMOE_F32) ? 1 : 2;
+  if (variant == 0) {
+    if (dtype == STMOE_F32) variant = 1;
+    else variant = (p.offsets && p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ? 3 : 2;
+  }
+  if (variant == 3) {
+    int rc = launch_skinny(dtype, wtag, mode, p, max_rows, st);
+    if (rc != STMOE_ERR_UNSUPPORTED) return rc;
+    variant = 2;
+  }
   if (variant == 2) {
     int rc = launch_mfma_tile(dtype, wtag, mode, p, max_rows, st);
     if (rc != STMOE_ERR_UNSUPPORTED) return rc;
@@ -95,7 +104,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   GemmParams p{};
   p.a = x; p.lda = K; p.perm = perm; p.k_top = k; p.offsets = offsets; p.E = E; p.fixed_rows = 0;
   p.w0 = make_view(w_gate); p.w1 = make_view(w_up);
-  p.out = workspace; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr;
+  p.out = workspace; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr; p.expert_rows_bound = T;
   mark(events, 0, st);
   if ((rc = run_projection(variant, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st))) return rc;
   mark(events, 1, st);
@@ -103,7 +112,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   GemmParams q{};
   q.a = workspace; q.lda = N; q.perm = nullptr; q.k_top = 1; q.offsets = offsets; q.E = E; q.fixed_rows = 0;
   q.w0 = make_view(w_down); q.w1 = q.w0;
-  q.out = y_sorted; q.ldo = K; q.n_out = K; q.kred = N; q.act = act; q.x_scale = nullptr;
+  q.out = y_sorted; q.ldo = K; q.n_out = K; q.kred = N; q.act = act; q.x_scale = nullptr; q.expert_rows_bound = T;
   mark(events, 2, st);
   rc = run_projection(variant, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
   mark(events, 3, st);

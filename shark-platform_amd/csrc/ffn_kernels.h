@@ -27,6 +27,7 @@ struct GemmParams {
   int64_t kred;           // reduction length
   int32_t act;
   const float* x_scale;   // optional scale applied to the fp32 dot products (fp8 activations)
+  int64_t expert_rows_bound;  // host-side bound of rows per expert (a token gives an expert at most one row)
 };
 
 // (expert, first row, end row) of m-tile `slot` when every expert's rows are cut into tiles of BM.
@@ -70,4 +71,5 @@ namespace stmoe {
 // STMOE_ERR_UNSUPPORTED when the family has no instantiation for the combination.
 int launch_generic(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_mfma_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
+int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 }  // namespace stmoe

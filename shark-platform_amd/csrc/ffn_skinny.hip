@@ -1,0 +1,360 @@
+// Grouped projection for few rows per expert (decode): bandwidth-bound streaming of the expert weights.
+//
+// Every wavefront works alone (no LDS, no barriers).  A work item is one expert and 16 output features of
+// NT weight tiles (gate + up of the same features, or two adjacent 16-row tiles of the down matrix); the
+// wavefront walks the reduction dimension in chunks of 256, keeping one chunk of weights (and of the <= 16*MT
+// token rows, read through L2) in flight in registers while the matrix cores consume the previous one.
+// Weights are loaded with non-temporal 16-byte loads straight into the MFMA operand layout and dequantised
+// in registers.  Wavefronts are persistent: item ids are strided by the number of launched wavefronts, which
+// the host picks so that every wavefront gets the same number of items.
+//
+// MFMA roles as in the tile kernel: weight rows are the "A" rows, token rows the "B" columns.  Because the
+// operands of one MFMA only have to agree on which 32 reduction indices they cover, each format picks the
+// lane <-> k assignment that makes its own loads 16 bytes wide and row-contiguous:
+//   1 byte / element (Q8_0, fp8): lane (n, g) load i covers k = 64*i + 16*g .. +15; MFMA steps 2i, 2i+1 take its
+//                          low / high 8 bytes.  The token operand of lane (m, g) is x[m][64*i + 16*g .. +15].
+//   Q4_1 (1/2 byte):       lane (n, g) load i covers block 4*i + g (32 k); steps 4i .. 4i+3 take 4 bytes each.
+//                          Token operand: x[m][128*i + 32*g .. +31].
+//   16-bit dense:          as the 1-byte case with 32-byte loads.
+#include "ffn_kernels.h"
+
+namespace stmoe {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+template <typename T> __device__ __forceinline__ floatx4_t mfma16s(const u32x4_t& a, const u32x4_t& b, floatx4_t c);
+template <> __device__ __forceinline__ floatx4_t mfma16s<f16_t>(const u32x4_t& a, const u32x4_t& b, floatx4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ floatx4_t mfma16s<bf16_t>(const u32x4_t& a, const u32x4_t& b, floatx4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ u32x4_t ld_stream16(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+}
+__device__ __forceinline__ u32x2_t ld_stream8(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
+}
+__device__ __forceinline__ u32x4_t ld16(const void* p) { return *reinterpret_cast<const u32x4_t*>(p); }
+
+// fp16 pair -> T pair (identity for fp16; fp16 -> fp32 -> bf16 with round-to-nearest-even for bf16)
+template <typename T> __device__ __forceinline__ uint32_t h2_to_T(uint32_t h2) {
+  if constexpr (__is_same(T, f16_t)) return h2;
+  else return pack2<bf16_t>(f16_bits_to_f32(h2 & 0xffffu), f16_bits_to_f32(h2 >> 16));
+}
+
+// ---- per-format weight chunk: 256 reduction elements of one row, as seen by lane (n = lane%16, g = lane/16) ----
+template <int WF> struct SkinnyW;
+
+// Which 16 token elements lane group g needs for MFMA steps: returns element offset of the j-th 8-element
+// piece of step s inside the chunk.  Q4_1 differs from the others.
+template <int WF> __device__ __forceinline__ int x_offset(int s, int g) {
+  if constexpr (WF == WF_Q4_1) return 128 * (s >> 2) + 32 * g + 8 * (s & 3);
+  else return 64 * (s >> 1) + 16 * g + 8 * (s & 1);
+}
+
+template <> struct SkinnyW<WF_Q8_0> {
+  u32x4_t q[4];
+  u32x4_t d;  // the chunk's 8 block scales
+  __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
+    const uint8_t* base = w.qs + row * w.cols + c * 256 + 16 * g;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = ld_stream16(base + 64 * i);
+    d = ld_stream16(w.d + (row * (w.cols >> 5) + c * 8) * 2);
+  }
+  template <typename T> __device__ __forceinline__ u32x4_t frag(int s, int g) const {
+    const int i = s >> 1, h = s & 1;
+    const uint32_t dw = d[i];
+    const uint32_t dsel = (g & 2) ? (dw >> 16) : (dw & 0xffffu);
+    const half2_t dd = as_half2(dsel | (dsel << 16));
+    const half2_t bias = {(f16_t)1152.0f, (f16_t)1152.0f};
+    u32x4_t out;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t u = q[i][2 * h + j] ^ 0x80808080u;
+      const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
+      const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+      out[2 * j] = h2_to_T<T>(as_u32((as_half2(lo) - bias) * dd));
+      out[2 * j + 1] = h2_to_T<T>(as_u32((as_half2(hi) - bias) * dd));
+    }
+    return out;
+  }
+};
+
+template <> struct SkinnyW<WF_Q4_1> {
+  u32x4_t q[2];
+  u32x4_t d, m;  // 8 block scales / offsets of the chunk
+  __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
+    const uint8_t* base = w.qs + ((row * w.cols + c * 256) >> 1) + 16 * g;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) q[i] = ld_stream16(base + 64 * i);
+    const int64_t b = (row * (w.cols >> 5) + c * 8) * 2;
+    d = ld_stream16(w.d + b);
+    m = ld_stream16(w.m + b);
+  }
+  template <typename T> __device__ __forceinline__ u32x4_t frag(int s, int g) const {
+    const int i = s >> 2, j = s & 3;
+    // block 4*i + g of the chunk: dword (4i+g)/2 = 2i + (g>>1), half g&1
+    const uint32_t dw = (g & 2) ? d[2 * i + 1] : d[2 * i];
+    const uint32_t mw = (g & 2) ? m[2 * i + 1] : m[2 * i];
+    const uint32_t dsel = (g & 1) ? (dw >> 16) : (dw & 0xffffu);
+    const uint32_t msel = (g & 1) ? (mw >> 16) : (mw & 0xffffu);
+    const half2_t dd = as_half2(dsel | (dsel << 16)), mm = as_half2(msel | (msel << 16));
+    const half2_t bias = {(f16_t)1024.0f, (f16_t)1024.0f};
+    const uint32_t w4 = q[i][j];  // 8 nibbles: element 2b = low nibble of byte b, 2b+1 = high nibble
+    u32x4_t out;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const uint32_t byte = (w4 >> (8 * b));
+      const uint32_t pair = 0x64006400u | (byte & 0xfu) | ((byte & 0xf0u) << 12);
+      half2_t v = (as_half2(pair) - bias) * dd;
+      v = v + mm;
+      out[b] = h2_to_T<T>(as_u32(v));
+    }
+    return out;
+  }
+};
+
+template <> struct SkinnyW<WF_FP8_F32D> {
+  u32x4_t q[4];
+  float dv;
+  __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
+    const uint8_t* base = w.qs + row * w.cols + c * 256 + 16 * g;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = ld_stream16(base + 64 * i);
+    dv = reinterpret_cast<const float*>(w.d)[w.d_count > 1 ? row / w.rows : 0];
+  }
+  template <typename T> __device__ __forceinline__ u32x4_t frag(int s, int g) const {
+    const int i = s >> 1, h = s & 1;
+    u32x4_t out;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t u = q[i][2 * h + j];
+      float f[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) f[b] = __fmul_rn(fp8_e4m3fn_to_f32((uint8_t)(u >> (8 * b))), dv);
+      out[2 * j] = pack2<T>(f[0], f[1]);
+      out[2 * j + 1] = pack2<T>(f[2], f[3]);
+    }
+    return out;
+  }
+};
+
+template <bool BF> struct SkinnyWDense16 {
+  u32x4_t q[8];
+  __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
+    const uint8_t* base = w.qs + (row * w.cols + c * 256 + 16 * g) * 2;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      q[2 * i] = ld_stream16(base + 128 * i);
+      q[2 * i + 1] = ld_stream16(base + 128 * i + 16);
+    }
+  }
+  template <typename T> __device__ __forceinline__ u32x4_t frag(int s, int g) const { return q[s]; }
+};
+template <> struct SkinnyW<WF_DENSE_F16> : SkinnyWDense16<false> {};
+template <> struct SkinnyW<WF_DENSE_BF16> : SkinnyWDense16<true> {};
+
+// Token operand of one chunk for one 16-row M tile: 8 MFMA steps x 16 bytes.
+template <int WF> struct SkinnyX {
+  u32x4_t v[8];
+  __device__ __forceinline__ void load(const uint16_t* row_ptr, bool valid, int64_t c, int g) {
+    if (!valid) {
+#pragma unroll
+      for (int s = 0; s < 8; ++s) v[s] = (u32x4_t){0u, 0u, 0u, 0u};
+      return;
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) v[s] = ld16(row_ptr + c * 256 + x_offset<WF>(s, g));
+  }
+};
+
+template <typename T, int WF, int MODE, int MT>
+__global__ void __launch_bounds__(256, 2)
+grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
+  constexpr int NT = 2;
+  const int lane = threadIdx.x & 63;
+  const int g = lane >> 4, n_in = lane & 15;
+  const int wave_global = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t nch = p.kred >> 8;
+
+  // experts that received rows, in increasing id
+  int n_active = 0;
+  uint64_t active_mask = 0;
+  for (int e = 0; e < p.E; ++e)
+    if (p.offsets[e + 1] > p.offsets[e]) {
+      active_mask |= 1ull << e;
+      ++n_active;
+    }
+  const int n_items = n_active * tiles_per_expert;
+
+  for (int item = wave_global; item < n_items; item += total_waves) {
+    const int a_idx = item / tiles_per_expert, tile = item - a_idx * tiles_per_expert;
+    int e = 0;
+    {
+      int seen = 0;
+      for (int ee = 0; ee < p.E; ++ee)
+        if ((active_mask >> ee) & 1ull) {
+          if (seen == a_idx) { e = ee; break; }
+          ++seen;
+        }
+    }
+    const int rb = p.offsets[e], re = p.offsets[e + 1];
+
+    // the two weight tiles of this item
+    int64_t wrow[NT];
+    if (MODE == MODE_GATEUP) {
+      wrow[0] = (int64_t)e * p.w0.rows + tile * 16 + n_in;
+      wrow[1] = (int64_t)e * p.w1.rows + tile * 16 + n_in;
+    } else {
+      wrow[0] = (int64_t)e * p.w0.rows + tile * 32 + n_in;
+      wrow[1] = wrow[0] + 16;
+    }
+
+    for (int r0 = rb; r0 < re; r0 += 16 * MT) {  // one pass unless the expert has more than 16*MT rows
+      const uint16_t* xrow[MT];
+      bool xok[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int i = r0 + mt * 16 + n_in;
+        xok[mt] = i < re;
+        const int64_t src = xok[mt] ? (p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i) : 0;
+        xrow[mt] = reinterpret_cast<const uint16_t*>(p.a) + src * p.lda;
+      }
+      floatx4_t acc[MT][NT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[mt][t] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+
+      // MT == 1: weights and token rows of the next chunk are both in flight during a chunk's MFMAs.
+      // MT == 2: only the weights are double-buffered (the two token tiles of both buffers do not fit the
+      // 256-register budget of two wavefronts per SIMD); token rows come from L2 and are requested just
+      // before the next weight chunk so that weight requests stay in flight while they arrive.
+      constexpr bool XDB = MT == 1;
+      SkinnyW<WF> w0[NT], w1[NT];
+      SkinnyX<WF> x0[MT], x1[XDB ? MT : 1];
+      auto load_w = [&](SkinnyW<WF>* w, int64_t c) {
+        w[0].load(p.w0, wrow[0], c, g);
+        w[1].load(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1], c, g);
+      };
+      auto load_x = [&](SkinnyX<WF>* x, int64_t c) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) x[mt].load(xrow[mt], xok[mt], c, g);
+      };
+      auto compute = [&](const SkinnyW<WF>* w, const SkinnyX<WF>* x) {
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const u32x4_t wf = w[t].template frag<T>(s, g);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[mt][t] = mfma16s<T>(wf, x[mt].v[s], acc[mt][t]);
+          }
+        }
+      };
+
+      if constexpr (XDB) {
+        load_w(w0, 0);
+        load_x(x0, 0);
+        for (int64_t c = 0; c < nch; c += 2) {
+          if (c + 1 < nch) { load_w(w1, c + 1); load_x(x1, c + 1); }
+          compute(w0, x0);
+          if (c + 2 < nch) { load_w(w0, c + 2); load_x(x0, c + 2); }
+          if (c + 1 < nch) compute(w1, x1);
+        }
+      } else {
+        load_w(w0, 0);
+        for (int64_t c = 0; c < nch; c += 2) {
+          load_x(x0, c);
+          if (c + 1 < nch) load_w(w1, c + 1);
+          compute(w0, x0);
+          if (c + 1 < nch) {
+            load_x(x0, c + 1);
+            if (c + 2 < nch) load_w(w0, c + 2);
+            compute(w1, x0);
+          }
+        }
+      }
+
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int i = r0 + mt * 16 + n_in;
+        if (i < re) {
+          T* orow = reinterpret_cast<T*>(p.out) + (int64_t)i * p.ldo;
+          if (MODE == MODE_GATEUP) {
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] = gateup_epilogue<T>(p.act, acc[mt][0][r], acc[mt][1][r], 1.0f);
+            *reinterpret_cast<uint2*>(orow + tile * 16 + 4 * g) = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
+          } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              *reinterpret_cast<uint2*>(orow + tile * 32 + t * 16 + 4 * g) =
+                  make_uint2(pack2<T>(acc[mt][t][0], acc[mt][t][1]), pack2<T>(acc[mt][t][2], acc[mt][t][3]));
+          }
+        }
+      }
+    }
+  }
+}
+
+static int pick_waves(int64_t items) {
+  // 256 CUs x 2 workgroups x 4 wavefronts resident; give every wavefront the same number of items
+  const int64_t capacity = 2048;
+  if (items <= capacity) return (int)((items + 3) / 4 * 4);
+  const int64_t per_wave = (items + capacity - 1) / capacity;
+  const int64_t waves = (items + per_wave - 1) / per_wave;
+  return (int)((waves + 3) / 4 * 4);
+}
+
+template <typename T, int WF, int MT>
+static int launch_skinny_tw(int mode, const GemmParams& p, hipStream_t st) {
+  const int tiles = (int)(mode == MODE_GATEUP ? p.n_out / 16 : p.n_out / 32);
+  const int waves = pick_waves((int64_t)tiles * p.E);
+  dim3 grid((unsigned)(waves / 4));
+  if (mode == MODE_GATEUP) grouped_skinny_kernel<T, WF, MODE_GATEUP, MT><<<grid, 256, 0, st>>>(p, tiles, waves);
+  else grouped_skinny_kernel<T, WF, MODE_DOWN, MT><<<grid, 256, 0, st>>>(p, tiles, waves);
+  return check_launch("grouped_skinny");
+}
+
+template <typename T, int WF>
+static int launch_skinny_t(int mode, const GemmParams& p, int64_t max_rows_per_expert, hipStream_t st) {
+  if (max_rows_per_expert <= 16) return launch_skinny_tw<T, WF, 1>(mode, p, st);
+  return launch_skinny_tw<T, WF, 2>(mode, p, st);
+}
+
+int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
+  if (!p.offsets || p.E > 64)
+    return set_error(STMOE_ERR_UNSUPPORTED, "skinny kernel: needs per-expert offsets and at most 64 experts");
+  if (p.kred % 256 != 0 || p.n_out % 32 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0)
+    return set_error(STMOE_ERR_UNSUPPORTED, "skinny kernel: needs K %% 256 == 0 and N %% 32 == 0");
+  if (max_rows == 0) return STMOE_OK;
+  const int64_t per_expert = p.expert_rows_bound > 0 ? p.expert_rows_bound : max_rows;
+  if (act_dtype == STMOE_F16) {
+    switch (wtag) {
+      case WF_Q8_0: return launch_skinny_t<f16_t, WF_Q8_0>(mode, p, per_expert, st);
+      case WF_Q4_1: return launch_skinny_t<f16_t, WF_Q4_1>(mode, p, per_expert, st);
+      case WF_FP8_F32D: return launch_skinny_t<f16_t, WF_FP8_F32D>(mode, p, per_expert, st);
+      case WF_DENSE_F16: return launch_skinny_t<f16_t, WF_DENSE_F16>(mode, p, per_expert, st);
+      default: break;
+    }
+  } else if (act_dtype == STMOE_BF16) {
+    switch (wtag) {
+      case WF_Q8_0: return launch_skinny_t<bf16_t, WF_Q8_0>(mode, p, per_expert, st);
+      case WF_Q4_1: return launch_skinny_t<bf16_t, WF_Q4_1>(mode, p, per_expert, st);
+      case WF_FP8_F32D: return launch_skinny_t<bf16_t, WF_FP8_F32D>(mode, p, per_expert, st);
+      case WF_DENSE_BF16: return launch_skinny_t<bf16_t, WF_DENSE_BF16>(mode, p, per_expert, st);
+      default: break;
+    }
+  }
+  return set_error(STMOE_ERR_UNSUPPORTED, "skinny kernel: no instantiation for activation dtype %d with weight tag %d",
+                   act_dtype, wtag);
+}
+
+}  // namespace stmoe

@@ -23,7 +23,7 @@ ACT_SILU, ACT_GELU_ERF = 0, 1
 # enum stmoe_wfmt
 W_DENSE, W_Q8_0, W_Q4_1, W_FP8 = 0, 1, 2, 3
 # grouped_ffn variants
-VARIANT_AUTO, VARIANT_GENERIC, VARIANT_MFMA_TILE = 0, 1, 2
+VARIANT_AUTO, VARIANT_GENERIC, VARIANT_MFMA_TILE, VARIANT_SKINNY = 0, 1, 2, 3
 
 _DTYPE_ENUM = {
     torch.float32: F32,

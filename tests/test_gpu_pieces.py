@@ -208,3 +208,13 @@ def test_combine_with_output_norm_and_residual(device):
             assert torch.equal(got_plain, want_plain)  # products and the fp32 slot sum are exact: one rounding each
         assert O.rel_l2(got_plain, want_plain) < tol
         assert O.rel_l2(got_full, want_full) < tol
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8", "dense"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T", [1, 7, 16, 32, 45])
+def test_ffn_skinny_kernel(device, fmt, dtype, T):
+    """The decode kernel: 1, <16, =16, 17..32 and >32 rows per expert (the last takes two passes)."""
+    tol = 1e-3 if dtype == torch.float16 else 8e-3
+    act = "gelu" if T == 7 else "silu"
+    _ffn_parity(device, MC.Case(T=T, K=512, N=768, E=4 if T == 45 else 8, fmt=fmt, dtype=dtype, act=act, seed=40 + T), 3, tol)
