@@ -59,7 +59,12 @@ typedef enum {
   STMOE_W_DENSE = 0, /* DefaultPrimitiveTensor: qs = elements of `dtype` */
   STMOE_W_Q8_0 = 1,  /* BlockScaledLayout, block 32: d fp16 [.,K/32], qs int8 [.,K/32,32] */
   STMOE_W_Q4_1 = 2,  /* BlockScaledI4Layout, block 32, unsigned: d,m fp16 [.,K/32], qs u8 [.,K/32,16] */
-  STMOE_W_FP8 = 3    /* TensorScaledLayout: qs e4m3fn [.,K], d = d_count scales of `dtype` (f32 or f16) */
+  STMOE_W_FP8 = 3,   /* TensorScaledLayout: qs e4m3fn [.,K], d = d_count scales of `dtype` (f32 or f16) */
+  /* The same bytes re-ordered by stmoe_prepack() into the order the matrix-core kernels stream (every wavefront
+   * load is one contiguous kilobyte; see stmoe_prepack).  Plane sizes are unchanged. */
+  STMOE_W_Q8_0_PACKED = 4,
+  STMOE_W_Q4_1_PACKED = 5,
+  STMOE_W_FP8_PACKED = 6
 } stmoe_wfmt;
 
 /* One stacked expert weight `[experts, rows, cols]`, used as x @ W[e]^T. */
@@ -107,6 +112,16 @@ int stmoe_dequant_tensor_scaled(const void* qs, int qs_dtype, const void* d, con
  * computed in fp32 and rounded to x's dtype before the clamp.  `rscale` points to one device float. */
 int stmoe_quantize_fp8(const void* x, int x_dtype, const float* rscale, int64_t n, void* out_fp8,
                        stmoe_stream_t stream);
+
+/* Load-time re-ordering of a planar quantized weight into the streaming order (and back).  For every tile of 16
+ * consecutive rows: samples as [K/64][lane = 16*g + n][16 B] (Q8_0, fp8: row n, k = 64*kb + 16*g..+15) or
+ * [K/128][lane][16 B] (Q4_1: row n, block 4*kb + g); block scales/offsets as [K/256][16 rows][8] fp16.  A pure
+ * permutation of bytes: stmoe_unpack(stmoe_prepack(w)) == w bit for bit.  `planar` and `packed` describe the same
+ * [experts, rows, cols] with formats X and X_PACKED and caller-owned planes of equal sizes; rows % 16 == 0 and
+ * cols % 256 == 0.  The reference has no counterpart (its planes come from GGUF blocks,
+ * sharktank/sharktank/types/gguf_interop/layouts.py:51-60,285-300, and are consumed row-major). */
+int stmoe_prepack(const stmoe_weight* planar, const stmoe_weight* packed_out, stmoe_stream_t stream);
+int stmoe_unpack(const stmoe_weight* packed, const stmoe_weight* planar_out, stmoe_stream_t stream);
 
 /* ---- layer pieces ----------------------------------------------------------------------------- */
 

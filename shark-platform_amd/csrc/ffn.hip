@@ -12,17 +12,22 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
                 "%s: weight is [%lld,%lld,%lld], expected [%lld,%lld,%lld]", who, (long long)w->experts,
                 (long long)w->rows, (long long)w->cols, (long long)E, (long long)rows, (long long)cols);
   STMOE_REQUIRE(aligned16(w->qs), STMOE_ERR_ALIGN, "%s: qs plane must be 16-byte aligned", who);
+  if (w->format >= STMOE_W_Q8_0_PACKED && w->format <= STMOE_W_FP8_PACKED)
+    STMOE_REQUIRE(rows % 16 == 0 && cols % 256 == 0, STMOE_ERR_SHAPE, "%s: packed formats need rows %% 16 == 0 and cols %% 256 == 0", who);
   switch (w->format) {
     case STMOE_W_Q8_0:
+    case STMOE_W_Q8_0_PACKED:
       STMOE_REQUIRE(w->d, STMOE_ERR_NULL, "%s: Q8_0 needs d", who);
       STMOE_REQUIRE(w->m == nullptr, STMOE_ERR_UNSUPPORTED, "%s: Q8 block scaled with offset is not implemented", who);
       STMOE_REQUIRE(cols % 32 == 0, STMOE_ERR_SHAPE, "%s: Q8_0 needs cols %% 32 == 0", who);
       break;
     case STMOE_W_Q4_1:
+    case STMOE_W_Q4_1_PACKED:
       STMOE_REQUIRE(w->d && w->m, STMOE_ERR_NULL, "%s: Q4_1 needs d and m", who);
       STMOE_REQUIRE(cols % 32 == 0, STMOE_ERR_SHAPE, "%s: Q4_1 needs cols %% 32 == 0", who);
       break;
     case STMOE_W_FP8:
+    case STMOE_W_FP8_PACKED:
       STMOE_REQUIRE(w->d, STMOE_ERR_NULL, "%s: FP8 needs d", who);
       STMOE_REQUIRE(w->d_count == 1 || w->d_count == E, STMOE_ERR_SHAPE, "%s: FP8 d_count must be 1 or experts", who);
       STMOE_REQUIRE(cols % 16 == 0, STMOE_ERR_SHAPE, "%s: FP8 needs cols %% 16 == 0", who);

@@ -99,6 +99,9 @@ static int launch_generic_t(int wtag, int mode, const GemmParams& p, int64_t max
     case WF_DENSE_F32: return launch_generic_tw<T, WF_DENSE_F32>(mode, p, max_rows, st);
     case WF_DENSE_F16: return launch_generic_tw<T, WF_DENSE_F16>(mode, p, max_rows, st);
     case WF_DENSE_BF16: return launch_generic_tw<T, WF_DENSE_BF16>(mode, p, max_rows, st);
+    case WF_Q8_0_P: return launch_generic_tw<T, WF_Q8_0_P>(mode, p, max_rows, st);
+    case WF_Q4_1_P: return launch_generic_tw<T, WF_Q4_1_P>(mode, p, max_rows, st);
+    case WF_FP8_F32D_P: return launch_generic_tw<T, WF_FP8_F32D_P>(mode, p, max_rows, st);
     default: return set_error(STMOE_ERR_UNSUPPORTED, "generic kernel: unknown weight tag %d", wtag);
   }
 }

@@ -176,6 +176,9 @@ int launch_mfma_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int
       case WF_Q4_1: return launch_tw<f16_t, WF_Q4_1>(mode, p, max_rows, st);
       case WF_FP8_F32D: return launch_tw<f16_t, WF_FP8_F32D>(mode, p, max_rows, st);
       case WF_DENSE_F16: return launch_tw<f16_t, WF_DENSE_F16>(mode, p, max_rows, st);
+      case WF_Q8_0_P: return launch_tw<f16_t, WF_Q8_0_P>(mode, p, max_rows, st);
+      case WF_Q4_1_P: return launch_tw<f16_t, WF_Q4_1_P>(mode, p, max_rows, st);
+      case WF_FP8_F32D_P: return launch_tw<f16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
       default: break;
     }
   } else if (act_dtype == STMOE_BF16) {
@@ -184,6 +187,9 @@ int launch_mfma_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int
       case WF_Q4_1: return launch_tw<bf16_t, WF_Q4_1>(mode, p, max_rows, st);
       case WF_FP8_F32D: return launch_tw<bf16_t, WF_FP8_F32D>(mode, p, max_rows, st);
       case WF_DENSE_BF16: return launch_tw<bf16_t, WF_DENSE_BF16>(mode, p, max_rows, st);
+      case WF_Q8_0_P: return launch_tw<bf16_t, WF_Q8_0_P>(mode, p, max_rows, st);
+      case WF_Q4_1_P: return launch_tw<bf16_t, WF_Q4_1_P>(mode, p, max_rows, st);
+      case WF_FP8_F32D_P: return launch_tw<bf16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
       default: break;
     }
   }

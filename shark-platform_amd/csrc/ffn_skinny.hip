@@ -54,7 +54,7 @@ template <int WF> struct SkinnyW;
 // Which 16 token elements lane group g needs for MFMA steps: returns element offset of the j-th 8-element
 // piece of step s inside the chunk.  Q4_1 differs from the others.
 template <int WF> __device__ __forceinline__ int x_offset(int s, int g) {
-  if constexpr (WF == WF_Q4_1) return 128 * (s >> 2) + 32 * g + 8 * (s & 3);
+  if constexpr (IsQ4<WF>::value) return 128 * (s >> 2) + 32 * g + 8 * (s & 3);
   else return 64 * (s >> 1) + 16 * g + 8 * (s & 1);
 }
 
@@ -142,6 +142,39 @@ template <> struct SkinnyW<WF_FP8_F32D> {
       out[2 * j + 1] = pack2<T>(f[2], f[3]);
     }
     return out;
+  }
+};
+
+// Packed streaming order: the 16 lanes x 4 groups of one load instruction read one contiguous kilobyte.
+template <> struct SkinnyW<WF_Q8_0_P> : SkinnyW<WF_Q8_0> {
+  __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
+    const int64_t rt = row >> 4;
+    const int r = (int)(row & 15);
+    const uint8_t* base = w.qs + (rt * (w.cols >> 6) + c * 4) * 1024 + (g * 16 + r) * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = ld_stream16(base + 1024 * i);
+    d = ld_stream16(w.d + (rt * (w.cols >> 8) + c) * 256 + r * 16);
+  }
+};
+template <> struct SkinnyW<WF_Q4_1_P> : SkinnyW<WF_Q4_1> {
+  __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
+    const int64_t rt = row >> 4;
+    const int r = (int)(row & 15);
+    const uint8_t* base = w.qs + (rt * (w.cols >> 7) + c * 2) * 1024 + (g * 16 + r) * 16;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) q[i] = ld_stream16(base + 1024 * i);
+    const int64_t b = (rt * (w.cols >> 8) + c) * 256 + r * 16;
+    d = ld_stream16(w.d + b);
+    m = ld_stream16(w.m + b);
+  }
+};
+template <> struct SkinnyW<WF_FP8_F32D_P> : SkinnyW<WF_FP8_F32D> {
+  __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
+    const int64_t rt = row >> 4;
+    const uint8_t* base = w.qs + (rt * (w.cols >> 6) + c * 4) * 1024 + (g * 16 + (int)(row & 15)) * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = ld_stream16(base + 1024 * i);
+    dv = reinterpret_cast<const float*>(w.d)[w.d_count > 1 ? row / w.rows : 0];
   }
 };
 
@@ -342,6 +375,9 @@ int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_
       case WF_Q4_1: return launch_skinny_t<f16_t, WF_Q4_1>(mode, p, per_expert, st);
       case WF_FP8_F32D: return launch_skinny_t<f16_t, WF_FP8_F32D>(mode, p, per_expert, st);
       case WF_DENSE_F16: return launch_skinny_t<f16_t, WF_DENSE_F16>(mode, p, per_expert, st);
+      case WF_Q8_0_P: return launch_skinny_t<f16_t, WF_Q8_0_P>(mode, p, per_expert, st);
+      case WF_Q4_1_P: return launch_skinny_t<f16_t, WF_Q4_1_P>(mode, p, per_expert, st);
+      case WF_FP8_F32D_P: return launch_skinny_t<f16_t, WF_FP8_F32D_P>(mode, p, per_expert, st);
       default: break;
     }
   } else if (act_dtype == STMOE_BF16) {
@@ -350,6 +386,9 @@ int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_
       case WF_Q4_1: return launch_skinny_t<bf16_t, WF_Q4_1>(mode, p, per_expert, st);
       case WF_FP8_F32D: return launch_skinny_t<bf16_t, WF_FP8_F32D>(mode, p, per_expert, st);
       case WF_DENSE_BF16: return launch_skinny_t<bf16_t, WF_DENSE_BF16>(mode, p, per_expert, st);
+      case WF_Q8_0_P: return launch_skinny_t<bf16_t, WF_Q8_0_P>(mode, p, per_expert, st);
+      case WF_Q4_1_P: return launch_skinny_t<bf16_t, WF_Q4_1_P>(mode, p, per_expert, st);
+      case WF_FP8_F32D_P: return launch_skinny_t<bf16_t, WF_FP8_F32D_P>(mode, p, per_expert, st);
       default: break;
     }
   }

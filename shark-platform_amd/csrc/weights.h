@@ -35,7 +35,12 @@ static inline WeightView make_view(const stmoe_weight* w) {
 }
 
 // Formats as compile-time tags.  Dense weights are split by element type.
-enum : int { WF_Q8_0 = 0, WF_Q4_1 = 1, WF_FP8_F32D = 2, WF_FP8_F16D = 3, WF_DENSE_F32 = 4, WF_DENSE_F16 = 5, WF_DENSE_BF16 = 6 };
+enum : int { WF_Q8_0 = 0, WF_Q4_1 = 1, WF_FP8_F32D = 2, WF_FP8_F16D = 3, WF_DENSE_F32 = 4, WF_DENSE_F16 = 5, WF_DENSE_BF16 = 6,
+             // the same formats in the packed streaming order written by stmoe_prepack
+             WF_Q8_0_P = 7, WF_Q4_1_P = 8, WF_FP8_F32D_P = 9 };
+
+template <int WF> struct IsQ8 { static constexpr bool value = WF == WF_Q8_0 || WF == WF_Q8_0_P; };
+template <int WF> struct IsQ4 { static constexpr bool value = WF == WF_Q4_1 || WF == WF_Q4_1_P; };
 
 // pack two fp32 values, already rounded to T, into one dword of T bits
 template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
@@ -175,6 +180,41 @@ template <bool F16D> struct Chunk16Fp8 {
 template <> struct Chunk16<WF_FP8_F32D> : Chunk16Fp8<false> {};
 template <> struct Chunk16<WF_FP8_F16D> : Chunk16Fp8<true> {};
 
+// Packed streaming order (see prepack.hip): only the addresses differ from the planar accessors.
+__device__ __forceinline__ int64_t packed_piece(int64_t row, int64_t k0, int64_t cols, int kshift) {
+  // byte offset of the 16-byte piece holding (row, k0) when one piece covers 1 << (kshift - 2) reduction elements
+  // of one row and one 1 KB block covers 1 << kshift of them: kshift = 6 for 1-byte samples, 7 for nibbles
+  const int64_t rt = row >> 4, kb = k0 >> kshift;
+  const int g = (int)(k0 >> (kshift - 2)) & 3;
+  return ((rt * (cols >> kshift) + kb) * 64 + g * 16 + (row & 15)) << 4;
+}
+__device__ __forceinline__ int64_t packed_scale(int64_t row, int64_t k0, int64_t cols) {
+  return (((row >> 4) * (cols >> 8) + (k0 >> 8)) * 16 + (row & 15)) * 8 + ((k0 >> 5) & 7);
+}
+template <> struct Chunk16<WF_Q8_0_P> : Chunk16<WF_Q8_0> {
+  __device__ __forceinline__ void load(const WeightView& w, int64_t e, int64_t n, int64_t k0) {
+    const int64_t row = e * w.rows + n;
+    q = *reinterpret_cast<const uint4*>(w.qs + packed_piece(row, k0, w.cols, 6));
+    dbits = reinterpret_cast<const uint16_t*>(w.d)[packed_scale(row, k0, w.cols)];
+  }
+};
+template <> struct Chunk16<WF_Q4_1_P> : Chunk16<WF_Q4_1> {
+  __device__ __forceinline__ void load(const WeightView& w, int64_t e, int64_t n, int64_t k0) {
+    const int64_t row = e * w.rows + n;
+    q = *reinterpret_cast<const uint2*>(w.qs + packed_piece(row, k0, w.cols, 7) + ((k0 >> 4) & 1) * 8);
+    const int64_t b = packed_scale(row, k0, w.cols);
+    dbits = reinterpret_cast<const uint16_t*>(w.d)[b];
+    mbits = reinterpret_cast<const uint16_t*>(w.m)[b];
+  }
+};
+template <> struct Chunk16<WF_FP8_F32D_P> : Chunk16Fp8<false> {
+  __device__ __forceinline__ void load(const WeightView& w, int64_t e, int64_t n, int64_t k0) {
+    const int64_t row = e * w.rows + n;
+    q = *reinterpret_cast<const uint4*>(w.qs + packed_piece(row, k0, w.cols, 6));
+    dv = reinterpret_cast<const float*>(w.d)[w.d_count > 1 ? e : 0];
+  }
+};
+
 template <> struct Chunk16<WF_DENSE_F32> {
   float4 v[4];
   __device__ __forceinline__ void load(const WeightView& w, int64_t e, int64_t n, int64_t k0) {
@@ -229,7 +269,7 @@ template <> struct Chunk16<WF_DENSE_BF16> : Chunk16Dense16<true> {};
 // 16 values of T as 8 dwords, ready for LDS / MFMA operands.
 template <typename T, int WF>
 __device__ __forceinline__ void chunk_to_T(const Chunk16<WF>& c, uint32_t out[8]) {
-  if constexpr (WF == WF_Q8_0 || WF == WF_Q4_1) {
+  if constexpr (IsQ8<WF>::value || IsQ4<WF>::value) {
     if constexpr (__is_same(T, f16_t)) {
       c.to_f16x16(out);
       return;
@@ -251,6 +291,9 @@ static inline int weight_tag(const stmoe_weight* w) {
     case STMOE_W_Q8_0: return WF_Q8_0;
     case STMOE_W_Q4_1: return WF_Q4_1;
     case STMOE_W_FP8: return w->dtype == STMOE_F32 ? WF_FP8_F32D : (w->dtype == STMOE_F16 ? WF_FP8_F16D : -1);
+    case STMOE_W_Q8_0_PACKED: return WF_Q8_0_P;
+    case STMOE_W_Q4_1_PACKED: return WF_Q4_1_P;
+    case STMOE_W_FP8_PACKED: return w->dtype == STMOE_F32 ? WF_FP8_F32D_P : -1;
     case STMOE_W_DENSE:
       return w->dtype == STMOE_F32 ? WF_DENSE_F32 : (w->dtype == STMOE_F16 ? WF_DENSE_F16 : (w->dtype == STMOE_BF16 ? WF_DENSE_BF16 : -1));
     default: return -1;

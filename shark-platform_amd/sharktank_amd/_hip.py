@@ -22,6 +22,8 @@ F32, F16, BF16, F8E4M3FN, I8, U8 = 0, 1, 2, 3, 4, 5
 ACT_SILU, ACT_GELU_ERF = 0, 1
 # enum stmoe_wfmt
 W_DENSE, W_Q8_0, W_Q4_1, W_FP8 = 0, 1, 2, 3
+W_Q8_0_PACKED, W_Q4_1_PACKED, W_FP8_PACKED = 4, 5, 6
+_PACKED_OF = {W_Q8_0: W_Q8_0_PACKED, W_Q4_1: W_Q4_1_PACKED, W_FP8: W_FP8_PACKED}
 # grouped_ffn variants
 VARIANT_AUTO, VARIANT_GENERIC, VARIANT_MFMA_TILE, VARIANT_SKINNY = 0, 1, 2, 3
 
@@ -68,6 +70,8 @@ SIGNATURES = {
     "stmoe_dequant_block_scaled_i4": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p, c_int, c_void_p]),
     "stmoe_promote_i4": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
     "stmoe_dequant_tensor_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p]),
+    "stmoe_prepack": (c_int, [POINTER(StmoeWeight), POINTER(StmoeWeight), c_void_p]),
+    "stmoe_unpack": (c_int, [POINTER(StmoeWeight), POINTER(StmoeWeight), c_void_p]),
     "stmoe_quantize_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
     "stmoe_rms_norm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_float, c_void_p, c_void_p]),
     "stmoe_router_topk": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -302,7 +306,7 @@ class DeviceWeight:
         self.device = _dev(qs, d, m)
         self.desc = StmoeWeight(
             format=fmt, dtype=dtype_tag, experts=experts, rows=rows, cols=cols,
-            qs=_ptr(qs), d=_ptr(d), m=_ptr(m), d_count=(d.numel() if (d is not None and fmt == W_FP8) else 1),
+            qs=_ptr(qs), d=_ptr(d), m=_ptr(m), d_count=(d.numel() if (d is not None and fmt in (W_FP8, W_FP8_PACKED)) else 1),
         )
         self.format = fmt
         self.experts, self.rows, self.cols = experts, rows, cols
@@ -313,6 +317,39 @@ class DeviceWeight:
 
     def nbytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.keep if t is not None)
+
+    @property
+    def is_packed(self) -> bool:
+        return self.format in (W_Q8_0_PACKED, W_Q4_1_PACKED, W_FP8_PACKED)
+
+    def can_prepack(self) -> bool:
+        return (self.format in _PACKED_OF and self.rows % 16 == 0 and self.cols % 256 == 0
+                and (self.format != W_FP8 or self.desc.dtype == F32))
+
+    def prepack(self) -> "DeviceWeight":
+        """The same weight in the streaming order of stmoe_prepack (new planes; this object is unchanged)."""
+        qs, d, m = self.keep
+        lib = load_library()
+        new_qs = torch.empty_like(qs)
+        fp8 = self.format == W_FP8
+        new_d = d if fp8 else torch.empty_like(d)
+        new_m = None if m is None else torch.empty_like(m)
+        out = DeviceWeight(_PACKED_OF[self.format], self.experts, self.rows, self.cols, new_qs, new_d, new_m, self.desc.dtype)
+        with torch.cuda.device(self.device):
+            _check(lib.stmoe_prepack(self.ref, out.ref, _stream(self.device)))
+        return out
+
+    def unpack(self) -> "DeviceWeight":
+        """Inverse of prepack()."""
+        qs, d, m = self.keep
+        lib = load_library()
+        planar_fmt = {v: k for k, v in _PACKED_OF.items()}[self.format]
+        fp8 = planar_fmt == W_FP8
+        out = DeviceWeight(planar_fmt, self.experts, self.rows, self.cols, torch.empty_like(qs), d if fp8 else torch.empty_like(d),
+                           None if m is None else torch.empty_like(m), self.desc.dtype)
+        with torch.cuda.device(self.device):
+            _check(lib.stmoe_unpack(self.ref, out.ref, _stream(self.device)))
+        return out
 
 
 def grouped_ffn_workspace_bytes(T: int, k: int, K: int, N: int, dtype: torch.dtype) -> int:

@@ -39,14 +39,17 @@ class PreGatherFFNMOE(ThetaLayer):
         self._act = activation_enum(activation)
         self._dw = None
         self.kernel_variant = _hip.VARIANT_AUTO
+        # Re-order the quantized planes once into the kernels' streaming order (a second copy of the weights in
+        # HBM; the planar tensors stay owned by `theta` and can be released by the caller).
+        self.prepack_weights = True
 
     def device_weights(self):
         """C-ABI descriptors of the three stacked weights, built once (planes made contiguous once)."""
         if self._dw is None:
             self._dw = (
-                device_weight(self.ffn_gate, stacked=True),
-                device_weight(self.ffn_up, stacked=True),
-                device_weight(self.ffn_down, stacked=True),
+                device_weight(self.ffn_gate, stacked=True, prepack=self.prepack_weights),
+                device_weight(self.ffn_up, stacked=True, prepack=self.prepack_weights),
+                device_weight(self.ffn_down, stacked=True, prepack=self.prepack_weights),
             )
         return self._dw
 

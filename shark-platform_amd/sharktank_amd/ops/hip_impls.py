@@ -21,9 +21,17 @@ __all__ = ["device_weight"]
 _FLOAT_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
 
 
-def device_weight(w, *, stacked: bool) -> _hip.DeviceWeight:
+def device_weight(w, *, stacked: bool, prepack: bool = False) -> _hip.DeviceWeight:
     """C-ABI descriptor of a weight tensor.  `stacked`: [E, rows, cols]; otherwise a single [rows, cols] matrix.
-    Planes are made contiguous once here (GGUF-derived planes are strided views of the raw blocks)."""
+    Planes are made contiguous once here (GGUF-derived planes are strided views of the raw blocks).  With
+    `prepack`, quantized planes whose shape allows it are re-ordered once into the kernels' streaming order."""
+    dw = _device_weight_planar(w, stacked=stacked)
+    if prepack and dw.can_prepack():
+        dw = dw.prepack()
+    return dw
+
+
+def _device_weight_planar(w, *, stacked: bool) -> _hip.DeviceWeight:
     shape = list(w.shape)
     if stacked:
         assert len(shape) == 3, f"expert-stacked weight must be [E, rows, cols], got {shape}"

@@ -218,3 +218,66 @@ def test_ffn_skinny_kernel(device, fmt, dtype, T):
     tol = 1e-3 if dtype == torch.float16 else 8e-3
     act = "gelu" if T == 7 else "silu"
     _ffn_parity(device, MC.Case(T=T, K=512, N=768, E=4 if T == 45 else 8, fmt=fmt, dtype=dtype, act=act, seed=40 + T), 3, tol)
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8"])
+def test_prepack_round_trip_bit_exact(device, fmt):
+    from sharktank_amd.ops import device_weight
+
+    case = MC.build(MC.Case(T=4, K=512, N=256, E=3, fmt=fmt, seed=50))
+    it = MC.to_inference_tensor(fmt, case.planes["gate"], [3, 256, 512], "w", device)
+    planar = device_weight(it, stacked=True)
+    packed = planar.prepack()
+    assert packed.is_packed and packed.nbytes() == planar.nbytes()
+    back = packed.unpack()
+    for a, b in zip(planar.keep, back.keep):
+        if a is not None:
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    if fmt != "fp8":
+        assert not torch.equal(planar.keep[0].view(torch.uint8), packed.keep[0].view(torch.uint8))
+
+
+def test_prepack_layout_definition(device):
+    """Spot-checks the documented order: lane 16*g + n of block (row tile rt, k block kb) holds row 16*rt+n,
+    k = 64*kb + 16*g .. +15; scales of 8 consecutive blocks of a row are contiguous."""
+    from sharktank_amd.ops import device_weight
+    from sharktank_amd import types as ST
+
+    E, N, K = 2, 32, 512
+    qs = torch.arange(E * N * K, dtype=torch.int32).remainder(251).to(torch.int8).reshape(E, N, K // 32, 32)
+    d = torch.arange(E * N * K // 32, dtype=torch.float32).reshape(E, N, K // 32, 1).to(torch.float16)
+    it = ST.PlanarQuantizedTensor(shape=[E, N, K], layout=ST.BlockScaledLayout([E, N, K], d.to(device), qs.to(device)))
+    packed = device_weight(it, stacked=True, prepack=True)
+    pq = packed.keep[0].cpu().reshape(-1)
+    pd = packed.keep[1].cpu().reshape(-1)
+    flat = qs.reshape(E * N, K)
+    dflat = d.reshape(E * N, K // 32)
+    for rt, kb, g, n in [(0, 0, 0, 0), (1, 3, 2, 5), (3, 7, 3, 15), (2, 4, 1, 9)]:
+        off = ((rt * (K // 64) + kb) * 64 + g * 16 + n) * 16
+        assert torch.equal(pq[off : off + 16], flat[rt * 16 + n, kb * 64 + g * 16 : kb * 64 + g * 16 + 16])
+    for rt, c, n in [(0, 0, 0), (3, 1, 7), (1, 1, 15)]:
+        off = ((rt * (K // 256) + c) * 16 + n) * 8
+        assert torch.equal(pd[off : off + 8], dflat[rt * 16 + n, c * 8 : c * 8 + 8])
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("variant,T", [(1, 9), (2, 150), (3, 20)])
+def test_packed_weights_match_planar(device, fmt, dtype, variant, T):
+    """Every kernel family gives the same bits from packed planes as from planar planes."""
+    hip = _hip()
+    from sharktank_amd.ops import device_weight
+
+    case = MC.build(MC.Case(T=T, K=512, N=256, fmt=fmt, dtype=dtype, seed=51))
+    E, N, K = case.E, case.N, case.K
+    g = torch.Generator().manual_seed(3)
+    idx = torch.stack([torch.randperm(E, generator=g)[: case.k] for _ in range(T)]).to(torch.int32)
+    _, offsets, perm, inv = hip.dispatch_build(idx.to(device), E)
+    outs = []
+    for prepack in (False, True):
+        dws = [device_weight(MC.to_inference_tensor(fmt, case.planes[n], shp, n, device), stacked=True, prepack=prepack)
+               for n, shp in (("gate", [E, N, K]), ("up", [E, N, K]), ("down", [E, K, N]))]
+        assert dws[0].is_packed == prepack
+        outs.append(hip.grouped_ffn(case.planes["h"].to(device), dws[0], dws[1], dws[2], hip.ACT_SILU, offsets, perm, case.k,
+                                    variant=variant).cpu())
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
