@@ -207,12 +207,102 @@ template <int WF> struct SkinnyX {
   }
 };
 
+// One pass of one work item: rows [r0, min(r0 + 16*MT, re)) of expert rows against the item's two weight tiles.
 template <typename T, int WF, int MODE, int MT>
+__device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (&wrow)[2], int tile, int r0, int re,
+                                            int64_t nch, int lane) {
+  constexpr int NT = 2;
+  const int g = lane >> 4, n_in = lane & 15;
+  const uint16_t* xrow[MT];
+  bool xok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int i = r0 + mt * 16 + n_in;
+    xok[mt] = i < re;
+    const int64_t src = xok[mt] ? (p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i) : 0;
+    xrow[mt] = reinterpret_cast<const uint16_t*>(p.a) + src * p.lda;
+  }
+  floatx4_t acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[mt][t] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+
+  // MT == 1: weights and token rows of the next chunk are both in flight during a chunk's MFMAs.
+  // MT == 2: only the weights are double-buffered (the two token tiles of both buffers do not fit the
+  // 256-register budget of two wavefronts per SIMD); token rows come from L2 and are requested just
+  // before the next weight chunk so that weight requests stay in flight while they arrive.
+  constexpr bool XDB = MT == 1;
+  SkinnyW<WF> w0[NT], w1[NT];
+  SkinnyX<WF> x0[MT], x1[XDB ? MT : 1];
+  auto load_w = [&](SkinnyW<WF>* w, int64_t c) {
+    w[0].load(p.w0, wrow[0], c, g);
+    w[1].load(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1], c, g);
+  };
+  auto load_x = [&](SkinnyX<WF>* x, int64_t c) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) x[mt].load(xrow[mt], xok[mt], c, g);
+  };
+  auto compute = [&](const SkinnyW<WF>* w, const SkinnyX<WF>* x) {
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const u32x4_t wf = w[t].template frag<T>(s, g);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[mt][t] = mfma16s<T>(wf, x[mt].v[s], acc[mt][t]);
+      }
+    }
+  };
+
+  if constexpr (XDB) {
+    load_w(w0, 0);
+    load_x(x0, 0);
+    for (int64_t c = 0; c < nch; c += 2) {
+      if (c + 1 < nch) { load_w(w1, c + 1); load_x(x1, c + 1); }
+      compute(w0, x0);
+      if (c + 2 < nch) { load_w(w0, c + 2); load_x(x0, c + 2); }
+      if (c + 1 < nch) compute(w1, x1);
+    }
+  } else {
+    load_w(w0, 0);
+    for (int64_t c = 0; c < nch; c += 2) {
+      load_x(x0, c);
+      if (c + 1 < nch) load_w(w1, c + 1);
+      compute(w0, x0);
+      if (c + 1 < nch) {
+        load_x(x0, c + 1);
+        if (c + 2 < nch) load_w(w0, c + 2);
+        compute(w1, x0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int i = r0 + mt * 16 + n_in;
+    if (i < re) {
+      T* orow = reinterpret_cast<T*>(p.out) + (int64_t)i * p.ldo;
+      if (MODE == MODE_GATEUP) {
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = gateup_epilogue<T>(p.act, acc[mt][0][r], acc[mt][1][r], 1.0f);
+        *reinterpret_cast<uint2*>(orow + tile * 16 + 4 * g) = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
+      } else {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          *reinterpret_cast<uint2*>(orow + tile * 32 + t * 16 + 4 * g) =
+              make_uint2(pack2<T>(acc[mt][t][0], acc[mt][t][1]), pack2<T>(acc[mt][t][2], acc[mt][t][3]));
+      }
+    }
+  }
+}
+
+template <typename T, int WF, int MODE>
 __global__ void __launch_bounds__(256, 2)
 grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
-  constexpr int NT = 2;
   const int lane = threadIdx.x & 63;
-  const int g = lane >> 4, n_in = lane & 15;
+  const int n_in = lane & 15;
   const int wave_global = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int64_t nch = p.kred >> 8;
 
@@ -240,7 +330,7 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
     const int rb = p.offsets[e], re = p.offsets[e + 1];
 
     // the two weight tiles of this item
-    int64_t wrow[NT];
+    int64_t wrow[2];
     if (MODE == MODE_GATEUP) {
       wrow[0] = (int64_t)e * p.w0.rows + tile * 16 + n_in;
       wrow[1] = (int64_t)e * p.w1.rows + tile * 16 + n_in;
@@ -248,91 +338,11 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
       wrow[0] = (int64_t)e * p.w0.rows + tile * 32 + n_in;
       wrow[1] = wrow[0] + 16;
     }
-
-    for (int r0 = rb; r0 < re; r0 += 16 * MT) {  // one pass unless the expert has more than 16*MT rows
-      const uint16_t* xrow[MT];
-      bool xok[MT];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int i = r0 + mt * 16 + n_in;
-        xok[mt] = i < re;
-        const int64_t src = xok[mt] ? (p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i) : 0;
-        xrow[mt] = reinterpret_cast<const uint16_t*>(p.a) + src * p.lda;
-      }
-      floatx4_t acc[MT][NT];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[mt][t] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
-
-      // MT == 1: weights and token rows of the next chunk are both in flight during a chunk's MFMAs.
-      // MT == 2: only the weights are double-buffered (the two token tiles of both buffers do not fit the
-      // 256-register budget of two wavefronts per SIMD); token rows come from L2 and are requested just
-      // before the next weight chunk so that weight requests stay in flight while they arrive.
-      constexpr bool XDB = MT == 1;
-      SkinnyW<WF> w0[NT], w1[NT];
-      SkinnyX<WF> x0[MT], x1[XDB ? MT : 1];
-      auto load_w = [&](SkinnyW<WF>* w, int64_t c) {
-        w[0].load(p.w0, wrow[0], c, g);
-        w[1].load(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1], c, g);
-      };
-      auto load_x = [&](SkinnyX<WF>* x, int64_t c) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) x[mt].load(xrow[mt], xok[mt], c, g);
-      };
-      auto compute = [&](const SkinnyW<WF>* w, const SkinnyX<WF>* x) {
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-#pragma unroll
-          for (int t = 0; t < NT; ++t) {
-            const u32x4_t wf = w[t].template frag<T>(s, g);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[mt][t] = mfma16s<T>(wf, x[mt].v[s], acc[mt][t]);
-          }
-        }
-      };
-
-      if constexpr (XDB) {
-        load_w(w0, 0);
-        load_x(x0, 0);
-        for (int64_t c = 0; c < nch; c += 2) {
-          if (c + 1 < nch) { load_w(w1, c + 1); load_x(x1, c + 1); }
-          compute(w0, x0);
-          if (c + 2 < nch) { load_w(w0, c + 2); load_x(x0, c + 2); }
-          if (c + 1 < nch) compute(w1, x1);
-        }
-      } else {
-        load_w(w0, 0);
-        for (int64_t c = 0; c < nch; c += 2) {
-          load_x(x0, c);
-          if (c + 1 < nch) load_w(w1, c + 1);
-          compute(w0, x0);
-          if (c + 1 < nch) {
-            load_x(x0, c + 1);
-            if (c + 2 < nch) load_w(w0, c + 2);
-            compute(w1, x0);
-          }
-        }
-      }
-
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int i = r0 + mt * 16 + n_in;
-        if (i < re) {
-          T* orow = reinterpret_cast<T*>(p.out) + (int64_t)i * p.ldo;
-          if (MODE == MODE_GATEUP) {
-            float v[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) v[r] = gateup_epilogue<T>(p.act, acc[mt][0][r], acc[mt][1][r], 1.0f);
-            *reinterpret_cast<uint2*>(orow + tile * 16 + 4 * g) = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
-          } else {
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-              *reinterpret_cast<uint2*>(orow + tile * 32 + t * 16 + 4 * g) =
-                  make_uint2(pack2<T>(acc[mt][t][0], acc[mt][t][1]), pack2<T>(acc[mt][t][2], acc[mt][t][3]));
-          }
-        }
-      }
+    // up to 16 rows: one 16-row token tile; otherwise passes of two tiles (one pass up to 32 rows)
+    if (re - rb <= 16) {
+      skinny_pass<T, WF, MODE, 1>(p, wrow, tile, rb, re, nch, lane);
+    } else {
+      for (int r0 = rb; r0 < re; r0 += 32) skinny_pass<T, WF, MODE, 2>(p, wrow, tile, r0, re, nch, lane);
     }
   }
 }
@@ -346,20 +356,14 @@ static int pick_waves(int64_t items) {
   return (int)((waves + 3) / 4 * 4);
 }
 
-template <typename T, int WF, int MT>
-static int launch_skinny_tw(int mode, const GemmParams& p, hipStream_t st) {
+template <typename T, int WF>
+static int launch_skinny_t(int mode, const GemmParams& p, int64_t, hipStream_t st) {
   const int tiles = (int)(mode == MODE_GATEUP ? p.n_out / 16 : p.n_out / 32);
   const int waves = pick_waves((int64_t)tiles * p.E);
   dim3 grid((unsigned)(waves / 4));
-  if (mode == MODE_GATEUP) grouped_skinny_kernel<T, WF, MODE_GATEUP, MT><<<grid, 256, 0, st>>>(p, tiles, waves);
-  else grouped_skinny_kernel<T, WF, MODE_DOWN, MT><<<grid, 256, 0, st>>>(p, tiles, waves);
+  if (mode == MODE_GATEUP) grouped_skinny_kernel<T, WF, MODE_GATEUP><<<grid, 256, 0, st>>>(p, tiles, waves);
+  else grouped_skinny_kernel<T, WF, MODE_DOWN><<<grid, 256, 0, st>>>(p, tiles, waves);
   return check_launch("grouped_skinny");
-}
-
-template <typename T, int WF>
-static int launch_skinny_t(int mode, const GemmParams& p, int64_t max_rows_per_expert, hipStream_t st) {
-  if (max_rows_per_expert <= 16) return launch_skinny_tw<T, WF, 1>(mode, p, st);
-  return launch_skinny_tw<T, WF, 2>(mode, p, st);
 }
 
 int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
