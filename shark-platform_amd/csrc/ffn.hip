@@ -42,12 +42,19 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
   return STMOE_OK;
 }
 
-// variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile, 3 skinny streaming kernel (decode)
+// variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile, 3 skinny streaming kernel (decode),
+//          4 MFMA 256x256 tile (prefill; packed Q8_0)
 static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
-    else variant = (p.offsets && p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ? 3 : 2;
+    else if (p.offsets && p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) variant = 3;
+    else variant = max_rows >= 512 ? 4 : 2;
+  }
+  if (variant == 4) {
+    int rc = launch_mfma_big(dtype, wtag, mode, p, max_rows, st);
+    if (rc != STMOE_ERR_UNSUPPORTED) return rc;
+    variant = 2;
   }
   if (variant == 3) {
     int rc = launch_skinny(dtype, wtag, mode, p, max_rows, st);

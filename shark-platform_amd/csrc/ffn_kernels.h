@@ -71,5 +71,6 @@ namespace stmoe {
 // STMOE_ERR_UNSUPPORTED when the family has no instantiation for the combination.
 int launch_generic(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_mfma_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
+int launch_mfma_big(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 }  // namespace stmoe
