@@ -31,7 +31,13 @@ template <> __device__ __forceinline__ floatx4_t mfma16b<bf16_t>(const u32x4_t& 
 }
 
 static constexpr int BIG_BK = 64;
-static constexpr int BIG_LS = BIG_BK + 8;  // LDS row stride (elements)
+static constexpr int BIG_LS = BIG_BK;  // LDS row stride (elements): 128 bytes = 8 units of 16 bytes, no padding
+
+// LDS rows are XOR-swizzled: the 16-byte unit u of row r lives at unit u ^ (r & 7).  ds_read_b128 serves lanes
+// in groups {0-3, 20-23}, {32-35, 52-55}, ... (4 rows of one K group and the next 4 rows of the neighbouring
+// K group) and ds_write_b128 in groups of 8 consecutive lanes; with the swizzle every such group touches 8
+// distinct 16-byte bank groups for the operand reads, the weight-row writes and the token-row writes alike.
+__device__ __forceinline__ int lds_off(int row, int unit) { return row * BIG_LS + ((unit ^ (row & 7)) << 3); }
 
 // One packed 1 KB piece (16 rows x 64 k of 1-byte samples, or 16 rows x 128 k of nibbles) as held by one lane.
 template <int WF> struct BigPiece;
@@ -59,11 +65,14 @@ template <> struct BigPiece<WF_Q8_0_P> {
   }
 };
 
+struct BigTagOn { static constexpr bool value = true; };
+struct BigTagOff { static constexpr bool value = false; };
+
 // WN x WM wavefronts; each owns 128 weight rows x 64 token rows (32 accumulator tiles = 128 registers, which
 // leaves the register allocator room: a 128 x 128 wavefront tile fills all 256 accumulation registers and made
 // the compiler shuffle accumulators between register files around every MFMA).
-template <typename T, int WF, int MODE, int WN, int WM>
-__global__ void __launch_bounds__(64 * WN * WM, 1)
+template <typename T, int WF, int MODE, int WN, int WM, int STAGES>
+__global__ void __launch_bounds__(64 * WN * WM, STAGES == 1 ? 2 : 1)
 grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
   constexpr int NTHR = 64 * WN * WM;
   constexpr int BN = 128 * WN;           // weight rows per workgroup tile (GATEUP: BN/2 gate + BN/2 up)
@@ -127,7 +136,9 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
   auto load_global = [&](int64_t kt) {
 #pragma unroll
     for (int j = 0; j < WPIECES; ++j) {
-      wreg[j].q = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wq[j] + kt * 1024));
+      // plain (cacheable) loads: the token tiles of one (expert, feature tile) run back to back on one XCD and
+      // share the weight tile in its L2
+      wreg[j].q = *reinterpret_cast<const u32x4_t*>(wq[j] + kt * 1024);
       const uint32_t d = wd[j][(kt >> 2) * 128 + (kt & 3) * 2];
       wreg[j].dsel = d | (d << 16);
     }
@@ -141,13 +152,13 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
     for (int j = 0; j < WPIECES; ++j) {
       uint32_t v[8];
       wreg[j].template convert<T>(v);
-      u32x4_t* dst = reinterpret_cast<u32x4_t*>(&Ws[((wave * WPIECES + j) * 16 + n_in) * BIG_LS + g * 16]);
-      dst[0] = (u32x4_t){v[0], v[1], v[2], v[3]};
-      dst[1] = (u32x4_t){v[4], v[5], v[6], v[7]};
+      const int row = (wave * WPIECES + j) * 16 + n_in;
+      *reinterpret_cast<u32x4_t*>(&Ws[lds_off(row, 2 * g)]) = (u32x4_t){v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<u32x4_t*>(&Ws[lds_off(row, 2 * g + 1)]) = (u32x4_t){v[4], v[5], v[6], v[7]};
     }
 #pragma unroll
     for (int j = 0; j < XPIECES; ++j)
-      *reinterpret_cast<u32x4_t*>(&Xs[((tid >> 3) + XROWS_PER_PASS * j) * BIG_LS + (tid & 7) * 8]) = xreg[j];
+      *reinterpret_cast<u32x4_t*>(&Xs[lds_off((tid >> 3) + XROWS_PER_PASS * j, tid & 7)]) = xreg[j];
   };
 
   // ---- consumer -----------------------------------------------------------------------------------------
@@ -170,30 +181,54 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
     u32x4_t bf[4];
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj)
-      bf[tj] = *reinterpret_cast<const u32x4_t*>(&Xs[(wm * 64 + tj * 16 + n_in) * BIG_LS + ks * 32 + 8 * g]);
+      bf[tj] = *reinterpret_cast<const u32x4_t*>(&Xs[lds_off(wm * 64 + tj * 16 + n_in, ks * 4 + g)]);
 #pragma unroll
     for (int ti = 0; ti < 8; ++ti) {
-      const u32x4_t af = *reinterpret_cast<const u32x4_t*>(&Ws[(w_lds_row(ti) + n_in) * BIG_LS + ks * 32 + 8 * g]);
+      const u32x4_t af = *reinterpret_cast<const u32x4_t*>(&Ws[lds_off(w_lds_row(ti) + n_in, ks * 4 + g)]);
 #pragma unroll
       for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = mfma16b<T>(af, bf[tj], acc[ti][tj]);
     }
   };
 
   const int64_t nkt = p.kred >> 6;
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-  if (nkt > 1) load_global(1);
-  for (int64_t kt = 0; kt < nkt; ++kt) {
-    const int stage = (int)(kt & 1);
-    if (active) compute(stage, 0);
-    if (kt + 1 < nkt) {
-      store_lds(stage ^ 1);
-      if (kt + 2 < nkt) load_global(kt + 2);
+  // ACTIVE is a compile-time tag so that the steady-state loop is one straight-line block (producer and MFMA
+  // instructions can be interleaved by the scheduler); wavefronts whose token rows are all past the end run the
+  // producer-only copy of the loop.
+  auto main_loop = [&](auto active_tag) {
+    constexpr bool ACTIVE = decltype(active_tag)::value;
+    if constexpr (STAGES == 2) {
+      load_global(0);
+      store_lds(0);
+      __syncthreads();
+      if (nkt > 1) load_global(1);
+      for (int64_t kt = 0; kt < nkt; ++kt) {
+        const int stage = (int)(kt & 1);
+        if constexpr (ACTIVE) compute(stage, 0);
+        if (kt + 1 < nkt) {
+          store_lds(stage ^ 1);
+          if (kt + 2 < nkt) load_global(kt + 2);
+        }
+        if constexpr (ACTIVE) compute(stage, 1);
+        __syncthreads();
+      }
+    } else {
+      // one LDS stage, next K step prefetched into registers; two workgroups share a CU and fill each other's
+      // barrier and load bubbles
+      load_global(0);
+      for (int64_t kt = 0; kt < nkt; ++kt) {
+        store_lds(0);
+        __syncthreads();
+        load_global(kt + 1 < nkt ? kt + 1 : kt);
+        if constexpr (ACTIVE) {
+          compute(0, 0);
+          compute(0, 1);
+        }
+        __syncthreads();
+      }
     }
-    if (active) compute(stage, 1);
-    __syncthreads();
-  }
+  };
+  if (active) main_loop(BigTagOn{});
+  else main_loop(BigTagOff{});
 
   // ---- epilogue -------------------------------------------------------------------------------------------
 #pragma unroll
@@ -220,12 +255,12 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
   }
 }
 
-template <typename T, int WF, int MODE, int WN, int WM>
+template <typename T, int WF, int MODE, int WN, int WM, int STAGES>
 static int launch_big_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   constexpr int BN = 128 * WN, BM = 64 * WM;
-  constexpr size_t lds_bytes = (size_t)2 * (BN + BM) * BIG_LS * 2;
+  constexpr size_t lds_bytes = (size_t)STAGES * (BN + BM) * BIG_LS * 2;
   static bool attr_set = false;
-  auto kern = grouped_mfma_big_kernel<T, WF, MODE, WN, WM>;
+  auto kern = grouped_mfma_big_kernel<T, WF, MODE, WN, WM, STAGES>;
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
       return set_error(STMOE_ERR_LAUNCH, "mfma big kernel: cannot reserve %zu bytes of LDS", lds_bytes);
@@ -239,20 +274,26 @@ static int launch_big_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   return check_launch("grouped_mfma_big");
 }
 
+#ifndef STMOE_BIG_WN
+#define STMOE_BIG_WN 2
+#endif
 #ifndef STMOE_BIG_WM
 #define STMOE_BIG_WM 4
 #endif
+#ifndef STMOE_BIG_STAGES
+#define STMOE_BIG_STAGES 2
+#endif
 template <typename T, int WF>
 static int launch_big_t(int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
-  if (mode == MODE_GATEUP) return launch_big_m<T, WF, MODE_GATEUP, 2, STMOE_BIG_WM>(p, max_rows, st);
-  return launch_big_m<T, WF, MODE_DOWN, 2, STMOE_BIG_WM>(p, max_rows, st);
+  if (mode == MODE_GATEUP) return launch_big_m<T, WF, MODE_GATEUP, STMOE_BIG_WN, STMOE_BIG_WM, STMOE_BIG_STAGES>(p, max_rows, st);
+  return launch_big_m<T, WF, MODE_DOWN, STMOE_BIG_WN, STMOE_BIG_WM, STMOE_BIG_STAGES>(p, max_rows, st);
 }
 
 int launch_mfma_big(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (max_rows == 0) return STMOE_OK;
   if (wtag != WF_Q8_0_P)
     return set_error(STMOE_ERR_UNSUPPORTED, "mfma big kernel: needs weights in the packed Q8_0 order");
-  if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0 || p.n_out % (mode == MODE_GATEUP ? 128 : 256) != 0)
+  if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0 || p.n_out % (mode == MODE_GATEUP ? 64 * STMOE_BIG_WN : 128 * STMOE_BIG_WN) != 0)
     return set_error(STMOE_ERR_UNSUPPORTED, "mfma big kernel: needs K %% 256 == 0 and output features in whole tiles");
   if (act_dtype == STMOE_F16) return launch_big_t<f16_t, WF_Q8_0_P>(mode, p, max_rows, st);
   if (act_dtype == STMOE_BF16) return launch_big_t<bf16_t, WF_Q8_0_P>(mode, p, max_rows, st);
