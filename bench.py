@@ -157,6 +157,16 @@ def cpu_baseline(theta, h_cpu, sample_tokens):
     }, y_gather
 
 
+def measured_traffic(key):
+    """HBM bytes per launch from the committed rocprofv3 counter runs (profiles/traffic.json), or None."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            t = json.load(f)[key]
+        return t["read_bytes"] + t["write_bytes"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -165,6 +175,9 @@ def main():
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--decode-tokens", type=int, default=32)
     ap.add_argument("--cpu-sample", type=int, default=16, help="tokens timed on the CPU baseline (0 to skip)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (5 times) so that rocprofv3 FETCH_SIZE/WRITE_SIZE readings "
+                         "of the kernels can be scaled by what the same counters read for a copy of known size")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every box of this run has a single MI355X, so --gpus must be 1", file=sys.stderr)
@@ -187,7 +200,8 @@ def main():
     roofline = {
         "kernel": "grouped gate/up projection (prefill)", "bound": "mfma", "achieved": round(achieved, 2),
         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4),
-        "traffic": None, "avg_kernel_ms": round(st["gate_up"], 4),
+        "traffic": measured_traffic("prefill_gate_up") if T == 2048 else None, "avg_kernel_ms": round(st["gate_up"], 4),
+        "algorithmic": gateup_flops, "algorithmic_unit": "flop per launch",
     }
 
     dms, dgpu_ms, dst, _ = run_leg(block, h_dec.to(dev), max(args.steps, 50), args.warmup)
@@ -200,9 +214,19 @@ def main():
         "layer_frac_hbm": round(3 * wbytes_one / (dgpu_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "stage_ms": {k: round(v, 4) for k, v in dst.items()},
         "roofline": {"kernel": "grouped gate/up projection (decode)", "bound": "hbm", "achieved": round(d_achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(d_achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "avg_kernel_ms": round(dst["gate_up"], 4)},
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(d_achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": measured_traffic("decode_gate_up") if args.decode_tokens == 32 else None,
+                     "avg_kernel_ms": round(dst["gate_up"], 4), "algorithmic": 2 * wbytes_one,
+                     "algorithmic_unit": "expert-weight bytes per launch"},
     }
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     cpu = None
     if args.cpu_sample > 0:
