@@ -73,8 +73,21 @@ dispatch_build_kernel(const int32_t* __restrict__ idx, int64_t n, int E, int32_t
   }
 }
 
-// One workgroup per token.  o = sum over slots of round(gate * y) (fp32 sum in slot order, rounded to T);
-// optional RMS norm of o; optional residual add.
+// One workgroup per token; every thread owns 8 consecutive features (16-byte loads for 16-bit types).
+// o = sum over slots of round(gate * y) (fp32 sum in slot order, rounded to T); optional RMS norm of o;
+// optional residual add.
+template <typename T> struct Row8 {
+  float v[8];
+  __device__ __forceinline__ void load(const T* p) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = Cvt<T>::to_f32(p[i]);
+  }
+  __device__ __forceinline__ void store(T* p) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) p[i] = Cvt<T>::from_f32(v[i]);
+  }
+};
+
 template <typename T, typename W>
 __global__ void __launch_bounds__(256)
 combine_kernel(const T* __restrict__ y, const T* __restrict__ gate, const int32_t* __restrict__ inv, int k,
@@ -84,21 +97,31 @@ combine_kernel(const T* __restrict__ y, const T* __restrict__ gate, const int32_
   const int64_t t = blockIdx.x;
   T* orow = out + t * K;
   float ss = 0.0f;
-  for (int64_t i = threadIdx.x; i < K; i += 256) {
-    float acc = 0.0f;
+  for (int64_t i = (int64_t)threadIdx.x * 8; i < K; i += 256 * 8) {
+    float acc[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) acc[q] = 0.0f;
     for (int j = 0; j < k; ++j) {
       const int64_t r = inv[t * k + j];
       const float g = Cvt<T>::to_f32(gate[t * k + j]);
-      acc += round_to<T>(__fmul_rn(g, Cvt<T>::to_f32(y[r * K + i])));
+      Row8<T> yv;
+      yv.load(y + r * K + i);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc[q] += round_to<T>(__fmul_rn(g, yv.v[q]));
     }
-    const float o = round_to<T>(acc);
+    Row8<T> o;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) o.v[q] = round_to<T>(acc[q]);
     if (norm_w) {
-      ss = fmaf(o, o, ss);
-      orow[i] = Cvt<T>::from_f32(o);
-    } else {
-      const float r = residual ? round_to<T>(Cvt<T>::to_f32(residual[t * K + i]) + o) : o;
-      orow[i] = Cvt<T>::from_f32(r);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) ss = fmaf(o.v[q], o.v[q], ss);
+    } else if (residual) {
+      Row8<T> h;
+      h.load(residual + t * K + i);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) o.v[q] = round_to<T>(h.v[q] + o.v[q]);
     }
+    o.store(orow + i);
   }
   if (!norm_w) return;
   ss = wave_xor_sum(ss);
@@ -106,11 +129,17 @@ combine_kernel(const T* __restrict__ y, const T* __restrict__ gate, const int32_
   __syncthreads();
   const float total = (partial[0] + partial[1]) + (partial[2] + partial[3]);
   const float rs = 1.0f / sqrtf(total / (float)K + eps);
-  for (int64_t i = threadIdx.x; i < K; i += 256) {  // each thread re-reads only what it wrote itself
-    float o = round_to<W>(Cvt<T>::to_f32(orow[i]) * rs);
-    o = round_to<T>(round_to<W>(Cvt<W>::to_f32(norm_w[i]) * o));
-    if (residual) o = round_to<T>(Cvt<T>::to_f32(residual[t * K + i]) + o);
-    orow[i] = Cvt<T>::from_f32(o);
+  for (int64_t i = (int64_t)threadIdx.x * 8; i < K; i += 256 * 8) {  // each thread re-reads only what it wrote itself
+    Row8<T> o;
+    o.load(orow + i);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      float v = round_to<W>(o.v[q] * rs);
+      v = round_to<T>(round_to<W>(Cvt<W>::to_f32(norm_w[i + q]) * v));
+      if (residual) v = round_to<T>(Cvt<T>::to_f32(residual[t * K + i + q]) + v);
+      o.v[q] = v;
+    }
+    o.store(orow + i);
   }
 }
 
@@ -132,7 +161,8 @@ extern "C" int stmoe_dispatch_build(const int32_t* idx, int64_t n_pairs, int E, 
 extern "C" int stmoe_combine(const void* y_sorted, const void* gate, const int32_t* inv, int dtype, int64_t T, int k,
                              int64_t K, const void* out_norm_w, int w_dtype, float eps, const void* residual,
                              void* out, stmoe_stream_t stream) {
-  STMOE_REQUIRE(T >= 0 && K > 0 && k >= 1, STMOE_ERR_SHAPE, "combine: T=%lld K=%lld k=%d", (long long)T, (long long)K, k);
+  STMOE_REQUIRE(T >= 0 && K > 0 && K % 8 == 0 && k >= 1, STMOE_ERR_SHAPE, "combine: T=%lld K=%lld (a multiple of 8) k=%d",
+                (long long)T, (long long)K, k);
   if (T == 0) return STMOE_OK;
   STMOE_REQUIRE(y_sorted && gate && inv && out, STMOE_ERR_NULL, "combine: NULL pointer");
   STMOE_REQUIRE(T < 0x7fffffffLL, STMOE_ERR_SHAPE, "combine: T too large");

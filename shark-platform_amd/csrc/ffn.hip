@@ -217,11 +217,16 @@ static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int6
   hipStream_t st = as_stream(stream);
   // stages: 0 rms_norm, 1 router, 2 dispatch, 3 gate/up projection, 4 down projection, 5 combine;
   // stage s is bracketed by events[2s] and events[2s+1]
+  // ffn_norm and the router run as one launch when the token row fits the router's LDS row (stage 0 then has
+  // zero length in the event brackets); otherwise as two.
+  const bool fused_front = T < 0x7fffffffLL && K * dtype_size(dtype) <= 48 * 1024 && K % 8 == 0 && E <= 64 && aligned16(w_router);
   mark(events, 0, st);
-  if ((rc = stmoe_rms_norm(h, dtype, ffn_norm_w, w_dtype, T, K, eps, xn, stream))) return rc;
+  if (!fused_front && (rc = stmoe_rms_norm(h, dtype, ffn_norm_w, w_dtype, T, K, eps, xn, stream))) return rc;
   mark(events, 1, st);
   mark(events, 2, st);
-  if ((rc = stmoe_router_topk(xn, w_router, dtype, T, K, E, k, nullptr, idx, nullptr, gate, stream))) return rc;
+  if (fused_front) rc = norm_router(h, dtype, ffn_norm_w, w_dtype, eps, xn, w_router, T, K, E, k, idx, gate, st);
+  else rc = stmoe_router_topk(xn, w_router, dtype, T, K, E, k, nullptr, idx, nullptr, gate, stream);
+  if (rc) return rc;
   mark(events, 3, st);
   mark(events, 4, st);
   if ((rc = stmoe_dispatch_build(idx, T * k, E, counts, offsets, perm, inv, stream))) return rc;

@@ -160,6 +160,126 @@ router_topk_kernel(const T* __restrict__ x, const T* __restrict__ wr, int64_t T_
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// router, one workgroup (8 wavefronts) per token, optionally fused with the preceding RMS norm.
+//
+// Wavefront w computes the logits of experts w, w+8, ... with exactly the per-logit summation order documented
+// above (a logit is still produced by one wavefront: lane-owned 8-element pieces per 512-element chunk, then the
+// xor butterfly), so its bits are identical to router_topk_kernel's; spreading the experts over wavefronts lets
+// all loads of a logit be in flight at once, which is what a 32-token decode batch needs.
+// FUSE_NORM: the workgroup first normalises the token row (rms_norm_kernel's arithmetic), writes it to `xn`
+// (the expert projections read it) and routes the normalised row kept in LDS.
+template <typename T, typename W, bool FUSE_NORM>
+__global__ void __launch_bounds__(512)
+router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float eps, T* __restrict__ xn,
+                 const T* __restrict__ wr, int64_t K, int E, int k, T* __restrict__ logits_out,
+                 int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out, T* __restrict__ gate_out) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  T* xs = reinterpret_cast<T*>(smem);                                  // [K] the (normalised) token row
+  float* lg_s = reinterpret_cast<float*>(smem + ((K * sizeof(T) + 15) / 16) * 16);  // [E] logits, then 8 partials
+  float* part = lg_s + 64;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t t = blockIdx.x;
+  const T* xr = x + t * K;
+
+  if constexpr (FUSE_NORM) {
+    float ss = 0.0f;
+    for (int64_t i = tid; i < K; i += 512) {
+      const float v = Cvt<T>::to_f32(xr[i]);
+      ss = fmaf(v, v, ss);
+    }
+    ss = wave_xor_sum(ss);
+    if (lane == 0) part[wave] = ss;
+    __syncthreads();
+    const float total = ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+    const float rs = 1.0f / sqrtf(total / (float)K + eps);
+    for (int64_t i = tid; i < K; i += 512) {
+      float o = round_to<W>(Cvt<T>::to_f32(xr[i]) * rs);
+      o = round_to<W>(Cvt<W>::to_f32(norm_w[i]) * o);
+      const T r = Cvt<T>::from_f32(o);
+      xs[i] = r;
+      xn[t * K + i] = r;
+    }
+  } else {
+    for (int64_t i = (int64_t)tid * 8; i < K; i += 512 * 8)
+      *reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(xs) + i * sizeof(T)) =
+          *reinterpret_cast<const uint4*>(reinterpret_cast<const unsigned char*>(xr) + i * sizeof(T));
+    if constexpr (sizeof(T) == 4)
+      for (int64_t i = (int64_t)tid * 8 + 4; i < K; i += 512 * 8)
+        *reinterpret_cast<uint4*>(&xs[i]) = *reinterpret_cast<const uint4*>(&xr[i]);
+  }
+  __syncthreads();
+
+  for (int e = wave; e < E; e += 8) {
+    float acc = 0.0f;
+    const T* wrow = wr + (int64_t)e * K;
+    for (int64_t k0 = (int64_t)lane * 8; k0 < K; k0 += 512) {
+      Vec8<T> xv, wv;
+      xv.load(xs + k0);
+      wv.load(wrow + k0);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc = __fadd_rn(acc, __fmul_rn(xv.v[j], wv.v[j]));
+    }
+    const float l = round_to<T>(wave_xor_sum(acc));
+    if (lane == 0) {
+      lg_s[e] = l;
+      if (logits_out) logits_out[t * E + e] = Cvt<T>::from_f32(l);
+    }
+  }
+  __syncthreads();
+  if (tid != 0) return;
+
+  // fp32 softmax, top-k by (logit descending, index ascending), renormalised gates: same arithmetic and order
+  // as router_topk_kernel.
+  float mx = lg_s[0];
+  for (int e = 1; e < E; ++e) mx = fmaxf(mx, lg_s[e]);
+  float denom = 0.0f;
+  for (int e = 0; e < E; ++e) denom += expf(lg_s[e] - mx);
+  uint64_t taken = 0;
+  float vsum = 0.0f;
+  for (int j = 0; j < k; ++j) {
+    int best = -1;
+    float bestv = 0.0f;
+    for (int e = 0; e < E; ++e) {
+      const float v = lg_s[e];
+      if (!((taken >> e) & 1ull) && (best < 0 || v > bestv)) {
+        best = e;
+        bestv = v;
+      }
+    }
+    taken |= 1ull << best;
+    const float p = expf(bestv - mx) / denom;
+    idx_out[t * k + j] = best;
+    if (idx64_out) idx64_out[t * k + j] = best;
+    part[8 + j] = p;  // part has 64 + 8 floats of room after the partial sums
+    vsum += p;
+  }
+  for (int j = 0; j < k; ++j) gate_out[t * k + j] = Cvt<T>::from_f32(part[8 + j] / vsum);
+}
+
+template <typename T, typename W, bool FUSE_NORM>
+static int launch_router_wg(const void* x, const void* norm_w, float eps, void* xn, const void* wr, int64_t T_tokens,
+                            int64_t K, int E, int k, void* logits, int32_t* idx, int64_t* idx64, void* gate, hipStream_t st) {
+  const size_t lds = ((K * sizeof(T) + 15) / 16) * 16 + (64 + 8 + 64) * sizeof(float);
+  if (lds > 64 * 1024) return set_error(STMOE_ERR_UNSUPPORTED, "router: K=%lld does not fit the per-token LDS row", (long long)K);
+  router_wg_kernel<T, W, FUSE_NORM><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
+      (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate);
+  return check_launch("router_wg");
+}
+
+// ffn_norm + router in one launch (used by the fused layer forward).  norm weight dtype: f32, or the activation dtype.
+int norm_router(const void* h, int dtype, const void* norm_w, int w_dtype, float eps, void* xn, const void* wr,
+                int64_t T_tokens, int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st) {
+#define STMOE_NR(TT, WW) return launch_router_wg<TT, WW, true>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, nullptr, idx, nullptr, gate, st)
+  if (dtype == STMOE_F32 && w_dtype == STMOE_F32) STMOE_NR(float, float);
+  if (dtype == STMOE_F16 && w_dtype == STMOE_F32) STMOE_NR(f16_t, float);
+  if (dtype == STMOE_BF16 && w_dtype == STMOE_F32) STMOE_NR(bf16_t, float);
+  if (dtype == STMOE_F16 && w_dtype == STMOE_F16) STMOE_NR(f16_t, f16_t);
+  if (dtype == STMOE_BF16 && w_dtype == STMOE_BF16) STMOE_NR(bf16_t, bf16_t);
+#undef STMOE_NR
+  return set_error(STMOE_ERR_DTYPE, "norm_router: dtype %d with weight dtype %d not implemented", dtype, w_dtype);
+}
+
 template <typename T>
 static int launch_router(const void* x, const void* wr, int64_t T_tokens, int64_t K, int E, int k, void* logits,
                          int32_t* idx, int64_t* idx64, void* gate, hipStream_t st) {
@@ -209,6 +329,14 @@ extern "C" int stmoe_router_topk(const void* x, const void* w_router, int dtype,
   STMOE_REQUIRE(x && w_router && idx_out && gate_out, STMOE_ERR_NULL, "router_topk: NULL pointer");
   STMOE_REQUIRE(aligned16(x) && aligned16(w_router), STMOE_ERR_ALIGN, "router_topk: x and w_router must be 16-byte aligned");
   hipStream_t st = as_stream(stream);
+  if (T < 0x7fffffffLL && K * dtype_size(dtype) <= 48 * 1024) {  // one workgroup per token: lower latency
+    switch (dtype) {
+      case STMOE_F32: return launch_router_wg<float, float, false>(x, nullptr, 0.f, nullptr, w_router, T, K, E, k, logits_out, idx_out, idx64_out, gate_out, st);
+      case STMOE_F16: return launch_router_wg<f16_t, float, false>(x, nullptr, 0.f, nullptr, w_router, T, K, E, k, logits_out, idx_out, idx64_out, gate_out, st);
+      case STMOE_BF16: return launch_router_wg<bf16_t, float, false>(x, nullptr, 0.f, nullptr, w_router, T, K, E, k, logits_out, idx_out, idx64_out, gate_out, st);
+      default: return set_error(STMOE_ERR_DTYPE, "router_topk: dtype %d is not f32/f16/bf16", dtype);
+    }
+  }
   switch (dtype) {
     case STMOE_F32: return launch_router<float>(x, w_router, T, K, E, k, logits_out, idx_out, idx64_out, gate_out, st);
     case STMOE_F16: return launch_router<f16_t>(x, w_router, T, K, E, k, logits_out, idx_out, idx64_out, gate_out, st);
