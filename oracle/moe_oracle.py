@@ -20,6 +20,8 @@ How each function is pinned (tests/test_oracle_*.py):
   q8_0_unpack / q4_1_unpack ... hand-assembled ggml blocks (struct layouts quoted at
                                 ST/types/gguf_interop/layouts.py:33-39,263-270)
   rms_norm .................... the formula of the reference's test (tests/ops/ops_test.py:228-232) in float64
+  rms_norm_ordered ............ equals rms_norm bit for bit where every partial sum is exact, and within fp32 rounding of it
+                                elsewhere; a pure-Python sequential restatement of the order on a tiny case
   router ...................... float64 brute force on tiny inputs incl. forced ties (tie rule: lower index)
   router_logits_ordered ....... equals an exact (float64) dot product wherever rounding is not in play, and
                                 a pure-Python sequential restatement on a tiny case
@@ -240,6 +242,37 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return out.to(orig)
 
 
+def rms_norm_ordered(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """rms_norm with the mean-of-squares summation order the HIP kernels document (the reference leaves the order to
+    torch.mean): virtual thread j of 512 adds the fp32 squares of elements j, j+512, ... in order; the 64 sums of each of
+    the 8 groups of 64 threads are combined by the xor butterfly 32..1; the 8 group sums as ((s0+s1)+(s2+s3))+((s4+s5)+
+    (s6+s7)).  Everything else is the reference's arithmetic in fp32: sum / K, 1 / sqrt(. + eps), x * that, weight * ., cast."""
+    assert weight.dtype == torch.float32
+    T, K = x.shape
+    x32 = x.float().numpy()
+    C = (K + 511) // 512
+    sq = np.zeros((T, C * 512), dtype=np.float32)
+    sq[:, :K] = (x32 * x32).astype(np.float32)
+    sq = sq.reshape(T, C, 512)
+    acc = np.zeros((T, 512), dtype=np.float32)
+    for c in range(C):
+        acc = (acc + sq[:, c, :]).astype(np.float32)
+    acc = acc.reshape(T, 8, 64)
+    lanes = np.arange(64)
+    for off in (32, 16, 8, 4, 2, 1):
+        acc = (acc + acc[:, :, lanes ^ off]).astype(np.float32)
+    s = acc[:, :, 0]
+    f32 = np.float32
+    total = ((s[:, 0] + s[:, 1]).astype(f32) + (s[:, 2] + s[:, 3]).astype(f32)).astype(f32) + \
+            ((s[:, 4] + s[:, 5]).astype(f32) + (s[:, 6] + s[:, 7]).astype(f32)).astype(f32)
+    total = total.astype(f32)
+    var = (total / f32(K)).astype(f32)
+    rs = (f32(1.0) / np.sqrt((var + f32(eps)).astype(f32)).astype(f32)).astype(f32)
+    o = (x32 * rs[:, None]).astype(f32)
+    o = (weight.numpy()[None, :] * o).astype(f32)
+    return torch.from_numpy(o).to(x.dtype)
+
+
 def router_logits(x: torch.Tensor, w_router: torch.Tensor) -> torch.Tensor:
     """linear_default -> matmul_default (ST/ops/default_impls.py:328-359): weight cast to x's dtype, result in x's
     dtype.  For 16-bit types the products are exact in fp32 and torch accumulates in fp32; computing the fp32
@@ -359,8 +392,12 @@ def moe_block(h, ffn_norm_w, w_router, w_gate, w_up, w_down, k: int, eps: float,
     """MoeBlock.forward (ST/layers/mixture_of_experts_block.py:64-90).  h [B,S,K] or [T,K].
     Returns (y, idx, gate)."""
     shape = h.shape
-    x = rms_norm(h, ffn_norm_w, eps).reshape(-1, shape[-1])
-    logits = router_logits_ordered(x, w_router) if ordered_logits else router_logits(x, w_router)
+    if ordered_logits:  # the kernels' documented summation orders: routing becomes reproducible bit for bit
+        x = rms_norm_ordered(h.reshape(-1, shape[-1]), ffn_norm_w, eps)
+        logits = router_logits_ordered(x, w_router)
+    else:               # torch's own (unspecified) orders, as the reference runs
+        x = rms_norm(h, ffn_norm_w, eps).reshape(-1, shape[-1])
+        logits = router_logits(x, w_router)
     idx, gate, _ = route(logits, k)
     fn = grouped_ffn_moe if formulation == "grouped" else pre_gather_ffn_moe
     out = fn(x, idx, gate, w_gate, w_up, w_down, activation).reshape(shape)

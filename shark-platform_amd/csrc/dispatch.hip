@@ -128,14 +128,14 @@ combine_kernel(const T* __restrict__ y, const T* __restrict__ gate, const int32_
   if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
   __syncthreads();
   const float total = (partial[0] + partial[1]) + (partial[2] + partial[3]);
-  const float rs = 1.0f / sqrtf(total / (float)K + eps);
+  const float rs = rms_scale(total, K, eps);
   for (int64_t i = (int64_t)threadIdx.x * 8; i < K; i += 256 * 8) {  // each thread re-reads only what it wrote itself
     Row8<T> o;
     o.load(orow + i);
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-      float v = round_to<W>(o.v[q] * rs);
-      v = round_to<T>(round_to<W>(Cvt<W>::to_f32(norm_w[i + q]) * v));
+      float v = round_to<W>(keep_f32(__fmul_rn(o.v[q], rs)));
+      v = round_to<T>(round_to<W>(keep_f32(__fmul_rn(Cvt<W>::to_f32(norm_w[i + q]), v))));
       if (residual) v = round_to<T>(Cvt<T>::to_f32(residual[t * K + i + q]) + v);
       o.v[q] = v;
     }

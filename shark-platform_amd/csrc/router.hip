@@ -6,27 +6,37 @@
 namespace stmoe {
 
 // ---------------------------------------------------------------------------------------------------
-// rms_norm: one workgroup per row.  x32 = float(x); o = x32 * rsqrt(mean(x32^2) + eps);
+// rms_norm: one workgroup of 512 threads per row.  x32 = float(x); o = x32 * (1 / sqrt(mean(x32^2) + eps));
 // o = w * W(o) in W = dtype of w; result rounded to T.
+//
+// Summation order of the mean of squares (part of the contract, restated by the parity oracle, because the
+// router's top-k is only reproducible bit for bit if its input is): thread j adds the squares of elements
+// j, j+512, j+1024, ... in that order (square and add rounded separately), the 64 sums of a wavefront are
+// combined by the xor butterfly 32..1, and the 8 wavefront sums as ((s0+s1)+(s2+s3))+((s4+s5)+(s6+s7)).
+// The fused norm+router kernel below uses the same function.
+__device__ __forceinline__ float block512_sum_sq_finish(float ss, float* part) {
+  ss = wave_xor_sum(ss);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  return ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+}
+
 template <typename T, typename W>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 rms_norm_kernel(const T* __restrict__ x, const W* __restrict__ w, int64_t K, float eps, T* __restrict__ out) {
-  __shared__ float partial[4];
+  __shared__ float partial[8];
   const T* row = x + (int64_t)blockIdx.x * K;
   T* orow = out + (int64_t)blockIdx.x * K;
   float ss = 0.0f;
-  for (int64_t i = threadIdx.x; i < K; i += 256) {
+  for (int64_t i = threadIdx.x; i < K; i += 512) {
     const float v = Cvt<T>::to_f32(row[i]);
-    ss = fmaf(v, v, ss);
+    ss = __fadd_rn(ss, __fmul_rn(v, v));
   }
-  ss = wave_xor_sum(ss);
-  if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = ss;
-  __syncthreads();
-  const float total = (partial[0] + partial[1]) + (partial[2] + partial[3]);
-  const float rs = 1.0f / sqrtf(total / (float)K + eps);
-  for (int64_t i = threadIdx.x; i < K; i += 256) {
-    float o = round_to<W>(Cvt<T>::to_f32(row[i]) * rs);
-    o = round_to<W>(Cvt<W>::to_f32(w[i]) * o);
+  const float total = block512_sum_sq_finish(ss, partial);
+  const float rs = rms_scale(total, K, eps);
+  for (int64_t i = threadIdx.x; i < K; i += 512) {
+    float o = round_to<W>(keep_f32(__fmul_rn(Cvt<T>::to_f32(row[i]), rs)));
+    o = round_to<W>(keep_f32(__fmul_rn(Cvt<W>::to_f32(w[i]), o)));
     orow[i] = Cvt<T>::from_f32(o);
   }
 }
@@ -186,16 +196,13 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
     float ss = 0.0f;
     for (int64_t i = tid; i < K; i += 512) {
       const float v = Cvt<T>::to_f32(xr[i]);
-      ss = fmaf(v, v, ss);
+      ss = __fadd_rn(ss, __fmul_rn(v, v));
     }
-    ss = wave_xor_sum(ss);
-    if (lane == 0) part[wave] = ss;
-    __syncthreads();
-    const float total = ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
-    const float rs = 1.0f / sqrtf(total / (float)K + eps);
+    const float total = block512_sum_sq_finish(ss, part);
+    const float rs = rms_scale(total, K, eps);
     for (int64_t i = tid; i < K; i += 512) {
-      float o = round_to<W>(Cvt<T>::to_f32(xr[i]) * rs);
-      o = round_to<W>(Cvt<W>::to_f32(norm_w[i]) * o);
+      float o = round_to<W>(keep_f32(__fmul_rn(Cvt<T>::to_f32(xr[i]), rs)));
+      o = round_to<W>(keep_f32(__fmul_rn(Cvt<W>::to_f32(norm_w[i]), o)));
       const T r = Cvt<T>::from_f32(o);
       xs[i] = r;
       xn[t * K + i] = r;
@@ -307,7 +314,7 @@ extern "C" int stmoe_rms_norm(const void* x, int dtype, const void* w, int w_dty
   STMOE_REQUIRE(T < 0x7fffffffLL, STMOE_ERR_SHAPE, "rms_norm: T too large");
   hipStream_t st = as_stream(stream);
   dim3 g((unsigned)T);
-#define STMOE_RMS(TT, WW) rms_norm_kernel<TT, WW><<<g, 256, 0, st>>>((const TT*)x, (const WW*)w, K, eps, (TT*)out)
+#define STMOE_RMS(TT, WW) rms_norm_kernel<TT, WW><<<g, 512, 0, st>>>((const TT*)x, (const WW*)w, K, eps, (TT*)out)
   if (dtype == STMOE_F32 && w_dtype == STMOE_F32) STMOE_RMS(float, float);
   else if (dtype == STMOE_F16 && w_dtype == STMOE_F32) STMOE_RMS(f16_t, float);
   else if (dtype == STMOE_BF16 && w_dtype == STMOE_F32) STMOE_RMS(bf16_t, float);

@@ -66,6 +66,14 @@ template <> struct Cvt<bf16_t> {
   static __device__ __forceinline__ bf16_t from_f32(float v) { return f32_to_bf16(v); }
 };
 
+// Forces an fp32 value into a register as is.  Without it the compiler may fuse an fp32 multiply with the following
+// conversion to fp16 into one mixed-precision instruction (v_fma_mix*), which rounds the exact product once; eager
+// torch rounds the product to fp32 first and then to fp16, and the two differ about once in 2^13 values.
+__device__ __forceinline__ float keep_f32(float v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 // Round an fp32 value to T and widen it again: the value a tensor of dtype T would hold.
 template <typename T> __device__ __forceinline__ float round_to(float v) {
   return Cvt<T>::to_f32(Cvt<T>::from_f32(v));
@@ -112,6 +120,16 @@ __device__ __forceinline__ float act_silu(float v) { return v / (1.0f + expf(-v)
 __device__ __forceinline__ float act_gelu_erf(float v) { return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f)); }
 template <int ACT> __device__ __forceinline__ float apply_act(float v) {
   return ACT == STMOE_ACT_SILU ? act_silu(v) : act_gelu_erf(v);
+}
+
+// 1 / sqrt(total / K + eps) with every step (divide, add, square root, divide) correctly rounded in fp32, as IEEE
+// host arithmetic gives it.  The fp32 square-root and divide instructions of the GPU are not correctly rounded, so
+// the three operations are done in fp64 and rounded once to fp32 (innocuous double rounding: 53 >= 2*24 + 2 bits).
+__device__ __forceinline__ float rms_scale(float total, int64_t K, float eps) {
+  const float var = (float)((double)total / (double)K);
+  const float ve = __fadd_rn(var, eps);
+  const float s = (float)sqrt((double)ve);
+  return (float)(1.0 / (double)s);
 }
 
 // ---- wavefront helpers -----------------------------------------------------------------------------

@@ -90,6 +90,10 @@ def test_rms_norm(device, dtype):
     want = O.rms_norm(x, w, 1e-5)
     got = _hip().rms_norm(x.to(device), w.to(device), 1e-5).cpu()
     assert O.rel_l2(got, want) < (1e-6 if dtype == torch.float32 else 1e-3)
+    # bit-exact against the restatement with the documented summation order (the router's input must be reproducible)
+    ordered = O.rms_norm_ordered(x, w, 1e-5)
+    view = torch.int32 if dtype == torch.float32 else torch.int16
+    assert torch.equal(got.view(view), ordered.view(view))
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])

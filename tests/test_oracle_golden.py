@@ -193,6 +193,36 @@ def test_rms_norm_formula():
     assert O.rel_l2(got, want16) < 1e-3
 
 
+def test_rms_norm_ordered_pins():
+    g = torch.Generator().manual_seed(44)
+    # small integers: every partial sum of squares is exact, so the order cannot matter -> bit-identical to rms_norm
+    x = torch.randint(-8, 9, (6, 1536), generator=g).to(torch.float16)
+    w = torch.ones(1536) + 0.25 * torch.randint(-2, 3, (1536,), generator=g).float()
+    assert torch.equal(O.rms_norm_ordered(x, w, 1e-5), O.rms_norm(x, w, 1e-5))
+    # general values: agrees with torch's order up to fp32 rounding, and with a pure-Python restatement of the order
+    x = torch.randn(2, 1100, generator=g).to(torch.float16)  # 1100 = 2 full passes of 512 + a ragged third
+    w = torch.ones(1100) + 0.1 * torch.randn(1100, generator=g)
+    got = O.rms_norm_ordered(x, w, 1e-5)
+    assert O.rel_l2(got, O.rms_norm(x, w, 1e-5)) < 1e-3
+    f32 = np.float32
+    for t in range(2):
+        th = [f32(0.0)] * 512
+        for i in range(1100):
+            v = f32(x[t, i])
+            th[i % 512] = f32(th[i % 512] + f32(v * v))
+        groups = []
+        for gidx in range(8):
+            lanes = th[gidx * 64 : (gidx + 1) * 64]
+            for off in (32, 16, 8, 4, 2, 1):
+                lanes = [f32(lanes[l] + lanes[l ^ off]) for l in range(64)]
+            groups.append(lanes[0])
+        total = f32(f32(f32(groups[0] + groups[1]) + f32(groups[2] + groups[3])) + f32(f32(groups[4] + groups[5]) + f32(groups[6] + groups[7])))
+        rs = f32(f32(1.0) / f32(np.sqrt(f32(f32(total / f32(1100)) + f32(1e-5)))))
+        for i in (0, 7, 511, 512, 1099):
+            want = np.float16(f32(f32(w[i]) * f32(f32(x[t, i]) * rs)))
+            assert float(got[t, i]) == float(want)
+
+
 # ---- router -----------------------------------------------------------------------------------------------------
 def test_topk_tie_rule_brute_force():
     vals = torch.tensor([[0.1, 0.3, 0.3, 0.2, 0.3], [0.5, 0.5, 0.5, 0.5, 0.5], [0.0, 1.0, 0.0, 1.0, 0.5]])
