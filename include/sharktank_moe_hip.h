@@ -163,6 +163,17 @@ int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N,
                       void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
                       stmoe_stream_t stream);
 
+/* One gathered-expert projection over all (token, slot) pairs, without the [T,k,rows,cols] weight gather of
+ * `weights[experts]` + einsum_2args (ffn_moe_block.py:37-41; sharktank/sharktank/ops/default_impls.py:72-94):
+ *   out[p, :] = W[idx[p]] . a[src(p), :],  p = t*k + j,  src(p) = t  (a [T, cols],   "mk,menk->men")   if !a_per_pair
+ *                                                           src(p) = p  (a [T*k, cols], "mek,menk->men")  if a_per_pair
+ * out [T*k, rows] in pair order (i.e. [T, k, rows]); offsets/perm from stmoe_dispatch_build on idx. */
+int stmoe_grouped_mmt(const void* a, int dtype, int64_t T, int k, int a_per_pair, const stmoe_weight* w,
+                      const int32_t* offsets, const int32_t* perm, void* out, int variant, stmoe_stream_t stream);
+
+/* out[r, :] = g[r] * y[r, :] rounded to `dtype`: einsum "me,men->men" (default_impls.py:97-105) on flattened pairs. */
+int stmoe_scale_rows(const void* y, const void* g, int dtype, int64_t rows, int64_t K, void* out, stmoe_stream_t stream);
+
 /* Weighted combine (ffn_moe_block.py:73-74) and the layer tail (mixture_of_experts_block.py:86-90):
  *   o[t,:] = sum_j round(gate[t,j] * y[inv[t*k+j],:])   (slot order, fp32 sum, rounded to `dtype`)
  *   o = rms_norm(o; out_norm_w, eps) if out_norm_w != NULL     (layer_output_norm)

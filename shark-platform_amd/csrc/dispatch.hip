@@ -143,9 +143,35 @@ combine_kernel(const T* __restrict__ y, const T* __restrict__ gate, const int32_
   }
 }
 
+// out[r, :] = round(g[r] * y[r, :]) ("me,men->men": the gate weighting before the slot sum)
+template <typename T>
+__global__ void __launch_bounds__(256)
+scale_rows_kernel(const T* __restrict__ y, const T* __restrict__ g, int64_t K, T* __restrict__ out) {
+  const int64_t r = blockIdx.x;
+  const float gv = Cvt<T>::to_f32(g[r]);
+  for (int64_t i = threadIdx.x; i < K; i += 256)
+    out[r * K + i] = Cvt<T>::from_f32(keep_f32(__fmul_rn(gv, Cvt<T>::to_f32(y[r * K + i]))));
+}
+
 }  // namespace stmoe
 
 using namespace stmoe;
+
+extern "C" int stmoe_scale_rows(const void* y, const void* g, int dtype, int64_t rows, int64_t K, void* out,
+                                stmoe_stream_t stream) {
+  STMOE_REQUIRE(rows >= 0 && K > 0 && rows < 0x7fffffffLL, STMOE_ERR_SHAPE, "scale_rows: rows=%lld K=%lld", (long long)rows, (long long)K);
+  if (rows == 0) return STMOE_OK;
+  STMOE_REQUIRE(y && g && out, STMOE_ERR_NULL, "scale_rows: NULL pointer");
+  hipStream_t st = as_stream(stream);
+  dim3 grid((unsigned)rows);
+  switch (dtype) {
+    case STMOE_F32: scale_rows_kernel<float><<<grid, 256, 0, st>>>((const float*)y, (const float*)g, K, (float*)out); break;
+    case STMOE_F16: scale_rows_kernel<f16_t><<<grid, 256, 0, st>>>((const f16_t*)y, (const f16_t*)g, K, (f16_t*)out); break;
+    case STMOE_BF16: scale_rows_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)y, (const bf16_t*)g, K, (bf16_t*)out); break;
+    default: return set_error(STMOE_ERR_DTYPE, "scale_rows: dtype %d is not f32/f16/bf16", dtype);
+  }
+  return check_launch("scale_rows");
+}
 
 extern "C" int stmoe_dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets,
                                     int32_t* perm, int32_t* inv, stmoe_stream_t stream) {

@@ -160,6 +160,28 @@ extern "C" int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight
   return run_projection(variant, dtype, weight_tag(w), MODE_DOWN, p, M, as_stream(stream));
 }
 
+extern "C" int stmoe_grouped_mmt(const void* a, int dtype, int64_t T, int k, int a_per_pair, const stmoe_weight* w,
+                                 const int32_t* offsets, const int32_t* perm, void* out, int variant,
+                                 stmoe_stream_t stream) {
+  STMOE_REQUIRE(w, STMOE_ERR_NULL, "grouped_mmt: weight descriptor is NULL");
+  STMOE_REQUIRE(T >= 0 && k >= 1, STMOE_ERR_SHAPE, "grouped_mmt: T=%lld k=%d", (long long)T, k);
+  STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
+                "grouped_mmt: activation dtype %d is not f32/f16/bf16", dtype);
+  int rc;
+  if ((rc = check_weight(w, "grouped_mmt", w->experts, w->rows, w->cols))) return rc;
+  if (T == 0) return STMOE_OK;
+  STMOE_REQUIRE(a && offsets && perm && out, STMOE_ERR_NULL, "grouped_mmt: NULL pointer");
+  STMOE_REQUIRE(aligned16(a) && aligned16(out), STMOE_ERR_ALIGN, "grouped_mmt: a and out must be 16-byte aligned");
+  STMOE_REQUIRE((w->cols * dtype_size(dtype)) % 16 == 0 && (w->rows * dtype_size(dtype)) % 8 == 0, STMOE_ERR_SHAPE,
+                "grouped_mmt: row sizes must keep 16-byte (input) and 8-byte (output) alignment");
+  GemmParams p{};
+  p.a = a; p.lda = w->cols; p.perm = perm; p.k_top = a_per_pair ? 1 : k; p.offsets = offsets; p.E = (int32_t)w->experts;
+  p.w0 = make_view(w); p.w1 = p.w0;
+  p.out = out; p.ldo = w->rows; p.out_perm = perm; p.n_out = w->rows; p.kred = w->cols; p.act = 0; p.x_scale = nullptr;
+  p.expert_rows_bound = T;
+  return run_projection(variant, dtype, weight_tag(w), MODE_DOWN, p, T * k, as_stream(stream));
+}
+
 // ---- whole layer ----------------------------------------------------------------------------------
 // Workspace carve-up (each piece 256-byte aligned):
 //   xn [T,K] T | logits-free | idx i32 [T,k] | gate T [T,k] | counts i32 [E] | offsets i32 [E+1] |

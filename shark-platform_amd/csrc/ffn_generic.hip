@@ -74,7 +74,7 @@ grouped_generic_kernel(GemmParams p) {
   if (MODE == MODE_GATEUP) acc1 = wave_xor_sum(acc1);
   if (lane == 0) {
     const float scale = p.x_scale ? *p.x_scale : 1.0f;
-    T* o = reinterpret_cast<T*>(p.out) + (int64_t)i * p.ldo + n;
+    T* o = reinterpret_cast<T*>(p.out) + out_row(p, i) * p.ldo + n;
     if (MODE == MODE_GATEUP) *o = Cvt<T>::from_f32(gateup_epilogue<T>(p.act, acc0, acc1, scale));
     else *o = Cvt<T>::from_f32(acc0 * scale);
   }

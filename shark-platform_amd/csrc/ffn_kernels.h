@@ -23,6 +23,7 @@ struct GemmParams {
   WeightView w0, w1;      // GATEUP: gate, up.  DOWN: w0 only
   void* out;
   int64_t ldo;
+  const int32_t* out_perm;  // optional: output row of sorted position i is out_perm[i] (scatter back to pair order)
   int64_t n_out;          // rows of the weight matrices
   int64_t kred;           // reduction length
   int32_t act;
@@ -55,6 +56,8 @@ __device__ __forceinline__ bool find_tile(const GemmParams& p, int slot, int BM,
 __device__ __forceinline__ float act_rt(int act, float v) {
   return act == STMOE_ACT_SILU ? act_silu(v) : act_gelu_erf(v);
 }
+
+__device__ __forceinline__ int64_t out_row(const GemmParams& p, int i) { return p.out_perm ? (int64_t)p.out_perm[i] : (int64_t)i; }
 
 template <typename T> __device__ __forceinline__ float gateup_epilogue(int act, float g, float u, float scale) {
   const float gr = round_to<T>(g * scale);

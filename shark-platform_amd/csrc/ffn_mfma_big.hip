@@ -235,7 +235,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
   for (int tj = 0; tj < 4; ++tj) {
     const int r = wm * 64 + tj * 16 + n_in;
     if (r < rows_here) {
-      T* orow = reinterpret_cast<T*>(p.out) + (int64_t)(row_begin + r) * p.ldo;
+      T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo;
       if (MODE == MODE_GATEUP) {
 #pragma unroll
         for (int ti = 0; ti < 4; ++ti) {

@@ -151,7 +151,7 @@ grouped_mfma_tile_kernel(GemmParams p) {
           else v[r] = acc[0][ti][tj][r] * scale;
         }
         uint2 pk = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
-        *reinterpret_cast<uint2*>(reinterpret_cast<T*>(p.out) + (int64_t)i * p.ldo + n) = pk;
+        *reinterpret_cast<uint2*>(reinterpret_cast<T*>(p.out) + out_row(p, i) * p.ldo + n) = pk;
       }
     }
 }

@@ -282,7 +282,7 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
   for (int mt = 0; mt < MT; ++mt) {
     const int i = r0 + mt * 16 + n_in;
     if (i < re) {
-      T* orow = reinterpret_cast<T*>(p.out) + (int64_t)i * p.ldo;
+      T* orow = reinterpret_cast<T*>(p.out) + out_row(p, i) * p.ldo;
       if (MODE == MODE_GATEUP) {
         float v[4];
 #pragma unroll

@@ -80,6 +80,8 @@ SIGNATURES = {
     "stmoe_moe_forward_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int64, c_int64, c_int]),
     "stmoe_grouped_ffn": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, POINTER(StmoeWeight), POINTER(StmoeWeight),
                                   POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    "stmoe_grouped_mmt": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, POINTER(StmoeWeight), c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "stmoe_scale_rows": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "stmoe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int64, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p]),
     "stmoe_moe_forward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
                                   POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
@@ -373,6 +375,32 @@ def grouped_ffn(x, w_gate: DeviceWeight, w_up: DeviceWeight, w_down: DeviceWeigh
                                      _ptr(offsets), _ptr(perm), None, _ptr(y), _ptr(workspace), workspace.numel(), variant,
                                      _stream(dev)))
     return y
+
+
+def grouped_mmt(a: torch.Tensor, w: "DeviceWeight", offsets, perm, T: int, k: int, *, a_per_pair: bool,
+                variant: int = VARIANT_AUTO) -> torch.Tensor:
+    """a [T, cols] (or [T*k, cols] when a_per_pair) -> out [T, k, rows]: every pair's row times its expert's matrix."""
+    dev = _dev(a, offsets, perm)
+    lib = load_library()
+    a_c = _contig(a)
+    out = torch.empty((T, k, w.rows), dtype=a_c.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_grouped_mmt(_ptr(a_c), dtype_enum(a_c.dtype), T, k, int(bool(a_per_pair)), w.ref, _ptr(offsets),
+                                     _ptr(perm), _ptr(out), variant, _stream(dev)))
+    return out
+
+
+def scale_rows(y: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """y [..., K] * g [...] (one factor per row), rounded to y's dtype."""
+    dev = _dev(y, g)
+    lib = load_library()
+    y_c, g_c = _contig(y), _contig(g.to(y.dtype))
+    K = y_c.shape[-1]
+    rows = y_c.numel() // K if K else 0
+    out = torch.empty_like(y_c)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_scale_rows(_ptr(y_c), _ptr(g_c), dtype_enum(y_c.dtype), rows, K, _ptr(out), _stream(dev)))
+    return out
 
 
 def combine(y_sorted, gate, inv, T: int, k: int, *, out_norm_w=None, eps: float = 0.0, residual=None) -> torch.Tensor:

@@ -12,7 +12,8 @@ import torch
 import torch.nn.functional as F
 
 from .. import _hip
-from ..ops import device_weight
+from .. import ops
+from ..ops import device_weight, gather_experts
 from ..types import Theta
 from .base import ThetaLayer
 
@@ -52,6 +53,21 @@ class PreGatherFFNMOE(ThetaLayer):
                 device_weight(self.ffn_down, stacked=True, prepack=self.prepack_weights),
             )
         return self._dw
+
+    def pre_matmul_gather(self, inputs, weights, experts, einstring="mk,menk->men"):
+        """`einsum_2args(inputs, weights[experts, :, :], einstring)` as in the reference
+        (sharktank/sharktank/layers/ffn_moe_block.py:37-41); the gather stays lazy and the product is grouped by expert."""
+        return ops.einsum_2args(inputs, gather_experts(weights, experts), einstring)
+
+    def forward_unfused(self, h: torch.Tensor, experts: torch.Tensor, expert_gate: torch.Tensor):
+        """The reference's forward written with the same `ops` calls, one kernel per einsum (ffn_moe_block.py:60-74).
+        `forward` computes the same values with fused kernels; this path exists for callers that compose the ops."""
+        act = {_hip.ACT_SILU: F.silu, _hip.ACT_GELU_ERF: F.gelu}[self._act]
+        ffn_gate = ops.elementwise(act, self.pre_matmul_gather(h, self.ffn_gate, experts))
+        ffn_up = self.pre_matmul_gather(h, self.ffn_up, experts)
+        ffn_down = self.pre_matmul_gather(ffn_gate * ffn_up, self.ffn_down, experts, einstring="mek,menk->men")
+        ffn_down = ops.einsum_2args(expert_gate, ffn_down, "me,men->men")
+        return torch.sum(ffn_down, dim=1)
 
     @property
     def expert_count(self) -> int:

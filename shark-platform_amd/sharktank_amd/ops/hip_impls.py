@@ -12,11 +12,11 @@ from torch import Tensor
 
 from .. import _hip
 from ..types.layouts import BlockScaledI4Layout, BlockScaledLayout, TensorScaledLayout
-from ..types.tensors import InferenceTensor, PrimitiveTensor, QuantizedTensor, unbox_tensor
+from ..types.tensors import GatheredExpertsTensor, InferenceTensor, PrimitiveTensor, QuantizedTensor, unbox_tensor
 from ._registry import AllOfType
 from .signatures import *
 
-__all__ = ["device_weight"]
+__all__ = ["device_weight", "gather_experts"]
 
 _FLOAT_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
 
@@ -148,3 +148,79 @@ linear.override(Tensor, QuantizedTensor)(_linear)
 @get_index.override(AllOfType(Tensor, PrimitiveTensor))
 def get_index_default(tensor, key):
     return unbox_tensor(tensor)[key]
+
+
+# ---- the gathered-expert einsums of PreGatherFFNMOE -------------------------------------------------------------
+
+
+def _is_expert_index(key):
+    """`weights[experts, :, :]` / `weights[experts]` with an integer index tensor of shape [T, k]."""
+    if isinstance(key, torch.Tensor):
+        first, rest = key, ()
+    elif isinstance(key, tuple) and key and isinstance(key[0], torch.Tensor):
+        first, rest = key[0], key[1:]
+    else:
+        return None
+    if first.dim() != 2 or first.dtype not in (torch.int32, torch.int64):
+        return None
+    if any(not (isinstance(r, slice) and r == slice(None)) for r in rest):
+        return None
+    return first
+
+
+def gather_experts(weights, experts: torch.Tensor) -> GatheredExpertsTensor:
+    """Lazy `weights[experts, :, :]` for an expert-stacked weight [E, rows, cols] of any supported kind."""
+    if len(weights.shape) != 3:
+        raise ValueError(f"gather_experts: expert-stacked weight must be [E, rows, cols], got {list(weights.shape)}")
+    w = weights if isinstance(weights, InferenceTensor) else None
+    if w is None:
+        from ..types.tensors import DefaultPrimitiveTensor
+
+        w = DefaultPrimitiveTensor(data=weights)
+    return GatheredExpertsTensor(weights=w, experts=experts)
+
+
+@get_index.override(QuantizedTensor)
+def get_index_quantized_experts(tensor: QuantizedTensor, key):
+    experts = _is_expert_index(key)
+    if experts is None or len(tensor.shape) != 3:
+        return NotImplemented
+    return gather_experts(tensor, experts)
+
+
+def _gathered_state(g: GatheredExpertsTensor):
+    if g._device_weight is None:
+        g._device_weight = device_weight(g.weights, stacked=True)
+    if g._dispatch is None:
+        _, offsets, perm, _ = _hip.dispatch_build(g.experts, g._device_weight.experts)
+        g._dispatch = (offsets, perm)
+    return g._device_weight, g._dispatch
+
+
+@einsum_2args.override(Tensor, GatheredExpertsTensor)
+def einsum_2args_gathered_experts(input0, input1: GatheredExpertsTensor, einsum_str: str):
+    x = unbox_tensor(input0)
+    T, k = input1.experts.shape
+    if x.dtype not in _FLOAT_DTYPES:
+        return NotImplemented
+    if einsum_str == "mk,menk->men":
+        if x.dim() != 2 or x.shape[0] != T:
+            return NotImplemented
+        dw, (offsets, perm) = _gathered_state(input1)
+        return _hip.grouped_mmt(x, dw, offsets, perm, T, k, a_per_pair=False)
+    if einsum_str == "mek,menk->men":
+        if x.dim() != 3 or x.shape[0] != T or x.shape[1] != k:
+            return NotImplemented
+        dw, (offsets, perm) = _gathered_state(input1)
+        return _hip.grouped_mmt(x.reshape(T * k, x.shape[2]), dw, offsets, perm, T, k, a_per_pair=True)
+    return NotImplemented
+
+
+@einsum_2args.override(Tensor, Tensor)
+def einsum_2args_me_men(input0, input1, einsum_str: str):
+    if einsum_str != "me,men->men":
+        return NotImplemented
+    g, y = unbox_tensor(input0), unbox_tensor(input1)
+    if g.dim() != 2 or y.dim() != 3 or tuple(g.shape) != tuple(y.shape[:2]) or y.dtype not in _FLOAT_DTYPES:
+        return NotImplemented
+    return _hip.scale_rows(y, g)

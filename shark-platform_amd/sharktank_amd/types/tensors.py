@@ -17,6 +17,7 @@ import torch
 __all__ = [
     "AnyTensor",
     "DefaultPrimitiveTensor",
+    "GatheredExpertsTensor",
     "InferenceTensor",
     "PlanarQuantizedTensor",
     "PrimitiveTensor",
@@ -188,6 +189,38 @@ class PlanarQuantizedTensor(QuantizedTensor):
 
     def __repr__(self):
         return f"PlanarQuantized({self.name}, {self.shape}, layout={self.layout})"
+
+
+class GatheredExpertsTensor(InferenceTensor):
+    """`weights[experts, :, :]` of an expert-stacked weight, kept lazy.
+
+    The reference materialises this gather as a [T, k, rows, cols] copy of expert weights per token
+    (sharktank/sharktank/layers/ffn_moe_block.py:39, ops/default_impls.py:204-218) and then runs T batched M=1
+    products.  Here the indexing result only records the stacked weight and the index tensor; `einsum_2args` on it
+    groups the (token, slot) pairs by expert and multiplies each group with its expert's matrix once.
+    """
+
+    def __init__(self, *, weights: InferenceTensor, experts: torch.Tensor, name: str = UnnamedTensorName):
+        T, k = experts.shape
+        super().__init__(name=name, shape=[T, k] + list(weights.shape[1:]))
+        self.weights = weights
+        self.experts = experts
+        self._dispatch = None  # (offsets, perm) of `experts`, built on first use
+        self._device_weight = None
+
+    @property
+    def globals(self) -> Dict[str, torch.Tensor]:
+        g = dict(self.weights.globals)
+        g[f"{self.name}:experts"] = self.experts
+        return g
+
+    def _clone_with_globals(self, new_globals):
+        experts = new_globals[f"{self.name}:experts"]
+        weights = self.weights._clone_with_globals({k: v for k, v in new_globals.items() if k in self.weights.globals})
+        return GatheredExpertsTensor(weights=weights, experts=experts, name=self.name)
+
+    def __repr__(self):
+        return f"GatheredExperts({self.weights!r}[{list(self.experts.shape)}])"
 
 
 AnyTensor = Union[torch.Tensor, InferenceTensor]

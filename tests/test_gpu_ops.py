@@ -1,0 +1,147 @@
+"""The `sharktank.ops`-level surface on the GPU: quantized matmul/linear with the generators of the reference's own
+kernel tests, dispatch selection, and layout dequant through the layout classes."""
+
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def test_mmt_block_scaled_q8_reference_generator(device):
+    """Shapes, generators and tolerances of sharktank/tests/kernels/mmt_block_scaled_q8_test.py:24-41 (seed 42):
+    a [4,16,3200], d [3200,100,1], qs [3200,100,32]; expected = a @ (d*qs).flatten(1).T, atol 1e-3 (scaled), rtol 1e-5."""
+    from sharktank_amd import ops, types as ST
+
+    torch.manual_seed(42)
+    for dtype, atol, rtol in ((torch.float32, 1e-3, 1e-5), (torch.float16, 1.0, 1e-3)):
+        a = (torch.rand([4, 16, 3200], dtype=torch.float32) / 64).to(dtype)
+        d = (torch.rand([3200, 100, 1], dtype=torch.float32) / 64).to(torch.float16)
+        qs = (torch.rand([3200, 100, 32], dtype=torch.float32) * 32.0).to(torch.int8)
+        w = ST.PlanarQuantizedTensor(shape=[3200, 3200], layout=ST.BlockScaledLayout([3200, 3200], d.to(device), qs.to(device)))
+        ops._test_enable_last_op_dispatch(True)
+        try:
+            got = ops.matmul(a.to(device), w, transpose_rhs=True)
+            assert ops._test_get_last_op_dispatch().__name__ == "matmul_tensor_quantized"
+        finally:
+            ops._test_enable_last_op_dispatch(False)
+        assert got.shape == (4, 16, 3200) and got.dtype == dtype
+        b = O.dequant_block_scaled(d, qs).flatten(1).to(dtype)
+        ref = O.mmt(a, b)
+        torch.testing.assert_close(got.cpu(), ref, atol=atol * 1e-2, rtol=max(rtol, 2e-3 if dtype == torch.float16 else 1e-4))
+
+
+def test_mmt_block_scaled_offset_q4_reference_generator(device):
+    """sharktank/tests/kernels/mmt_block_scaled_offset_q4_test.py:25-44: a/256, d/256, qs uint8*255, m + 16."""
+    from sharktank_amd import ops, types as ST
+
+    torch.manual_seed(42)
+    a = torch.rand([4, 16, 3200], dtype=torch.float32) / 256.0
+    d = (torch.rand([3200, 100, 1], dtype=torch.float32) / 256.0).to(torch.float16)
+    qs = (torch.rand([3200, 100, 16], dtype=torch.float32) * 255.0).to(torch.uint8)
+    m = (torch.rand([3200, 100, 1], dtype=torch.float32) + 16.0).to(torch.float16)
+    w = ST.PlanarQuantizedTensor(shape=[3200, 3200], layout=ST.BlockScaledI4Layout(
+        [3200, 3200], d.to(device), qs.to(device), m=m.to(device), signed=False))
+    got = ops.matmul(a.to(device), w, transpose_rhs=True)
+    b = O.dequant_block_scaled_i4(d, qs, m).flatten(1).float()
+    ref = torch.matmul(a, b.T)
+    torch.testing.assert_close(got.cpu(), ref, atol=1e-2, rtol=1e-3)
+
+
+def test_linear_and_dense_matmul(device):
+    from sharktank_amd import ops, types as ST
+
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(33, 256, generator=g).to(torch.float16)
+    w = torch.randn(48, 256, generator=g) * 0.05  # f32 weight, cast to the activation dtype as linear_default does
+    got = ops.linear(x.to(device), ST.DefaultPrimitiveTensor(data=w.to(device)))
+    ref = O.mmt(x, w)
+    assert got.dtype == torch.float16 and O.rel_l2(got.cpu(), ref) < 1e-3
+    with pytest.raises(NotImplementedError):
+        ops.matmul(x.to(device), w.to(device), transpose_rhs=False)
+
+
+def test_layout_classes_dequant_on_device(device):
+    from sharktank_amd import types as ST
+
+    g = torch.Generator().manual_seed(2)
+    w = torch.randn(3, 64, 128, generator=g) * 0.02
+    d, qs = O.quantize_q8_0(w)
+    lay = ST.BlockScaledLayout([3, 64, 128], d.to(device), qs.to(device))
+    assert torch.equal(lay.dequant().cpu(), O.dequant_block_scaled(d, qs).reshape(3, 64, 128))
+    d4, m4, q4 = O.quantize_q4_1(w)
+    lay4 = ST.BlockScaledI4Layout([3, 64, 128], d4.to(device), q4.to(device), m=m4.to(device))
+    assert torch.equal(lay4.dequant(torch.float32).cpu(), O.dequant_block_scaled_i4(d4, q4, m4, dtype=torch.float32).reshape(3, 64, 128))
+    assert torch.equal(lay4.qs.cpu(), O.promote_linear_i4_block_to_i8(q4))
+    # GGUF raw blocks -> planar planes -> device
+    raw = torch.cat([d.view(torch.uint8).reshape(-1, 2), qs.view(torch.uint8).reshape(-1, 32)], dim=1).reshape(-1)
+    q8 = ST.Q8_0(raw=raw, shape=[3, 64, 128]).to_planar().to(device="cuda:0")
+    assert torch.equal(q8.unpack().dequant().cpu(), O.dequant_block_scaled(d, qs).reshape(3, 64, 128))
+
+
+def test_static_scaled_quantizer_fp8(device):
+    from sharktank_amd import types as ST
+
+    x = torch.randn(64, 32, generator=torch.Generator().manual_seed(3)).to(torch.float16)
+    rscale = torch.tensor(0.0118, dtype=torch.float32)
+    q = ST.StaticScaledQuantizer(scale=(1.0 / rscale).to(device), reciprocal_scale=rscale.to(device), dtype=torch.float8_e4m3fn)
+    qt = q.quantize(x.to(device))
+    want_qs, _, _ = O.static_quantize_per_tensor(x, rscale, torch.float8_e4m3fn)
+    assert torch.equal(qt.unpack().qs.cpu().view(torch.uint8), want_qs.view(torch.uint8))
+    deq = qt.unpack().dequant()
+    assert deq.dtype == torch.float16
+    assert torch.equal(deq.cpu(), O.dequant_tensor_scaled(rscale, want_qs, layout_dtype=torch.float16))
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8", "dense"])
+@pytest.mark.parametrize("dtype,T", [(torch.float16, 40), (torch.bfloat16, 9), (torch.float32, 12)])
+def test_gathered_expert_einsums(device, fmt, dtype, T):
+    """`weights[experts]` + einsum_2args for the three einsum strings of PreGatherFFNMOE
+    (shapes as in sharktank/tests/kernels/einsum_q4_test.py:32-89, enlarged), against the materialised gather."""
+    import moe_cases as MC
+    from sharktank_amd import ops, types as ST
+
+    case = MC.build(MC.Case(T=T, K=128, N=96 if fmt == "dense" else 256, fmt=fmt, dtype=dtype, seed=70))
+    E, N, K, k = case.E, case.N, case.K, case.k
+    g = torch.Generator().manual_seed(71)
+    experts = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    x = case.planes["h"]
+    wg, wu, wd = MC.dense_weights(case)
+    w_it = MC.to_inference_tensor(fmt, case.planes["gate"], [E, N, K], "w", device)
+    gathered = w_it[experts.to(device), :, :] if fmt != "dense" else ops.gather_experts(w_it, experts.to(device))
+    assert isinstance(gathered, ST.GatheredExpertsTensor) and gathered.shape == [T, k, N, K]
+    got = ops.einsum_2args(x.to(device), gathered, "mk,menk->men")
+    want = O._mm_rt(x.unsqueeze(1), wg[experts].reshape(T, k * N, K)).reshape(T, k, N)
+    tol = 1e-5 if dtype == torch.float32 else (1e-3 if dtype == torch.float16 else 8e-3)
+    assert got.shape == (T, k, N) and O.rel_l2(got.cpu(), want) < tol
+    # "mek,menk->men" with the down matrix
+    z = torch.randn(T, k, N, generator=g).to(dtype)
+    wd_it = MC.to_inference_tensor(fmt, case.planes["down"], [E, K, N], "wd", device)
+    got2 = ops.einsum_2args(z.to(device), ops.gather_experts(wd_it, experts.to(device)), "mek,menk->men")
+    want2 = O._mm_rt(z.reshape(T * k, 1, N), wd[experts].reshape(T * k, K, N)).reshape(T, k, K)
+    assert O.rel_l2(got2.cpu(), want2) < tol
+    # "me,men->men"
+    gate = torch.rand(T, k, generator=g).to(dtype)
+    got3 = ops.einsum_2args(gate.to(device), got2, "me,men->men")
+    assert torch.equal(got3.cpu(), (gate.unsqueeze(-1) * got2.cpu()))
+    with pytest.raises(NotImplementedError):
+        ops.einsum_2args(x.to(device), gathered, "mk,bnk->bmn")
+
+
+def test_forward_unfused_equals_fused(device):
+    import moe_cases as MC
+    from sharktank_amd.layers import PreGatherFFNMOE
+
+    case = MC.build(MC.Case(T=70, K=256, N=512, fmt="q4_1", dtype=torch.float16, act="gelu", seed=72))
+    layer = PreGatherFFNMOE(MC.make_theta(case, device), activation=torch.nn.functional.gelu)
+    g = torch.Generator().manual_seed(73)
+    experts = torch.stack([torch.randperm(case.E, generator=g)[: case.k] for _ in range(case.T)]).to(device)
+    gate = torch.rand(case.T, case.k, generator=g).to(case.dtype).to(device)
+    h = case.planes["h"].to(device)
+    a = layer(h, experts, gate)
+    b = layer.forward_unfused(h, experts, gate)
+    assert O.rel_l2(b.cpu(), a.cpu()) < 1e-3
+    wg, wu, wd = MC.dense_weights(case)
+    want = O.pre_gather_ffn_moe(case.planes["h"], experts.cpu(), gate.cpu(), wg, wu, wd, torch.nn.functional.gelu)
+    assert O.rel_l2(b.cpu(), want) < 1e-3
