@@ -113,10 +113,15 @@ int stmoe_dequant_tensor_scaled(const void* qs, int qs_dtype, const void* d, con
 int stmoe_quantize_fp8(const void* x, int x_dtype, const float* rscale, int64_t n, void* out_fp8,
                        stmoe_stream_t stream);
 
+/* quantize(x).unpack().dequant() of the same quantizer in one pass (the fake-quantised activations of
+ * sharktank/sharktank/layers/linear.py:72-78): out = T(f32(e4m3fn(clamp(T(x / rscale)))) * rscale), T = `dtype`. */
+int stmoe_fake_quant_fp8(const void* x, int dtype, const float* rscale, int64_t n, void* out, stmoe_stream_t stream);
+
 /* Load-time re-ordering of a planar quantized weight into the streaming order (and back).  For every tile of 16
  * consecutive rows: samples as [K/64][lane = 16*g + n][16 B] (Q8_0, fp8: row n, k = 64*kb + 16*g..+15) or
- * [K/128][lane][16 B] (Q4_1: row n, block 4*kb + g); block scales/offsets as [K/256][16 rows][8] fp16.  A pure
- * permutation of bytes: stmoe_unpack(stmoe_prepack(w)) == w bit for bit.  `planar` and `packed` describe the same
+ * [K/128][lane][16 B] (Q4_1: row n, block 4*kb + g; inside every dword the even elements fill the low half-word and
+ * the odd ones the high half-word); block scales/offsets as [K/256][16 rows][8] fp16.  A pure permutation of bytes
+ * (of nibbles for Q4_1): stmoe_unpack(stmoe_prepack(w)) == w bit for bit.  `planar` and `packed` describe the same
  * [experts, rows, cols] with formats X and X_PACKED and caller-owned planes of equal sizes; rows % 16 == 0 and
  * cols % 256 == 0.  The reference has no counterpart (its planes come from GGUF blocks,
  * sharktank/sharktank/types/gguf_interop/layouts.py:51-60,285-300, and are consumed row-major). */
@@ -154,14 +159,20 @@ size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int64_t K, int
  * for sorted position i (pair p = perm[i], token t = p / k, expert e with offsets[e] <= i < offsets[e+1])
  *   y[i,:] = Wd[e] . ( act(Wg[e] . x[t]) * (Wu[e] . x[t]) )
  * with each intermediate rounded to `dtype` where the reference materialises a tensor.  x [T,K];
- * y [T*k, K] in `dtype`.  `x_scale` (nullable, device float) is the reciprocal scale of fp8-quantised
- * activations: when given with FP8 weights, x is taken as e4m3fn [T,K] and results are scaled by it.
+ * y [T*k, K] in `dtype`.
+ * Quantised activations: `x_scale` / `z_scale` (nullable; each one device float) are the reciprocal scales of static
+ * per-tensor e4m3fn quantizers (StaticScaledQuantizer, quantizers.py:153-183) applied to x before the gate/up
+ * projections and to the intermediate before the down projection.  The reference semantics is quantise then
+ * dequantise (`quantize(x).unpack().dequant()`, sharktank/sharktank/layers/linear.py:72-78) followed by the
+ * floating-point path.  With FP8 weights and more than 32 tokens both operands are fed to the fp8 matrix cores as
+ * bytes and the fp32 dot product is scaled once by scale_x * d_w; otherwise the re-dequantised values go through the
+ * 16-bit kernels.  x itself is always given unquantised in `dtype`.
  * `variant` 0 picks the kernel by shape; other values force one (see the kernel list in ffn.hip). */
 int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                       const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
-                      int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
-                      void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
-                      stmoe_stream_t stream);
+                      int act, const int32_t* offsets, const int32_t* perm, const float* x_scale /*nullable*/,
+                      const float* z_scale /*nullable*/, void* y_sorted, void* workspace, size_t workspace_bytes,
+                      int variant, stmoe_stream_t stream);
 
 /* One gathered-expert projection over all (token, slot) pairs, without the [T,k,rows,cols] weight gather of
  * `weights[experts]` + einsum_2args (ffn_moe_block.py:37-41; sharktank/sharktank/ops/default_impls.py:72-94):
@@ -184,11 +195,13 @@ int stmoe_combine(const void* y_sorted, const void* gate, const int32_t* inv, in
 
 /* Whole MoeBlock.forward (mixture_of_experts_block.py:64-90) on h [T,K] -> out [T,K]:
  * ffn_norm -> router -> dispatch -> grouped FFN -> combine (+ layer_output_norm) + residual.
- * ffn_norm_w / out_norm_w are of w_dtype; out_norm_w may be NULL.  idx_out/gate_out ([T,k]) may be NULL. */
+ * ffn_norm_w / out_norm_w are of w_dtype; out_norm_w may be NULL.  idx_out/gate_out ([T,k]) may be NULL.
+ * x_scale / z_scale: activation quantizers of the expert FFN as in stmoe_grouped_ffn (NULL: none). */
 int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                       const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
                       const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
-                      const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
+                      const stmoe_weight* w_down, int act, const float* x_scale /*nullable*/,
+                      const float* z_scale /*nullable*/, void* out, int32_t* idx_out, void* gate_out,
                       void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream);
 
 /* stmoe_moe_forward with per-stage timing for benchmarks: `events` is a host array of 12 hipEvent_t created by
@@ -199,7 +212,8 @@ int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K, int64_t N,
 int stmoe_moe_forward_timed(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                             const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
                             const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
-                            const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
+                            const stmoe_weight* w_down, int act, const float* x_scale /*nullable*/,
+                            const float* z_scale /*nullable*/, void* out, int32_t* idx_out, void* gate_out,
                             void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream,
                             void** events);
 

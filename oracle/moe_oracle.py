@@ -149,6 +149,13 @@ def static_quantize_per_tensor(t, reciprocal_scale, dtype, offset=None):
     return qs, reciprocal_scale, offset
 
 
+def fake_quant_per_tensor(t, reciprocal_scale, dtype=torch.float8_e4m3fn):
+    """`q_input.quantize(x).unpack().dequant()` of a static per-tensor quantizer (ST/layers/linear.py:72-78): the
+    layout built by the quantizer has d = reciprocal_scale and dtype = t.dtype (ST/types/quantizers.py:176-183)."""
+    qs, d, _ = static_quantize_per_tensor(t, reciprocal_scale, dtype)
+    return dequant_tensor_scaled(d, qs, layout_dtype=t.dtype)
+
+
 def static_quantize_per_axis(t, scale, axis: int, dtype, offset=None):
     """Per-axis branch (ST/types/quantizers.py:184-230): qs = saturate_cast(t * scale (+ offset)); d = 1/scale."""
     shape = [1] * t.dim()
@@ -343,13 +350,17 @@ def _mm_rt(a: torch.Tensor, b_t: torch.Tensor) -> torch.Tensor:
     return torch.matmul(a.float(), b_t.float().transpose(-1, -2)).to(a.dtype)
 
 
-def pre_gather_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation: Callable = F.silu, chunk: int = 8):
+def pre_gather_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation: Callable = F.silu, chunk: int = 8,
+                       x_rscale=None, z_rscale=None):
     """PreGatherFFNMOE.forward in the reference's own operation order (ST/layers/ffn_moe_block.py:37-41,60-74 with
     mk_menk_men / mek_menk_men / me_men_men, ST/ops/default_impls.py:72-105): per-token gathered weights,
     batched M=1 products, every intermediate materialised in h's dtype.  Weights are dense [E,N,K]/[E,K,N]
     tensors already in h's dtype (dequantize-then-cast).  Tokens are independent, so they are processed in
-    chunks to bound the [chunk,k,N,K] gather."""
+    chunks to bound the [chunk,k,N,K] gather.  x_rscale / z_rscale: reciprocal scales of fake-quantised activations
+    (input of gate/up, input of down), None for none."""
     T = h.shape[0]
+    if x_rscale is not None:
+        h = fake_quant_per_tensor(h, x_rscale)
     out = torch.empty_like(h)
     for s in range(0, T, chunk):
         x = h[s : s + chunk]
@@ -361,6 +372,8 @@ def pre_gather_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation
         ffn_gate = activation(ffn_gate)
         ffn_up = _mm_rt(x.unsqueeze(1), w_up[ex].reshape(m_, e_ * n_, k_)).reshape(m_, e_, n_)
         z = ffn_gate * ffn_up
+        if z_rscale is not None:
+            z = fake_quant_per_tensor(z, z_rscale)
         wd = w_down[ex]  # [m,e,K,N]
         down = _mm_rt(z.reshape(m_ * e_, 1, n_), wd.reshape(m_ * e_, k_, n_)).reshape(m_, e_, k_)
         down = (g.reshape(m_ * e_, 1, 1) * down.reshape(m_ * e_, k_, 1)).reshape(m_, e_, k_)  # "me,men->men"
@@ -368,13 +381,16 @@ def pre_gather_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation
     return out
 
 
-def grouped_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation: Callable = F.silu):
+def grouped_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation: Callable = F.silu, x_rscale=None,
+                    z_rscale=None):
     """Same function, independent formulation: per expert, dense FFN on the rows routed to it (the shape of
     FFNMOE.forward, ST/layers/ffn_moe_block.py:120-127), then the weighted slot sum."""
     T, K = h.shape
     k = experts.shape[1]
     E = w_gate.shape[0]
     down = torch.zeros(T, k, K, dtype=h.dtype)
+    if x_rscale is not None:
+        h = fake_quant_per_tensor(h, x_rscale)
     for e in range(E):
         t_idx, j_idx = torch.nonzero(experts == e, as_tuple=True)
         if t_idx.numel() == 0:
@@ -382,13 +398,17 @@ def grouped_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation: C
         x = h[t_idx]
         a = activation(_mm_rt(x, w_gate[e]))
         u = _mm_rt(x, w_up[e])
-        down[t_idx, j_idx] = _mm_rt(a * u, w_down[e])
+        z = a * u
+        if z_rscale is not None:
+            z = fake_quant_per_tensor(z, z_rscale)
+        down[t_idx, j_idx] = _mm_rt(z, w_down[e])
     down = expert_gate.unsqueeze(-1) * down
     return torch.sum(down, dim=1)
 
 
 def moe_block(h, ffn_norm_w, w_router, w_gate, w_up, w_down, k: int, eps: float, activation: Callable = F.silu,
-              out_norm_w: Optional[torch.Tensor] = None, formulation: str = "grouped", ordered_logits: bool = False):
+              out_norm_w: Optional[torch.Tensor] = None, formulation: str = "grouped", ordered_logits: bool = False,
+              x_rscale=None, z_rscale=None):
     """MoeBlock.forward (ST/layers/mixture_of_experts_block.py:64-90).  h [B,S,K] or [T,K].
     Returns (y, idx, gate)."""
     shape = h.shape
@@ -400,7 +420,7 @@ def moe_block(h, ffn_norm_w, w_router, w_gate, w_up, w_down, k: int, eps: float,
         logits = router_logits(x, w_router)
     idx, gate, _ = route(logits, k)
     fn = grouped_ffn_moe if formulation == "grouped" else pre_gather_ffn_moe
-    out = fn(x, idx, gate, w_gate, w_up, w_down, activation).reshape(shape)
+    out = fn(x, idx, gate, w_gate, w_up, w_down, activation, x_rscale=x_rscale, z_rscale=z_rscale).reshape(shape)
     if out_norm_w is not None:
         out = rms_norm(out, out_norm_w, eps)
     return h + out, idx, gate

@@ -92,6 +92,20 @@ quantize_fp8_kernel(const T* __restrict__ x, const float* __restrict__ rscale, i
   out[i] = f32_to_fp8_e4m3fn(q);
 }
 
+// Quantise and dequantise again in one pass: the values a fake-quantised activation tensor holds.
+template <typename T>
+__global__ void __launch_bounds__(256)
+fake_quant_fp8_kernel(const T* __restrict__ x, const float* __restrict__ rscale, int64_t n, T* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float rs = *rscale;
+  float q = round_to<T>(__fdiv_rn(Cvt<T>::to_f32(x[i]), rs));
+  q = fminf(fmaxf(q, -448.0f), 448.0f);
+  if (q != q) q = __uint_as_float(0x7fc00000u);
+  const float v = fp8_e4m3fn_to_f32(f32_to_fp8_e4m3fn(q));
+  out[i] = Cvt<T>::from_f32(keep_f32(__fmul_rn(v, rs)));
+}
+
 template <bool I4>
 static int launch_block_scaled(const void* d, const void* m, int dm_dtype, const uint8_t* qs, int64_t n_blocks,
                                int block_size, int is_signed, void* out, int out_dtype, hipStream_t st) {
@@ -216,4 +230,20 @@ extern "C" int stmoe_quantize_fp8(const void* x, int x_dtype, const float* rscal
     default: return set_error(STMOE_ERR_DTYPE, "quantize_fp8: x dtype %d is not f32/f16/bf16", x_dtype);
   }
   return check_launch("quantize_fp8");
+}
+
+extern "C" int stmoe_fake_quant_fp8(const void* x, int dtype, const float* rscale, int64_t n, void* out,
+                                    stmoe_stream_t stream) {
+  STMOE_REQUIRE(n >= 0, STMOE_ERR_SHAPE, "fake_quant_fp8: n %lld < 0", (long long)n);
+  if (n == 0) return STMOE_OK;
+  STMOE_REQUIRE(x && rscale && out, STMOE_ERR_NULL, "fake_quant_fp8: NULL pointer");
+  dim3 g((unsigned)((n + 255) / 256));
+  hipStream_t st = as_stream(stream);
+  switch (dtype) {
+    case STMOE_F32: fake_quant_fp8_kernel<float><<<g, 256, 0, st>>>((const float*)x, rscale, n, (float*)out); break;
+    case STMOE_F16: fake_quant_fp8_kernel<f16_t><<<g, 256, 0, st>>>((const f16_t*)x, rscale, n, (f16_t*)out); break;
+    case STMOE_BF16: fake_quant_fp8_kernel<bf16_t><<<g, 256, 0, st>>>((const bf16_t*)x, rscale, n, (bf16_t*)out); break;
+    default: return set_error(STMOE_ERR_DTYPE, "fake_quant_fp8: dtype %d is not f32/f16/bf16", dtype);
+  }
+  return check_launch("fake_quant_fp8");
 }

@@ -43,7 +43,7 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 }
 
 // variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile, 3 skinny streaming kernel (decode),
-//          4 MFMA 256x256 tile (prefill; packed Q8_0)
+//          4 MFMA 256x256 tile (prefill; packed Q8_0), 5 fp8 matrix cores (fp8 weights and quantised activations)
 static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (variant == 0) {
@@ -74,10 +74,24 @@ static int run_projection(int variant, int dtype, int wtag, int mode, const Gemm
 
 using namespace stmoe;
 
+// Workspace of the grouped FFN: the intermediate z [T*k, N] in `dtype`, then (used only with quantised activations)
+// the quantised or re-dequantised copy of x [T, K] and the quantised intermediate [T*k, N] bytes.
+struct FfnWs {
+  size_t z, xa, zq, total;
+};
+static FfnWs carve_ffn(int64_t T, int k, int64_t K, int64_t N, int dtype) {
+  FfnWs w{};
+  const size_t es = dtype_size(dtype);
+  w.z = 0;
+  w.xa = align_up((size_t)T * k * N * es, 256);
+  w.zq = w.xa + align_up((size_t)T * K * es, 256);
+  w.total = w.zq + align_up((size_t)T * k * N, 256);
+  return w;
+}
+
 extern "C" size_t stmoe_grouped_ffn_workspace_bytes(int64_t T, int k, int64_t K, int64_t N, int dtype) {
-  (void)K;
-  if (T <= 0 || k <= 0 || N <= 0) return 0;
-  return align_up((size_t)T * k * N * dtype_size(dtype), 256);
+  if (T <= 0 || k <= 0 || N <= 0 || K <= 0) return 0;
+  return carve_ffn(T, k, K, N, dtype).total;
 }
 
 static inline void mark(void** events, int i, hipStream_t st) {
@@ -87,14 +101,13 @@ static inline void mark(void** events, int i, hipStream_t st) {
 static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                             const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
                             int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
-                            void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
+                            const float* z_scale, void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
                             stmoe_stream_t stream, void** events) {
   STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1, STMOE_ERR_SHAPE, "grouped_ffn: T=%lld K=%lld N=%lld E=%d k=%d",
                 (long long)T, (long long)K, (long long)N, E, k);
   STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
                 "grouped_ffn: activation dtype %d is not f32/f16/bf16", dtype);
   STMOE_REQUIRE(act == STMOE_ACT_SILU || act == STMOE_ACT_GELU_ERF, STMOE_ERR_UNSUPPORTED, "grouped_ffn: activation %d", act);
-  STMOE_REQUIRE(x_scale == nullptr, STMOE_ERR_UNSUPPORTED, "grouped_ffn: quantised activations are not implemented");
   int rc;
   if ((rc = check_weight(w_gate, "grouped_ffn(ffn_gate_exps)", E, N, K))) return rc;
   if ((rc = check_weight(w_up, "grouped_ffn(ffn_up_exps)", E, N, K))) return rc;
@@ -112,21 +125,63 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
                 workspace_bytes, need);
   hipStream_t st = as_stream(stream);
   const int64_t rows = T * k;
+  const FfnWs ws = carve_ffn(T, k, K, N, dtype);
+  char* base = (char*)workspace;
+  void* z = base + ws.z;
+  void* xa = base + ws.xa;
+  void* zq = base + ws.zq;
+
+  // Quantised activations (fp8 e4m3fn, static per-tensor scale).  With few rows per expert the projections are bound
+  // by the weight stream, so the samples are re-dequantised (the reference's own formulation) and the streaming kernel
+  // runs unchanged; otherwise both operands go to the fp8 matrix cores as bytes (variant 5).
+  const bool fp8_w_in = w_gate->format == STMOE_W_FP8 || w_gate->format == STMOE_W_FP8_PACKED;
+  const bool fp8_w_out = w_down->format == STMOE_W_FP8 || w_down->format == STMOE_W_FP8_PACKED;
+  const bool few_rows = T <= kSkinnyMaxRowsPerExpert;
+  STMOE_REQUIRE(variant != 5 || (x_scale && z_scale), STMOE_ERR_UNSUPPORTED, "grouped_ffn: variant 5 (fp8 matrix cores) needs x_scale and z_scale");
+  const bool t16 = dtype == STMOE_F16 || dtype == STMOE_BF16;
+  const bool mfma8_in = t16 && x_scale && fp8_w_in && w_gate->dtype == STMOE_F32 && K % 16 == 0 && (variant == 5 || (variant == 0 && !few_rows));
+  const bool mfma8_out = t16 && z_scale && fp8_w_out && w_down->dtype == STMOE_F32 && N % 16 == 0 && (variant == 5 || (variant == 0 && !few_rows));
+  const int v16 = variant == 5 ? 0 : variant;
 
   GemmParams p{};
   p.a = x; p.lda = K; p.perm = perm; p.k_top = k; p.offsets = offsets; p.E = E; p.fixed_rows = 0;
   p.w0 = make_view(w_gate); p.w1 = make_view(w_up);
-  p.out = workspace; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr; p.expert_rows_bound = T;
+  p.out = z; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr; p.expert_rows_bound = T;
   mark(events, 0, st);
-  if ((rc = run_projection(variant, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st))) return rc;
+  if (x_scale) {
+    if (mfma8_in) rc = stmoe_quantize_fp8(x, dtype, x_scale, T * K, xa, stream);
+    else rc = stmoe_fake_quant_fp8(x, dtype, x_scale, T * K, xa, stream);
+    if (rc) return rc;
+    p.a = xa;
+  }
+  if (mfma8_in) {
+    p.x_scale = x_scale;
+    if (mfma8_out) { p.out = zq; p.out_scale = z_scale; }
+    rc = launch_fp8_tile(dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
+  } else {
+    rc = run_projection(v16, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
+  }
+  if (rc) return rc;
   mark(events, 1, st);
 
   GemmParams q{};
-  q.a = workspace; q.lda = N; q.perm = nullptr; q.k_top = 1; q.offsets = offsets; q.E = E; q.fixed_rows = 0;
+  q.a = z; q.lda = N; q.perm = nullptr; q.k_top = 1; q.offsets = offsets; q.E = E; q.fixed_rows = 0;
   q.w0 = make_view(w_down); q.w1 = q.w0;
   q.out = y_sorted; q.ldo = K; q.n_out = K; q.kred = N; q.act = act; q.x_scale = nullptr; q.expert_rows_bound = T;
   mark(events, 2, st);
-  rc = run_projection(variant, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
+  if (z_scale) {
+    if (mfma8_out && !mfma8_in) rc = stmoe_quantize_fp8(z, dtype, z_scale, rows * N, zq, stream);
+    else if (!mfma8_out) rc = stmoe_fake_quant_fp8(z, dtype, z_scale, rows * N, z, stream);  // in place
+    else rc = STMOE_OK;
+    if (rc) return rc;
+  }
+  if (mfma8_out) {
+    q.a = zq;
+    q.x_scale = z_scale;
+    rc = launch_fp8_tile(dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
+  } else {
+    rc = run_projection(v16, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
+  }
   mark(events, 3, st);
   return rc;
 }
@@ -134,9 +189,9 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
 extern "C" int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                                  const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
                                  int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
-                                 void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
-                                 stmoe_stream_t stream) {
-  return grouped_ffn_impl(x, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, y_sorted,
+                                 const float* z_scale, void* y_sorted, void* workspace, size_t workspace_bytes,
+                                 int variant, stmoe_stream_t stream) {
+  return grouped_ffn_impl(x, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, z_scale, y_sorted,
                           workspace, workspace_bytes, variant, stream, nullptr);
 }
 
@@ -215,9 +270,9 @@ extern "C" size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int
 static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                             const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
                             const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
-                            const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
-                            void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream,
-                            void** events) {
+                            const stmoe_weight* w_down, int act, const float* x_scale, const float* z_scale, void* out,
+                            int32_t* idx_out, void* gate_out, void* workspace, size_t workspace_bytes, int variant,
+                            stmoe_stream_t stream, void** events) {
   STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1 && k <= E, STMOE_ERR_SHAPE,
                 "moe_forward: T=%lld K=%lld N=%lld E=%d k=%d", (long long)T, (long long)K, (long long)N, E, k);
   if (T == 0) return STMOE_OK;
@@ -253,7 +308,7 @@ static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int6
   mark(events, 4, st);
   if ((rc = stmoe_dispatch_build(idx, T * k, E, counts, offsets, perm, inv, stream))) return rc;
   mark(events, 5, st);
-  if ((rc = grouped_ffn_impl(xn, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, nullptr, y,
+  if ((rc = grouped_ffn_impl(xn, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, z_scale, y,
                              base + ws.ffn, workspace_bytes - ws.ffn, variant, stream, events ? events + 6 : nullptr)))
     return rc;
   mark(events, 10, st);
@@ -265,18 +320,19 @@ static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int6
 extern "C" int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                                  const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
                                  const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
-                                 const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
-                                 void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream) {
+                                 const stmoe_weight* w_down, int act, const float* x_scale, const float* z_scale,
+                                 void* out, int32_t* idx_out, void* gate_out, void* workspace, size_t workspace_bytes,
+                                 int variant, stmoe_stream_t stream) {
   return moe_forward_impl(h, dtype, T, K, N, E, k, ffn_norm_w, out_norm_w, w_dtype, eps, w_router, w_gate, w_up, w_down,
-                          act, out, idx_out, gate_out, workspace, workspace_bytes, variant, stream, nullptr);
+                          act, x_scale, z_scale, out, idx_out, gate_out, workspace, workspace_bytes, variant, stream, nullptr);
 }
 
 extern "C" int stmoe_moe_forward_timed(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                                        const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
                                        const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
-                                       const stmoe_weight* w_down, int act, void* out, int32_t* idx_out, void* gate_out,
-                                       void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream,
-                                       void** events) {
+                                       const stmoe_weight* w_down, int act, const float* x_scale, const float* z_scale,
+                                       void* out, int32_t* idx_out, void* gate_out, void* workspace,
+                                       size_t workspace_bytes, int variant, stmoe_stream_t stream, void** events) {
   return moe_forward_impl(h, dtype, T, K, N, E, k, ffn_norm_w, out_norm_w, w_dtype, eps, w_router, w_gate, w_up, w_down,
-                          act, out, idx_out, gate_out, workspace, workspace_bytes, variant, stream, events);
+                          act, x_scale, z_scale, out, idx_out, gate_out, workspace, workspace_bytes, variant, stream, events);
 }

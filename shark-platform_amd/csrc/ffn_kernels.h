@@ -28,6 +28,7 @@ struct GemmParams {
   int64_t kred;           // reduction length
   int32_t act;
   const float* x_scale;   // optional scale applied to the fp32 dot products (fp8 activations)
+  const float* out_scale; // fp8 kernel only: quantise the result with this reciprocal scale and store e4m3fn bytes
   int64_t expert_rows_bound;  // host-side bound of rows per expert (a token gives an expert at most one row)
 };
 
@@ -76,4 +77,5 @@ int launch_generic(int act_dtype, int wtag, int mode, const GemmParams& p, int64
 int launch_mfma_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_mfma_big(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
+int launch_fp8_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 }  // namespace stmoe

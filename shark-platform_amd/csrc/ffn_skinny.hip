@@ -88,34 +88,28 @@ template <> struct SkinnyW<WF_Q8_0> {
 
 template <> struct SkinnyW<WF_Q4_1> {
   u32x4_t q[2];
-  u32x4_t d, m;  // 8 block scales / offsets of the chunk
+  uint16_t d[2], m[2];  // scale / offset of the lane's own two blocks (4*i + g, i = 0, 1)
   __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
     const uint8_t* base = w.qs + ((row * w.cols + c * 256) >> 1) + 16 * g;
 #pragma unroll
     for (int i = 0; i < 2; ++i) q[i] = ld_stream16(base + 64 * i);
-    const int64_t b = (row * (w.cols >> 5) + c * 8) * 2;
-    d = ld_stream16(w.d + b);
-    m = ld_stream16(w.m + b);
+    const int64_t b = row * (w.cols >> 5) + c * 8 + g;
+    load_dm(reinterpret_cast<const uint16_t*>(w.d) + b, reinterpret_cast<const uint16_t*>(w.m) + b);
   }
-  template <typename T> __device__ __forceinline__ u32x4_t frag(int s, int g) const {
+  __device__ __forceinline__ void load_dm(const uint16_t* dp, const uint16_t* mp) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      d[i] = __builtin_nontemporal_load(dp + 4 * i);
+      m[i] = __builtin_nontemporal_load(mp + 4 * i);
+    }
+  }
+  template <typename T, bool PACKED = false> __device__ __forceinline__ u32x4_t frag(int s, int g) const {
     const int i = s >> 2, j = s & 3;
-    // block 4*i + g of the chunk: dword (4i+g)/2 = 2i + (g>>1), half g&1
-    const uint32_t dw = (g & 2) ? d[2 * i + 1] : d[2 * i];
-    const uint32_t mw = (g & 2) ? m[2 * i + 1] : m[2 * i];
-    const uint32_t dsel = (g & 1) ? (dw >> 16) : (dw & 0xffffu);
-    const uint32_t msel = (g & 1) ? (mw >> 16) : (mw & 0xffffu);
-    const half2_t dd = as_half2(dsel | (dsel << 16)), mm = as_half2(msel | (msel << 16));
-    const half2_t bias = {(f16_t)1024.0f, (f16_t)1024.0f};
-    const uint32_t w4 = q[i][j];  // 8 nibbles: element 2b = low nibble of byte b, 2b+1 = high nibble
+    const uint32_t w4 = q[i][j];  // 8 nibbles of block 4*i + g
     u32x4_t out;
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const uint32_t byte = (w4 >> (8 * b));
-      const uint32_t pair = 0x64006400u | (byte & 0xfu) | ((byte & 0xf0u) << 12);
-      half2_t v = (as_half2(pair) - bias) * dd;
-      v = v + mm;
-      out[b] = h2_to_T<T>(as_u32(v));
-    }
+    for (int b = 0; b < 4; ++b)
+      out[b] = h2_to_T<T>(q4_pair_dequant(PACKED ? q4_pair_packed(w4, b) : q4_pair_linear(w4, b), d[i], m[i]));
     return out;
   }
 };
@@ -136,8 +130,9 @@ template <> struct SkinnyW<WF_FP8_F32D> {
     for (int j = 0; j < 2; ++j) {
       const uint32_t u = q[i][2 * h + j];
       float f[4];
+      fp8x4_to_f32(u, f);
 #pragma unroll
-      for (int b = 0; b < 4; ++b) f[b] = __fmul_rn(fp8_e4m3fn_to_f32((uint8_t)(u >> (8 * b))), dv);
+      for (int b = 0; b < 4; ++b) f[b] = __fmul_rn(f[b], dv);
       out[2 * j] = pack2<T>(f[0], f[1]);
       out[2 * j + 1] = pack2<T>(f[2], f[3]);
     }
@@ -163,9 +158,11 @@ template <> struct SkinnyW<WF_Q4_1_P> : SkinnyW<WF_Q4_1> {
     const uint8_t* base = w.qs + (rt * (w.cols >> 7) + c * 2) * 1024 + (g * 16 + r) * 16;
 #pragma unroll
     for (int i = 0; i < 2; ++i) q[i] = ld_stream16(base + 1024 * i);
-    const int64_t b = (rt * (w.cols >> 8) + c) * 256 + r * 16;
-    d = ld_stream16(w.d + b);
-    m = ld_stream16(w.m + b);
+    const int64_t b = (rt * (w.cols >> 8) + c) * 128 + r * 8 + g;
+    load_dm(reinterpret_cast<const uint16_t*>(w.d) + b, reinterpret_cast<const uint16_t*>(w.m) + b);
+  }
+  template <typename T> __device__ __forceinline__ u32x4_t frag(int s, int g) const {
+    return SkinnyW<WF_Q4_1>::template frag<T, true>(s, g);
   }
 };
 template <> struct SkinnyW<WF_FP8_F32D_P> : SkinnyW<WF_FP8_F32D> {
@@ -298,8 +295,11 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
   }
 }
 
+// Workgroups resident per CU (two wavefronts per SIMD: the double-buffered chunks need about 200 registers).
+template <int WF> struct SkinnyOcc { static constexpr int value = 2; };
+
 template <typename T, int WF, int MODE>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(256, SkinnyOcc<WF>::value)
 grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
   const int lane = threadIdx.x & 63;
   const int n_in = lane & 15;
@@ -347,9 +347,9 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
   }
 }
 
-static int pick_waves(int64_t items) {
-  // 256 CUs x 2 workgroups x 4 wavefronts resident; give every wavefront the same number of items
-  const int64_t capacity = 2048;
+static int pick_waves(int64_t items, int wg_per_cu) {
+  // 256 CUs x resident workgroups x 4 wavefronts; give every wavefront the same number of items
+  const int64_t capacity = 1024 * wg_per_cu;
   if (items <= capacity) return (int)((items + 3) / 4 * 4);
   const int64_t per_wave = (items + capacity - 1) / capacity;
   const int64_t waves = (items + per_wave - 1) / per_wave;
@@ -359,7 +359,7 @@ static int pick_waves(int64_t items) {
 template <typename T, int WF>
 static int launch_skinny_t(int mode, const GemmParams& p, int64_t, hipStream_t st) {
   const int tiles = (int)(mode == MODE_GATEUP ? p.n_out / 16 : p.n_out / 32);
-  const int waves = pick_waves((int64_t)tiles * p.E);
+  const int waves = pick_waves((int64_t)tiles * p.E, SkinnyOcc<WF>::value);
   dim3 grid((unsigned)(waves / 4));
   if (mode == MODE_GATEUP) grouped_skinny_kernel<T, WF, MODE_GATEUP><<<grid, 256, 0, st>>>(p, tiles, waves);
   else grouped_skinny_kernel<T, WF, MODE_DOWN><<<grid, 256, 0, st>>>(p, tiles, waves);

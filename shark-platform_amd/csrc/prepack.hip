@@ -5,10 +5,13 @@
 // stores, for every tile of 16 consecutive weight rows, the bytes of one load instruction contiguously
 // (1 KB: lane l = 16*g + n holds row n of the tile, 16 bytes of reduction group g), so that every wavefront
 // load is one contiguous kilobyte, and stores the block scales of 256 reduction elements of the 16 rows as one
-// contiguous 256-byte piece.  It is a permutation of the same bytes: unpacking restores the planes bit for bit.
+// contiguous 256-byte piece.  It is a permutation of the same bytes (nibbles for Q4_1): unpacking restores the planes bit for bit.
 //
 //   Q8_0 / fp8 samples: qs_p[rt][K/64][64 lanes][16 B]   lane (n,g): row 16*rt+n, k = 64*kb + 16*g .. +15
-//   Q4_1 samples:       qs_p[rt][K/128][64 lanes][16 B]  lane (n,g): row 16*rt+n, k = 128*kb + 32*g .. +31 (one block)
+//   Q4_1 samples:       qs_p[rt][K/128][64 lanes][16 B]  lane (n,g): row 16*rt+n, k = 128*kb + 32*g .. +31 (one block);
+//                       inside every dword (8 elements) the even elements fill the low half-word and the odd ones the
+//                       high half-word (element 2p at bits 4p, 2p+1 at bits 16+4p): a pair comes out with one shift
+//                       and one and-or
 //   scales / offsets:   d_p[rt][K/256][16 rows][8] fp16  (8 consecutive blocks of one row)
 // with rt running over all E*rows/16 row tiles.  Requires rows % 16 == 0 and cols % 256 == 0.
 #include "weights.h"
@@ -35,8 +38,13 @@ repack_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n1
     const int64_t blk = i >> 4, cs = cols >> 8, rt = blk / cs, c = blk - rt * cs;
     planar = ((rt * 16 + n) * (cols >> 5) + c * 8) >> 3;
   }
-  if (DIR == 0) dst[i] = src[planar];
-  else dst[planar] = src[i];
+  uint4 v = DIR == 0 ? src[planar] : src[i];
+  if (KIND == 1) {  // nibbles of every dword: linear order <-> even elements low / odd elements high
+    if (DIR == 0) v = make_uint4(q4_dword_to_packed(v.x), q4_dword_to_packed(v.y), q4_dword_to_packed(v.z), q4_dword_to_packed(v.w));
+    else v = make_uint4(q4_dword_to_linear(v.x), q4_dword_to_linear(v.y), q4_dword_to_linear(v.z), q4_dword_to_linear(v.w));
+  }
+  if (DIR == 0) dst[i] = v;
+  else dst[planar] = v;
 }
 
 template <int KIND>

@@ -41,14 +41,9 @@ struct bf16_t { uint16_t bits; };
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
+  // v_cvt_pk_bf16_f32: round to nearest even, NaN stays a quiet NaN
   bf16_t r;
-  if ((u & 0x7fffffffu) > 0x7f800000u) {  // NaN: keep it quiet
-    r.bits = (uint16_t)((u >> 16) | 0x40u);
-    return r;
-  }
-  u += 0x7fffu + ((u >> 16) & 1u);
-  r.bits = (uint16_t)(u >> 16);
+  r.bits = __builtin_bit_cast(uint16_t, (__bf16)f);
   return r;
 }
 
@@ -80,16 +75,13 @@ template <typename T> __device__ __forceinline__ float round_to(float v) {
 }
 
 // ---- fp8 e4m3fn (OCP) ---------------------------------------------------------------------------
-__device__ __forceinline__ float fp8_e4m3fn_to_f32(uint8_t b) {
-  const uint32_t sign = (uint32_t)(b & 0x80u) << 24;
-  const uint32_t e = (b >> 3) & 0xfu;
-  const uint32_t mnt = b & 0x7u;
-  if (e == 0) {  // subnormal: mnt * 2^-9
-    float v = (float)mnt * 0.001953125f;
-    return __uint_as_float(__float_as_uint(v) | sign);
-  }
-  if (e == 0xf && mnt == 0x7) return __uint_as_float(0x7fc00000u | sign);  // NaN (no inf in e4m3fn)
-  return __uint_as_float(sign | ((e + 120u) << 23) | (mnt << 20));
+// gfx950 converts OCP e4m3fn in hardware (v_cvt_f32_fp8 / v_cvt_pk_f32_fp8); every e4m3fn value is exact in fp32.
+__device__ __forceinline__ float fp8_e4m3fn_to_f32(uint8_t b) { return __builtin_amdgcn_cvt_f32_fp8((int)b, 0); }
+// the four samples of one dword, lowest byte first
+__device__ __forceinline__ void fp8x4_to_f32(uint32_t u, float out[4]) {
+  typedef float float2_t __attribute__((ext_vector_type(2)));
+  const float2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)u, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)u, true);
+  out[0] = lo[0]; out[1] = lo[1]; out[2] = hi[0]; out[3] = hi[1];
 }
 
 // Round-to-nearest-even fp32 -> e4m3fn; magnitudes above 448 that round past it become NaN (0x7f),

@@ -51,7 +51,9 @@ template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi)
   return c.u;
 }
 template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) {
-  return (uint32_t)f32_to_bf16(lo).bits | ((uint32_t)f32_to_bf16(hi).bits << 16);
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  const bf16x2_t v = {(__bf16)lo, (__bf16)hi};  // one v_cvt_pk_bf16_f32 (round to nearest even)
+  return __builtin_bit_cast(uint32_t, v);
 }
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
@@ -70,6 +72,44 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
   union { uint16_t u; f16_t h; } c;
   c.u = (uint16_t)b;
   return (float)c.h;
+}
+
+// ---- Q4_1 helpers ------------------------------------------------------------------------------------
+// f16(f16(d*q) + m) for a pair of nibbles given as fp16 numbers 1024 + q (bits 0x6400 | q).  d*q is formed as
+// fma(1024 + q, d, -1024*d): the fma rounds the exact value d*q once, like the multiply of the reference.  -1024*d
+// must be finite for that, so scales of magnitude >= 32 take the subtract-then-multiply form.
+__device__ __forceinline__ uint32_t q4_pair_dequant(uint32_t pair_bits, uint32_t dbits, uint32_t mbits) {
+  const half2_t dd = as_half2(dbits | (dbits << 16)), mm = as_half2(mbits | (mbits << 16));
+  half2_t v;
+  if (__builtin_expect((dbits & 0x7fffu) >= 0x5000u, 0)) {
+    const half2_t bias = {(f16_t)1024.0f, (f16_t)1024.0f};
+    v = (as_half2(pair_bits) - bias) * dd;
+  } else {
+    const half2_t nb = as_half2((dbits | (dbits << 16)) ^ 0x80008000u) * (half2_t){(f16_t)1024.0f, (f16_t)1024.0f};
+    v = __builtin_elementwise_fma(as_half2(pair_bits), dd, nb);
+  }
+  return as_u32(v + mm);
+}
+// Pair p (elements 2p, 2p+1) of the 8 nibbles of a dword, as two fp16 numbers 1024 + q.
+//   linear order (planar planes): element i is nibble i
+//   packed order (written by stmoe_prepack): even elements in the low half-word, odd ones in the high half-word
+//   (element 2p at bits 4p, element 2p+1 at bits 16 + 4p), so one shift and one and-or extract a pair
+__device__ __forceinline__ uint32_t q4_pair_linear(uint32_t w, int p) {
+  const uint32_t byte = w >> (8 * p);
+  return 0x64006400u | (byte & 0xfu) | ((byte & 0xf0u) << 12);
+}
+__device__ __forceinline__ uint32_t q4_pair_packed(uint32_t w, int p) { return ((w >> (4 * p)) & 0x000f000fu) | 0x64006400u; }
+__device__ __forceinline__ uint32_t q4_dword_to_packed(uint32_t w) {
+  uint32_t out = 0;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) out |= (((w >> (8 * p)) & 0xfu) << (4 * p)) | (((w >> (8 * p + 4)) & 0xfu) << (16 + 4 * p));
+  return out;
+}
+__device__ __forceinline__ uint32_t q4_dword_to_linear(uint32_t w) {
+  uint32_t out = 0;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) out |= (((w >> (4 * p)) & 0xfu) << (8 * p)) | (((w >> (16 + 4 * p)) & 0xfu) << (8 * p + 4));
+  return out;
 }
 
 // Raw bytes of a 16-element chunk and its conversion.  `load` only issues the global loads (so a caller
@@ -127,25 +167,15 @@ template <> struct Chunk16<WF_Q4_1> {
   }
   __device__ __forceinline__ void zero() { q = make_uint2(0, 0); dbits = 0; mbits = 0; }
   // element 2i = low nibble of byte i, element 2i+1 = high nibble.  f16(f16(d*q) + m): two roundings.
-  __device__ __forceinline__ void to_f16x16(uint32_t out[8]) const {
+  template <bool PACKED = false> __device__ __forceinline__ void decode(uint32_t out[8]) const {
     const uint32_t r[2] = {q.x, q.y};
-    union { uint16_t u; f16_t h; } dc, mc;
-    dc.u = dbits;
-    mc.u = mbits;
-    const half2_t dd = {dc.h, dc.h}, mm = {mc.h, mc.h};
-    const half2_t bias = {(f16_t)1024.0f, (f16_t)1024.0f};
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const uint32_t byte = (r[i] >> (8 * b)) & 0xffu;
-        const uint32_t pair = 0x64006400u | (byte & 0xfu) | ((byte >> 4) << 16);
-        half2_t v = (as_half2(pair) - bias) * dd;
-        v = v + mm;
-        out[4 * i + b] = as_u32(v);
-      }
-    }
+      for (int b = 0; b < 4; ++b)
+        out[4 * i + b] = q4_pair_dequant(PACKED ? q4_pair_packed(r[i], b) : q4_pair_linear(r[i], b), dbits, mbits);
   }
+  __device__ __forceinline__ void to_f16x16(uint32_t out[8]) const { decode<false>(out); }
   __device__ __forceinline__ void to_f32(float out[16]) const {
     uint32_t h[8];
     to_f16x16(h);
@@ -170,10 +200,14 @@ template <bool F16D> struct Chunk16Fp8 {
   __device__ __forceinline__ void to_f32(float out[16]) const {
     const uint32_t r[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float v = fp8_e4m3fn_to_f32((uint8_t)(r[i >> 2] >> (8 * (i & 3))));
-      const float p = __fmul_rn(v, dv);
-      out[i] = F16D ? round_to<f16_t>(p) : p;
+    for (int j = 0; j < 4; ++j) {
+      float v[4];
+      fp8x4_to_f32(r[j], v);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = __fmul_rn(v[i], dv);
+        out[4 * j + i] = F16D ? round_to<f16_t>(p) : p;
+      }
     }
   }
 };
@@ -205,6 +239,16 @@ template <> struct Chunk16<WF_Q4_1_P> : Chunk16<WF_Q4_1> {
     const int64_t b = packed_scale(row, k0, w.cols);
     dbits = reinterpret_cast<const uint16_t*>(w.d)[b];
     mbits = reinterpret_cast<const uint16_t*>(w.m)[b];
+  }
+  __device__ __forceinline__ void to_f16x16(uint32_t out[8]) const { decode<true>(out); }
+  __device__ __forceinline__ void to_f32(float out[16]) const {
+    uint32_t h[8];
+    decode<true>(h);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      out[2 * i] = f16_bits_to_f32(h[i] & 0xffffu);
+      out[2 * i + 1] = f16_bits_to_f32(h[i] >> 16);
+    }
   }
 };
 template <> struct Chunk16<WF_FP8_F32D_P> : Chunk16Fp8<false> {

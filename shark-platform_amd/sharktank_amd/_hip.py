@@ -25,7 +25,7 @@ W_DENSE, W_Q8_0, W_Q4_1, W_FP8 = 0, 1, 2, 3
 W_Q8_0_PACKED, W_Q4_1_PACKED, W_FP8_PACKED = 4, 5, 6
 _PACKED_OF = {W_Q8_0: W_Q8_0_PACKED, W_Q4_1: W_Q4_1_PACKED, W_FP8: W_FP8_PACKED}
 # grouped_ffn variants
-VARIANT_AUTO, VARIANT_GENERIC, VARIANT_MFMA_TILE, VARIANT_SKINNY, VARIANT_MFMA_BIG = 0, 1, 2, 3, 4
+VARIANT_AUTO, VARIANT_GENERIC, VARIANT_MFMA_TILE, VARIANT_SKINNY, VARIANT_MFMA_BIG, VARIANT_FP8_MFMA = 0, 1, 2, 3, 4, 5
 
 _DTYPE_ENUM = {
     torch.float32: F32,
@@ -73,22 +73,24 @@ SIGNATURES = {
     "stmoe_prepack": (c_int, [POINTER(StmoeWeight), POINTER(StmoeWeight), c_void_p]),
     "stmoe_unpack": (c_int, [POINTER(StmoeWeight), POINTER(StmoeWeight), c_void_p]),
     "stmoe_quantize_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
+    "stmoe_fake_quant_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
     "stmoe_rms_norm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_float, c_void_p, c_void_p]),
     "stmoe_router_topk": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "stmoe_dispatch_build": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "stmoe_grouped_ffn_workspace_bytes": (c_size_t, [c_int64, c_int, c_int64, c_int64, c_int]),
     "stmoe_moe_forward_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int64, c_int64, c_int]),
     "stmoe_grouped_ffn": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, POINTER(StmoeWeight), POINTER(StmoeWeight),
-                                  POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+                                  POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int,
+                                  c_void_p]),
     "stmoe_grouped_mmt": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, POINTER(StmoeWeight), c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "stmoe_scale_rows": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "stmoe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int64, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p]),
     "stmoe_moe_forward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
-                                  POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
-                                  c_void_p, c_size_t, c_int, c_void_p]),
+                                  POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "stmoe_moe_forward_timed": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
                                         POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
-                                        c_void_p, c_size_t, c_int, c_void_p, POINTER(c_void_p)]),
+                                        c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p, POINTER(c_void_p)]),
     "stmoe_mmt": (c_int, [c_void_p, c_int, c_int64, POINTER(StmoeWeight), c_void_p, c_int, c_void_p]),
 }
 
@@ -243,11 +245,30 @@ def quantize_fp8(x: torch.Tensor, rscale: torch.Tensor) -> torch.Tensor:
     dev = _dev(x, rscale)
     lib = load_library()
     x_c = _contig(x)
-    rs = rscale.to(torch.float32).reshape(1)
+    rs = _scale1(rscale)
     out = torch.empty(x_c.shape, dtype=torch.float8_e4m3fn, device=dev)
     with torch.cuda.device(dev):
         _check(lib.stmoe_quantize_fp8(_ptr(x_c), dtype_enum(x_c.dtype), _ptr(rs), x_c.numel(), _ptr(out), _stream(dev)))
     return out
+
+
+def fake_quant_fp8(x: torch.Tensor, rscale: torch.Tensor) -> torch.Tensor:
+    """quantize(x).unpack().dequant() of a static per-tensor e4m3fn quantizer, in x's dtype."""
+    dev = _dev(x, rscale)
+    lib = load_library()
+    x_c = _contig(x)
+    rs = _scale1(rscale)
+    out = torch.empty_like(x_c)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_fake_quant_fp8(_ptr(x_c), dtype_enum(x_c.dtype), _ptr(rs), x_c.numel(), _ptr(out), _stream(dev)))
+    return out
+
+
+def _scale1(s: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """A reciprocal scale as one contiguous device fp32 value (None stays None)."""
+    if s is None:
+        return None
+    return s.to(torch.float32).reshape(1).contiguous()
 
 
 # ---- layer pieces -----------------------------------------------------------------------------------
@@ -359,8 +380,10 @@ def grouped_ffn_workspace_bytes(T: int, k: int, K: int, N: int, dtype: torch.dty
 
 
 def grouped_ffn(x, w_gate: DeviceWeight, w_up: DeviceWeight, w_down: DeviceWeight, act: int, offsets, perm, k: int,
-                *, variant: int = VARIANT_AUTO, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x [T,K] -> y_sorted [T*k, K] (rows in dispatch order)."""
+                *, variant: int = VARIANT_AUTO, workspace: Optional[torch.Tensor] = None,
+                x_scale: Optional[torch.Tensor] = None, z_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [T,K] -> y_sorted [T*k, K] (rows in dispatch order).  x_scale / z_scale: reciprocal scales of the static
+    e4m3fn quantizers of x and of the intermediate (None: not quantised)."""
     dev = _dev(x, offsets, perm)
     lib = load_library()
     x_c = _contig(x)
@@ -370,9 +393,10 @@ def grouped_ffn(x, w_gate: DeviceWeight, w_up: DeviceWeight, w_down: DeviceWeigh
     if workspace is None:
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
     y = torch.empty((T * k, K), dtype=x_c.dtype, device=dev)
+    xs, zs = _scale1(x_scale), _scale1(z_scale)
     with torch.cuda.device(dev):
         _check(lib.stmoe_grouped_ffn(_ptr(x_c), dtype_enum(x_c.dtype), T, K, N, E, k, w_gate.ref, w_up.ref, w_down.ref, act,
-                                     _ptr(offsets), _ptr(perm), None, _ptr(y), _ptr(workspace), workspace.numel(), variant,
+                                     _ptr(offsets), _ptr(perm), _ptr(xs), _ptr(zs), _ptr(y), _ptr(workspace), workspace.numel(), variant,
                                      _stream(dev)))
     return y
 
@@ -423,7 +447,8 @@ def moe_forward_workspace_bytes(T: int, k: int, E: int, K: int, N: int, dtype: t
 
 def moe_forward(h, ffn_norm_w, out_norm_w, eps: float, w_router, w_gate: DeviceWeight, w_up: DeviceWeight, w_down: DeviceWeight,
                 act: int, k: int, *, variant: int = VARIANT_AUTO, workspace: Optional[torch.Tensor] = None, want_routing: bool = False,
-                out: Optional[torch.Tensor] = None, events=None):
+                out: Optional[torch.Tensor] = None, events=None, x_scale: Optional[torch.Tensor] = None,
+                z_scale: Optional[torch.Tensor] = None):
     """h [T,K] -> out [T,K] (and, if asked, idx int32 [T,k] and gate [T,k]).  `events`: optional ctypes array of
     12 hipEvent_t handles that bracket the six stages (see stmoe_moe_forward_timed)."""
     dev = _dev(h, ffn_norm_w, out_norm_w, w_router)
@@ -438,9 +463,10 @@ def moe_forward(h, ffn_norm_w, out_norm_w, eps: float, w_router, w_gate: DeviceW
         out = torch.empty_like(h_c)
     idx = torch.empty((T, k), dtype=torch.int32, device=dev) if want_routing else None
     gate = torch.empty((T, k), dtype=h_c.dtype, device=dev) if want_routing else None
+    xs, zs = _scale1(x_scale), _scale1(z_scale)
     args = (_ptr(h_c), dtype_enum(h_c.dtype), T, K, N, E, k, _ptr(ffn_norm_w), _ptr(out_norm_w),
             dtype_enum(ffn_norm_w.dtype), float(eps), _ptr(w_router), w_gate.ref, w_up.ref, w_down.ref, act,
-            _ptr(out), _ptr(idx), _ptr(gate), _ptr(workspace), workspace.numel(), variant, _stream(dev))
+            _ptr(xs), _ptr(zs), _ptr(out), _ptr(idx), _ptr(gate), _ptr(workspace), workspace.numel(), variant, _stream(dev))
     with torch.cuda.device(dev):
         if events is None:
             _check(lib.stmoe_moe_forward(*args))

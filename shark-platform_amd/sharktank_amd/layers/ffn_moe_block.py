@@ -14,7 +14,7 @@ import torch.nn.functional as F
 from .. import _hip
 from .. import ops
 from ..ops import device_weight, gather_experts
-from ..types import Theta
+from ..types import StaticScaledQuantizer, Theta
 from .base import ThetaLayer
 
 __all__ = ["PreGatherFFNMOE", "activation_enum"]
@@ -36,6 +36,15 @@ class PreGatherFFNMOE(ThetaLayer):
         self.ffn_gate = theta.tensor("ffn_gate_exps", "weight")
         self.ffn_up = theta.tensor("ffn_up_exps", "weight")
         self.ffn_down = theta.tensor("ffn_down_exps", "weight")
+        # Optional static per-tensor fp8 quantizers of the activations, named as LinearLayer names its input quantizer
+        # (sharktank/sharktank/layers/linear.py:49): `ffn_gate_exps.q_input` quantises h for the gate and up
+        # projections, `ffn_down_exps.q_input` the gated intermediate for the down projection.  The values are the
+        # reference's quantise-then-dequantise ones (linear.py:72-78).
+        self.q_input = theta.optional_tensor("ffn_gate_exps", "q_input")
+        self.q_intermediate = theta.optional_tensor("ffn_down_exps", "q_input")
+        for q in (self.q_input, self.q_intermediate):
+            if q is not None and not isinstance(q, StaticScaledQuantizer):
+                raise NotImplementedError(f"PreGatherFFNMOE: activation quantizer {type(q).__name__} has no kernel")
         self.activation = activation
         self._act = activation_enum(activation)
         self._dw = None
@@ -63,11 +72,19 @@ class PreGatherFFNMOE(ThetaLayer):
         """The reference's forward written with the same `ops` calls, one kernel per einsum (ffn_moe_block.py:60-74).
         `forward` computes the same values with fused kernels; this path exists for callers that compose the ops."""
         act = {_hip.ACT_SILU: F.silu, _hip.ACT_GELU_ERF: F.gelu}[self._act]
+        if self.q_input is not None or self.q_intermediate is not None:
+            raise NotImplementedError("forward_unfused: activation quantizers are handled by forward only")
         ffn_gate = ops.elementwise(act, self.pre_matmul_gather(h, self.ffn_gate, experts))
         ffn_up = self.pre_matmul_gather(h, self.ffn_up, experts)
         ffn_down = self.pre_matmul_gather(ffn_gate * ffn_up, self.ffn_down, experts, einstring="mek,menk->men")
         ffn_down = ops.einsum_2args(expert_gate, ffn_down, "me,men->men")
         return torch.sum(ffn_down, dim=1)
+
+    def activation_scales(self):
+        """(reciprocal scale of the input quantizer, of the intermediate quantizer); None where there is none."""
+        xs = self.q_input.reciprocal_scale if self.q_input is not None else None
+        zs = self.q_intermediate.reciprocal_scale if self.q_intermediate is not None else None
+        return xs, zs
 
     @property
     def expert_count(self) -> int:
@@ -77,5 +94,6 @@ class PreGatherFFNMOE(ThetaLayer):
         wg, wu, wd = self.device_weights()
         T, k = experts.shape
         _, offsets, perm, inv = _hip.dispatch_build(experts, wg.experts)
-        y = _hip.grouped_ffn(h, wg, wu, wd, self._act, offsets, perm, k, variant=self.kernel_variant)
+        xs, zs = self.activation_scales()
+        y = _hip.grouped_ffn(h, wg, wu, wd, self._act, offsets, perm, k, variant=self.kernel_variant, x_scale=xs, z_scale=zs)
         return _hip.combine(y, expert_gate.to(h.dtype), inv, T, k)

@@ -61,10 +61,12 @@ class MoeBlock(ThetaLayer):
         need = _hip.moe_forward_workspace_bytes(T, self.expert_used_count, self.expert_count, feature_dim, wg.rows, h.dtype)
         if self._workspace is None or self._workspace.numel() < need or self._workspace.device != h.device:
             self._workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=h.device)
+        xs, zs = self.experts.activation_scales()
         res = _hip.moe_forward(
             x, unbox_tensor(self.ffn_norm.weight), out_norm_w, self.rms_epsilon, self._router_weight(h.dtype),
             wg, wu, wd, self.experts._act, self.expert_used_count,
             variant=self.experts.kernel_variant, workspace=self._workspace, want_routing=return_routing,
+            x_scale=xs, z_scale=zs,
         )
         if return_routing:
             out, idx, gate = res

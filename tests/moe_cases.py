@@ -26,6 +26,7 @@ class Case:
     seed: int = 0
     eps: float = 1e-5
     out_norm: bool = False
+    act_quant: bool = False  # static per-tensor e4m3fn quantizers on the FFN input and on the gated intermediate
     router_bias: Optional[torch.Tensor] = None  # added to the router rows' effect via a skewed input direction
     planes: dict = field(default_factory=dict)
 
@@ -78,6 +79,14 @@ def build(case: Case, dense_dtype: Optional[torch.dtype] = None) -> Case:
     case.planes["ffn_norm"] = torch.ones(K) + 0.1 * torch.randn(K, generator=g)
     case.planes["out_norm"] = (torch.ones(K) + 0.1 * torch.randn(K, generator=g)) if case.out_norm else None
     case.planes["h"] = torch.randn(case.T, K, generator=g).to(case.dtype)
+    case.planes["x_rscale"] = case.planes["z_rscale"] = None
+    if case.act_quant:
+        # calibrate as a static quantizer would be: amax over a sample of the unquantised activations, 448 = e4m3fn max
+        xn = O.rms_norm(case.planes["h"][:16], case.planes["ffn_norm"], case.eps)
+        wg, wu, _ = dense_weights(case)
+        z = case.activation(O._mm_rt(xn, wg[0])) * O._mm_rt(xn, wu[0])
+        case.planes["x_rscale"] = (xn.float().abs().amax() * 1.25 / 448.0).to(torch.float32)
+        case.planes["z_rscale"] = (z.float().abs().amax() * 2.0 / 448.0).to(torch.float32)
     return case
 
 
@@ -117,6 +126,10 @@ def make_theta(case: Case, device):
         "ffn_up_exps.weight": to_inference_tensor(case.fmt, case.planes["up"], [E, N, K], "ffn_up_exps.weight", device),
         "ffn_down_exps.weight": to_inference_tensor(case.fmt, case.planes["down"], [E, K, N], "ffn_down_exps.weight", device),
     }
+    if case.act_quant:
+        for key, rs in (("ffn_gate_exps.q_input", case.planes["x_rscale"]), ("ffn_down_exps.q_input", case.planes["z_rscale"])):
+            tensors[key] = ST.StaticScaledQuantizer(name=key, scale=(1.0 / rs).to(device), reciprocal_scale=rs.to(device),
+                                                    dtype=torch.float8_e4m3fn)
     if case.planes["out_norm"] is not None:
         tensors["layer_output_norm.weight"] = ST.DefaultPrimitiveTensor(
             name="layer_output_norm.weight", data=case.planes["out_norm"].to(device))
@@ -128,4 +141,5 @@ def oracle_block(case: Case, formulation: str = "grouped", ordered_logits: bool 
     return O.moe_block(
         case.planes["h"], case.planes["ffn_norm"], case.planes["router"], wg, wu, wd, case.k, case.eps,
         case.activation, out_norm_w=case.planes["out_norm"], formulation=formulation, ordered_logits=ordered_logits,
+        x_rscale=case.planes["x_rscale"], z_rscale=case.planes["z_rscale"],
     )

@@ -50,10 +50,10 @@ def test_argument_validation_without_a_gpu():
     assert lib.stmoe_router_topk(None, None, _hip.F16, 0, 64, 8, 2, None, None, None, None, None) == 0  # zero tokens
     assert lib.stmoe_dispatch_build(None, 0, 0, None, None, None, None, None) == 2
     assert lib.stmoe_dequant_block_scaled(None, None, _hip.F16, None, 0, 32, None, _hip.F16, None) == 0
-    assert lib.stmoe_grouped_ffn_workspace_bytes(32, 2, 4096, 14336, _hip.F16) == 32 * 2 * 14336 * 2
+    assert lib.stmoe_grouped_ffn_workspace_bytes(32, 2, 4096, 14336, _hip.F16) == 32 * 2 * 14336 * 2 + 32 * 4096 * 2 + 32 * 2 * 14336  # z, copy of x, fp8 z
     w = _hip.StmoeWeight(format=_hip.W_Q8_0, dtype=0, experts=8, rows=64, cols=48, qs=16, d=16, m=None, d_count=1)
     rc = lib.stmoe_grouped_ffn(None, _hip.F16, 4, 48, 64, 8, 2, ctypes.byref(w), ctypes.byref(w), ctypes.byref(w), 0,
-                               None, None, None, None, None, 0, 0, None)
+                               None, None, None, None, None, None, 0, 0, None)
     assert rc == 2 and b"32" in lib.stmoe_last_error()  # Q8_0 needs cols % 32 == 0
 
 

@@ -18,7 +18,8 @@ import moe_cases as MC
 pytestmark = pytest.mark.gpu
 
 
-def build_device_case(device, T, K, N, fmt, dtype, act="silu", seed=0, E=8, k=2, out_norm=False, router_skew=None):
+def build_device_case(device, T, K, N, fmt, dtype, act="silu", seed=0, E=8, k=2, out_norm=False, router_skew=None,
+                      act_quant=False):
     """Weights N(0, 0.02) generated and quantized on the device (data generation only); returns (theta, pieces)."""
     from sharktank_amd import types as ST
 
@@ -57,8 +58,23 @@ def build_device_case(device, T, K, N, fmt, dtype, act="silu", seed=0, E=8, k=2,
     tensors["ffn_norm.weight"] = ST.DefaultPrimitiveTensor(name="ffn_norm.weight", data=ffn_norm.to(device))
     if out_norm_w is not None:
         tensors["layer_output_norm.weight"] = ST.DefaultPrimitiveTensor(name="layer_output_norm.weight", data=out_norm_w.to(device))
+    act_fn = F.silu if act == "silu" else F.gelu
+    x_rscale = z_rscale = None
+    if act_quant:
+        # static e4m3fn quantizers calibrated on a sample: 8 tokens through expert 0, with head-room
+        xn = O.rms_norm(h[:8], ffn_norm, 1e-5)
+        dense0 = {}
+        for name, shape in (("gate", [N, K]), ("up", [N, K])):
+            pe = {kk: (v[0].cpu() if v.dim() > 0 and v.shape[0] == E else v.cpu()) for kk, v in planes[name].items()}
+            dense0[name] = MC.dense_from_planes(fmt, pe, shape, dtype)
+        z = act_fn(O._mm_rt(xn, dense0["gate"])) * O._mm_rt(xn, dense0["up"])
+        x_rscale = (xn.float().abs().amax() * 1.25 / 448.0).to(torch.float32)
+        z_rscale = (z.float().abs().amax() * 2.0 / 448.0).to(torch.float32)
+        for key, rs in (("ffn_gate_exps.q_input", x_rscale), ("ffn_down_exps.q_input", z_rscale)):
+            tensors[key] = ST.StaticScaledQuantizer(name=key, scale=(1.0 / rs).to(device), reciprocal_scale=rs.to(device),
+                                                    dtype=torch.float8_e4m3fn)
     return ST.Theta(tensors), dict(planes=planes, router=router, ffn_norm=ffn_norm, out_norm=out_norm_w, h=h, fmt=fmt,
-                                   dtype=dtype, act=F.silu if act == "silu" else F.gelu, E=E, k=k, K=K, N=N, T=T)
+                                   dtype=dtype, act=act_fn, E=E, k=k, K=K, N=N, T=T, x_rscale=x_rscale, z_rscale=z_rscale)
 
 
 def oracle_rows(pc, rows, eps=1e-5):
@@ -82,9 +98,14 @@ def oracle_rows(pc, rows, eps=1e-5):
         for j in range(pc["k"]):
             e = int(idx[t, j])
             xt = x[t : t + 1]
+            if pc.get("x_rscale") is not None:
+                xt = O.fake_quant_per_tensor(xt, pc["x_rscale"])
             a = pc["act"](O._mm_rt(xt, dense["gate"][e]))
             u = O._mm_rt(xt, dense["up"][e])
-            dn = O._mm_rt(a * u, dense["down"][e])
+            z = a * u
+            if pc.get("z_rscale") is not None:
+                z = O.fake_quant_per_tensor(z, pc["z_rscale"])
+            dn = O._mm_rt(z, dense["down"][e])
             acc.append(gate[t, j] * dn)
         o = torch.sum(torch.stack(acc, dim=1), dim=1)
         if pc["out_norm"] is not None:
@@ -172,10 +193,26 @@ def test_config4_grok_q4_1_gelu_skewed_routing(device):
 
 def test_config5_mixtral_fp8_weights(device):
     """fp8 e4m3 per-tensor-scaled expert weights, uniform routing is not forced (the router decides); 4096-token prefill
-    and a 1-token decode.  Activations stay fp16 (fp8 activation quantisation has no kernel yet)."""
+    and a 1-token decode.  Activations stay fp16 here; the next test quantises them too."""
     theta, pc = build_device_case(device, 4096, 4096, 14336, "fp8", torch.float16, seed=5)
     y, idx, gate, block = run_layer(theta, pc, device)
     check_against_oracle(y, idx, pc, [0, 2047, 4095], 2e-2)
     y1, idx1, _ = block(pc["h"][:1].reshape(1, 1, 4096).to(device), return_routing=True)
     assert torch.equal(idx1.cpu(), idx.cpu()[:1])
     assert O.rel_l2(y1.reshape(1, 4096).cpu(), y[:1].cpu()) < 1e-3
+
+
+def test_config5_mixtral_fp8_weights_and_activations(device):
+    """Config 5 with static e4m3fn quantizers on the FFN input and on the gated intermediate: the 4096-token prefill
+    runs both operands on the fp8 matrix cores, the 1-token decode re-dequantises and streams the weights.  Both are
+    held to the fp8 tolerance against the reference's quantise-dequantise-then-multiply arithmetic."""
+    theta, pc = build_device_case(device, 4096, 4096, 14336, "fp8", torch.float16, seed=5, act_quant=True)
+    y, idx, gate, block = run_layer(theta, pc, device)
+    check_against_oracle(y, idx, pc, [0, 2047, 4095], 2e-2)
+    y1, idx1, _ = block(pc["h"][:1].reshape(1, 1, 4096).to(device), return_routing=True)
+    assert torch.equal(idx1.cpu(), idx.cpu()[:1])
+    want1, _, _ = oracle_rows(pc, [0])
+    assert O.rel_l2(y1.reshape(1, 4096).cpu(), want1) < 1e-3  # the decode path follows the reference's arithmetic
+    # run-to-run bit identity of the matrix-core path
+    y2, _, _, _ = run_layer(theta, pc, device)
+    assert torch.equal(y2, y)

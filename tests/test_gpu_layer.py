@@ -62,6 +62,59 @@ def test_small_quantized_layers(device, fmt, dtype):
     check_case(case, device)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T", [1, 24, 200, 700])
+def test_fp8_weights_and_fp8_activations(device, dtype, T):
+    """fp8 tensor-scaled weights with static fp8 quantizers on the FFN input and the gated intermediate.  Up to 32
+    tokens the re-dequantised activations go through the streaming kernel (the reference's own arithmetic); above,
+    both operands run on the fp8 matrix cores and the dot product is scaled once.  That path skips the rounding of the
+    dequantised samples to the activation dtype (2^-11 relative for fp16, 2^-8 for bf16, on both operands), so the
+    MoE contribution alone, without the residual, differs from the dequantise-first arithmetic by about 1e-2 (fp16)
+    and 4e-2 (bf16); the layer output is held to the 2e-2 tolerance of the fp8 configuration."""
+    case = MC.Case(T=T, K=512, N=768, fmt="fp8", dtype=dtype, act_quant=True, seed=40 + T)
+    err, err_y = check_case(case, device, tol=2e-2)
+    if T <= 32:
+        assert err < 1e-3, f"MoE contribution rel-L2 {err:.3e} on the dequantise-first path"
+    else:
+        assert err < (2e-2 if dtype == torch.float16 else 6e-2), f"MoE contribution rel-L2 {err:.3e}"
+
+
+def test_fp8_matrix_core_path_is_exact_up_to_dequant_rounding(device):
+    """With activations that are exactly representable after quantisation (integers times the scale) and power-of-two
+    scales, scaling the fp32 dot product once equals dequantise-then-multiply: the fp8 path must then agree with the
+    16-bit path to the rounding of the result only."""
+    from sharktank_amd import _hip
+    from sharktank_amd.ops import device_weight
+    import sharktank_amd.types as ST
+
+    g = torch.Generator().manual_seed(3)
+    T, K, N, E, k = 256, 256, 512, 4, 2
+    def w8(shape):
+        q = torch.randint(-8, 9, shape, generator=g).float()
+        return q.to(torch.float8_e4m3fn)
+    planes = {n: w8(s) for n, s in (("gate", (E, N, K)), ("up", (E, N, K)), ("down", (E, K, N)))}
+    d = torch.tensor(2.0 ** -6)
+    x = (torch.randint(-6, 7, (T, K), generator=g).float() * 0.25).to(torch.float16)
+    experts = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    dw = [device_weight(ST.PlanarQuantizedTensor(name=n, shape=list(q.shape),
+                                                 layout=ST.TensorScaledLayout(shape=list(q.shape), d=d.to(device), qs=q.to(device))),
+                        stacked=True, prepack=pp)
+          for (n, q), pp in zip(planes.items(), (True, True, False))]
+    _, offsets, perm, inv = _hip.dispatch_build(experts.to(device), E)
+    xs = torch.tensor(0.25)
+    zs = torch.tensor(2.0 ** -4)
+    got = _hip.grouped_ffn(x.to(device), *dw, _hip.ACT_SILU, offsets, perm, k, variant=_hip.VARIANT_FP8_MFMA,
+                           x_scale=xs.to(device), z_scale=zs.to(device)).cpu()
+    dense = [O.dequant_tensor_scaled(d, q).to(torch.float16) for q in planes.values()]
+    want_pairs = torch.zeros(T * k, K, dtype=torch.float16)
+    xq = O.fake_quant_per_tensor(x, xs)
+    for p_sorted, pair in enumerate(perm.cpu().tolist()):
+        t, e = pair // k, int(experts.reshape(-1)[pair])
+        z = F.silu(O._mm_rt(xq[t:t + 1], dense[0][e])) * O._mm_rt(xq[t:t + 1], dense[1][e])
+        want_pairs[p_sorted] = O._mm_rt(O.fake_quant_per_tensor(z, zs), dense[2][e])[0]
+    assert O.rel_l2(got, want_pairs) < 1e-3
+
+
 def test_gelu_and_output_norm(device):
     """Grok-style block: exact-erf GELU and a layer_output_norm (sharktank/sharktank/models/grok/grok.py:102-109)."""
     case = MC.Case(T=80, K=384, N=512, fmt="q4_1", dtype=torch.float16, act="gelu", out_norm=True, seed=22)

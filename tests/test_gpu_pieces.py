@@ -83,6 +83,17 @@ def test_quantize_fp8_bit_exact(device, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_fake_quant_fp8_bit_exact(device, dtype):
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(4096, generator=g) * 3).to(dtype)
+    x[:4] = torch.tensor([1000.0, -1000.0, 0.0, 448.0]).to(dtype)
+    rscale = torch.tensor(0.0118, dtype=torch.float32)
+    want = O.fake_quant_per_tensor(x, rscale)
+    got = _hip().fake_quant_fp8(x.to(device), rscale.to(device)).cpu()
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_rms_norm(device, dtype):
     g = torch.Generator().manual_seed(4)
     x = torch.randn(37, 1024, generator=g).to(dtype)

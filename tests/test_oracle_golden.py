@@ -145,6 +145,20 @@ def test_quark_fp8_vector():  # :172-244
     assert torch.equal(qs_fn.view(torch.int8), torch.tensor(QUARK_FP8, dtype=torch.int8))
 
 
+def test_fake_quant_is_quantize_then_dequant_and_idempotent():
+    """fake_quant_per_tensor on the quark vector gives the vector back (its samples are e4m3fn values times the scale),
+    applying it twice changes nothing, and values beyond 448 * scale saturate."""
+    scale = torch.tensor(0.0118, dtype=torch.float32)
+    orig = torch.tensor(QUARK_FP8[:-2], dtype=torch.int8).view(torch.float8_e4m3fn)  # drop the NaN / -0 patterns
+    x = (orig.to(torch.float32) * scale).to(torch.float16)
+    fq = O.fake_quant_per_tensor(x, scale)
+    torch.testing.assert_close(fq, x, atol=1e-3, rtol=1e-3)
+    assert torch.equal(O.fake_quant_per_tensor(fq, scale), fq)
+    big = torch.tensor([100.0, -100.0], dtype=torch.float16)
+    assert O.fake_quant_per_tensor(big, scale).tolist() == [(torch.tensor(448.0) * scale).to(torch.float16).item()] * 1 + [
+        (torch.tensor(-448.0) * scale).to(torch.float16).item()]
+
+
 # ---- GGUF raw blocks: struct layouts quoted at sharktank/sharktank/types/gguf_interop/layouts.py:33-39,263-270 --
 def test_q8_0_unpack_hand_assembled_block():
     d = np.float16(0.25)
