@@ -205,10 +205,15 @@ template <int WF> struct SkinnyX {
 };
 
 // One pass of one work item: rows [r0, min(r0 + 16*MT, re)) of expert rows against the item's two weight tiles.
-template <typename T, int WF, int MODE, int MT>
+// KS > 1: the KS wavefronts of a workgroup share the item, each takes a contiguous 1/KS of the chunks, and the partial
+// sums are added through LDS in a fixed order ((w0 + w1) + (w2 + w3)) by wavefront 0, which then writes the result.
+template <typename T, int WF, int MODE, int MT, int KS>
 __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (&wrow)[2], int tile, int r0, int re,
-                                            int64_t nch, int lane) {
+                                            int64_t nch_total, int lane) {
   constexpr int NT = 2;
+  const int kw = KS > 1 ? (int)(threadIdx.x >> 6) : 0;
+  const int64_t c_begin = KS > 1 ? nch_total * kw / KS : 0;
+  const int64_t nch = KS > 1 ? nch_total * (kw + 1) / KS : nch_total;  // end of this wavefront's chunk range
   const int g = lane >> 4, n_in = lane & 15;
   const uint16_t* xrow[MT];
   bool xok[MT];
@@ -253,17 +258,19 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
   };
 
   if constexpr (XDB) {
-    load_w(w0, 0);
-    load_x(x0, 0);
-    for (int64_t c = 0; c < nch; c += 2) {
+    if (c_begin < nch) {
+      load_w(w0, c_begin);
+      load_x(x0, c_begin);
+    }
+    for (int64_t c = c_begin; c < nch; c += 2) {
       if (c + 1 < nch) { load_w(w1, c + 1); load_x(x1, c + 1); }
       compute(w0, x0);
       if (c + 2 < nch) { load_w(w0, c + 2); load_x(x0, c + 2); }
       if (c + 1 < nch) compute(w1, x1);
     }
   } else {
-    load_w(w0, 0);
-    for (int64_t c = 0; c < nch; c += 2) {
+    if (c_begin < nch) load_w(w0, c_begin);
+    for (int64_t c = c_begin; c < nch; c += 2) {
       load_x(x0, c);
       if (c + 1 < nch) load_w(w1, c + 1);
       compute(w0, x0);
@@ -273,6 +280,28 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
         compute(w1, x0);
       }
     }
+  }
+
+  if constexpr (KS > 1) {
+    __shared__ floatx4_t red[KS][MT * NT][64];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) red[kw][mt * NT + t][lane] = acc[mt][t];
+    __syncthreads();
+    if (kw == 0) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          floatx4_t sum = red[0][mt * NT + t][lane] + red[1][mt * NT + t][lane];
+#pragma unroll
+          for (int w = 2; w < KS; w += 2) sum = sum + (red[w][mt * NT + t][lane] + red[w + 1][mt * NT + t][lane]);
+          acc[mt][t] = sum;
+        }
+    }
+    __syncthreads();  // the buffer is reused by the next pass
+    if (kw != 0) return;
   }
 
 #pragma unroll
@@ -298,12 +327,14 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
 // Workgroups resident per CU (two wavefronts per SIMD: the double-buffered chunks need about 200 registers).
 template <int WF> struct SkinnyOcc { static constexpr int value = 2; };
 
-template <typename T, int WF, int MODE>
+// KS == 1: `total_workers` wavefronts, one item each at a time.  KS == 4: `total_workers` workgroups, the four
+// wavefronts of a workgroup split the reduction of one item (for launches with too few items to fill the chip).
+template <typename T, int WF, int MODE, int KS>
 __global__ void __launch_bounds__(256, SkinnyOcc<WF>::value)
 grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
   const int lane = threadIdx.x & 63;
   const int n_in = lane & 15;
-  const int wave_global = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int wave_global = KS > 1 ? (int)blockIdx.x : (int)(blockIdx.x * 4 + (threadIdx.x >> 6));
   const int64_t nch = p.kred >> 8;
 
   // experts that received rows, in increasing id
@@ -340,9 +371,9 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
     }
     // up to 16 rows: one 16-row token tile; otherwise passes of two tiles (one pass up to 32 rows)
     if (re - rb <= 16) {
-      skinny_pass<T, WF, MODE, 1>(p, wrow, tile, rb, re, nch, lane);
+      skinny_pass<T, WF, MODE, 1, KS>(p, wrow, tile, rb, re, nch, lane);
     } else {
-      for (int r0 = rb; r0 < re; r0 += 32) skinny_pass<T, WF, MODE, 2>(p, wrow, tile, r0, re, nch, lane);
+      for (int r0 = rb; r0 < re; r0 += 32) skinny_pass<T, WF, MODE, 2, KS>(p, wrow, tile, r0, re, nch, lane);
     }
   }
 }
@@ -357,12 +388,22 @@ static int pick_waves(int64_t items, int wg_per_cu) {
 }
 
 template <typename T, int WF>
-static int launch_skinny_t(int mode, const GemmParams& p, int64_t, hipStream_t st) {
+static int launch_skinny_t(int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   const int tiles = (int)(mode == MODE_GATEUP ? p.n_out / 16 : p.n_out / 32);
+  // at most min(E, rows) experts receive rows; with so few items that four wavefronts per item still fit the chip,
+  // a workgroup shares each item and splits its reduction
+  const int64_t active_bound = max_rows < p.E ? max_rows : p.E;
+  const int64_t items_bound = active_bound * tiles;
+  if (items_bound * 4 <= 1024 * SkinnyOcc<WF>::value && (p.kred >> 8) >= 4) {
+    dim3 grid((unsigned)items_bound);
+    if (mode == MODE_GATEUP) grouped_skinny_kernel<T, WF, MODE_GATEUP, 4><<<grid, 256, 0, st>>>(p, tiles, (int)items_bound);
+    else grouped_skinny_kernel<T, WF, MODE_DOWN, 4><<<grid, 256, 0, st>>>(p, tiles, (int)items_bound);
+    return check_launch("grouped_skinny(split)");
+  }
   const int waves = pick_waves((int64_t)tiles * p.E, SkinnyOcc<WF>::value);
   dim3 grid((unsigned)(waves / 4));
-  if (mode == MODE_GATEUP) grouped_skinny_kernel<T, WF, MODE_GATEUP><<<grid, 256, 0, st>>>(p, tiles, waves);
-  else grouped_skinny_kernel<T, WF, MODE_DOWN><<<grid, 256, 0, st>>>(p, tiles, waves);
+  if (mode == MODE_GATEUP) grouped_skinny_kernel<T, WF, MODE_GATEUP, 1><<<grid, 256, 0, st>>>(p, tiles, waves);
+  else grouped_skinny_kernel<T, WF, MODE_DOWN, 1><<<grid, 256, 0, st>>>(p, tiles, waves);
   return check_launch("grouped_skinny");
 }
 
@@ -372,27 +413,26 @@ int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_
   if (p.kred % 256 != 0 || p.n_out % 32 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0)
     return set_error(STMOE_ERR_UNSUPPORTED, "skinny kernel: needs K %% 256 == 0 and N %% 32 == 0");
   if (max_rows == 0) return STMOE_OK;
-  const int64_t per_expert = p.expert_rows_bound > 0 ? p.expert_rows_bound : max_rows;
-  if (act_dtype == STMOE_F16) {
+    if (act_dtype == STMOE_F16) {
     switch (wtag) {
-      case WF_Q8_0: return launch_skinny_t<f16_t, WF_Q8_0>(mode, p, per_expert, st);
-      case WF_Q4_1: return launch_skinny_t<f16_t, WF_Q4_1>(mode, p, per_expert, st);
-      case WF_FP8_F32D: return launch_skinny_t<f16_t, WF_FP8_F32D>(mode, p, per_expert, st);
-      case WF_DENSE_F16: return launch_skinny_t<f16_t, WF_DENSE_F16>(mode, p, per_expert, st);
-      case WF_Q8_0_P: return launch_skinny_t<f16_t, WF_Q8_0_P>(mode, p, per_expert, st);
-      case WF_Q4_1_P: return launch_skinny_t<f16_t, WF_Q4_1_P>(mode, p, per_expert, st);
-      case WF_FP8_F32D_P: return launch_skinny_t<f16_t, WF_FP8_F32D_P>(mode, p, per_expert, st);
+      case WF_Q8_0: return launch_skinny_t<f16_t, WF_Q8_0>(mode, p, max_rows, st);
+      case WF_Q4_1: return launch_skinny_t<f16_t, WF_Q4_1>(mode, p, max_rows, st);
+      case WF_FP8_F32D: return launch_skinny_t<f16_t, WF_FP8_F32D>(mode, p, max_rows, st);
+      case WF_DENSE_F16: return launch_skinny_t<f16_t, WF_DENSE_F16>(mode, p, max_rows, st);
+      case WF_Q8_0_P: return launch_skinny_t<f16_t, WF_Q8_0_P>(mode, p, max_rows, st);
+      case WF_Q4_1_P: return launch_skinny_t<f16_t, WF_Q4_1_P>(mode, p, max_rows, st);
+      case WF_FP8_F32D_P: return launch_skinny_t<f16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
       default: break;
     }
   } else if (act_dtype == STMOE_BF16) {
     switch (wtag) {
-      case WF_Q8_0: return launch_skinny_t<bf16_t, WF_Q8_0>(mode, p, per_expert, st);
-      case WF_Q4_1: return launch_skinny_t<bf16_t, WF_Q4_1>(mode, p, per_expert, st);
-      case WF_FP8_F32D: return launch_skinny_t<bf16_t, WF_FP8_F32D>(mode, p, per_expert, st);
-      case WF_DENSE_BF16: return launch_skinny_t<bf16_t, WF_DENSE_BF16>(mode, p, per_expert, st);
-      case WF_Q8_0_P: return launch_skinny_t<bf16_t, WF_Q8_0_P>(mode, p, per_expert, st);
-      case WF_Q4_1_P: return launch_skinny_t<bf16_t, WF_Q4_1_P>(mode, p, per_expert, st);
-      case WF_FP8_F32D_P: return launch_skinny_t<bf16_t, WF_FP8_F32D_P>(mode, p, per_expert, st);
+      case WF_Q8_0: return launch_skinny_t<bf16_t, WF_Q8_0>(mode, p, max_rows, st);
+      case WF_Q4_1: return launch_skinny_t<bf16_t, WF_Q4_1>(mode, p, max_rows, st);
+      case WF_FP8_F32D: return launch_skinny_t<bf16_t, WF_FP8_F32D>(mode, p, max_rows, st);
+      case WF_DENSE_BF16: return launch_skinny_t<bf16_t, WF_DENSE_BF16>(mode, p, max_rows, st);
+      case WF_Q8_0_P: return launch_skinny_t<bf16_t, WF_Q8_0_P>(mode, p, max_rows, st);
+      case WF_Q4_1_P: return launch_skinny_t<bf16_t, WF_Q4_1_P>(mode, p, max_rows, st);
+      case WF_FP8_F32D_P: return launch_skinny_t<bf16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
       default: break;
     }
   }
