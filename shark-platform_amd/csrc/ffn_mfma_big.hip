@@ -1,18 +1,27 @@
 // Prefill kernel: grouped projection on the matrix cores with a 256 x 256 workgroup tile.
 //
-//   workgroup = 4 wavefronts (2 x 2), each owning 128 weight rows x 128 token rows of the tile
-//               (GATEUP: 64 gate rows + the same 64 up rows, so the gated product is formed in registers)
-//   K step 64, two LDS stages (weights and tokens as 16-bit values, row stride 72 elements so that the
-//   16-byte operand reads of 16 consecutive rows fall into distinct banks), one barrier per K step
-//   producer: every wavefront loads whole 1 KB pieces of the packed weight order (prepack.hip), dequantises
-//             them in registers and writes 16-bit rows into the next LDS stage; token rows are gathered
-//             through the dispatch permutation with 128-byte row segments per 8 lanes
+//   workgroup = 8 wavefronts (2 x 4), each owning 128 weight rows x 64 token rows of the tile
+//               (GATEUP: 64 gate rows + the same 64 up rows, so the gated product is formed in registers);
+//               the 256 x 256 fp32 accumulators are half of the CU's register file, the largest tile that fits
+//   K step 64.  LDS (160 KB): two stages of dequantised weights (16-bit, 32 KB each) and three stages of token rows
+//               (32 KB each); rows are 128 bytes, XOR-swizzled in 16-byte units, one barrier per K step
+//   producer: every wavefront loads whole 1 KB pieces of the packed weight order (prepack.hip) into registers two
+//             K steps ahead, dequantises them and writes 16-bit rows into the next weight stage; token rows,
+//             gathered through the dispatch permutation, go from global memory straight into LDS
+//             (global_load_lds_dwordx4), also two K steps ahead, without passing through registers
 //   consumer: v_mfma_f32_16x16x32, weight rows as the "A" rows, token rows as the "B" columns; per K=32 step a
-//             wavefront reads 8 + 8 operand fragments from LDS for 64 MFMAs, i.e. half the LDS bytes per flop
-//             of a 64 x 64 wavefront tile
-//   ragged tiles: MFMAs of 16-token groups past the end of the expert's rows are skipped
+//             wavefront reads 8 + 4 operand fragments from LDS for 32 MFMAs
+//   the two wavefronts of a SIMD run producer and consumer halves of a K step in opposite orders, so that one
+//             converts and stores while the other feeds the matrix pipe
+//   ragged tiles: wavefronts whose 64 token rows are all past the end of the expert's rows skip their MFMAs
 //   scheduling: workgroup ids are remapped so that consecutive logical tiles run on the same XCD (one L2),
 //               with the token tiles of one (expert, feature tile) adjacent so they share its weights in L2.
+//
+// The direct loads are written as inline assembly: given the builtin, the compiler waits for every outstanding load
+// before each LDS read, which would undo the prefetch.  Their completion is therefore awaited by hand before the
+// barrier of the K step that precedes their use (s_waitcnt vmcnt(n): loads return in issue order, and per K step a
+// wavefront issues XPIECES token loads followed by WLOADS weight loads, one 16-byte and one 2-byte load per piece).
+// The compiler's own waits for the weight registers do not count the hidden token loads and can only be stricter.
 #include "ffn_kernels.h"
 
 namespace stmoe {
@@ -39,14 +48,22 @@ static constexpr int BIG_LS = BIG_BK;  // LDS row stride (elements): 128 bytes =
 // distinct 16-byte bank groups for the operand reads, the weight-row writes and the token-row writes alike.
 __device__ __forceinline__ int lds_off(int row, int unit) { return row * BIG_LS + ((unit ^ (row & 7)) << 3); }
 
+// ---- hand-issued vector-memory operations ------------------------------------------------------------
+// Lane l's 16 bytes at base + byte_off land at LDS byte address lds_addr + 16*l (base and lds_addr wave-uniform).
+__device__ __forceinline__ void vm_load16_to_lds(const void* base, uint32_t byte_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(byte_off), "s"(base), "s"(lds_addr)
+               : "memory", "m0");
+}
+template <int N> __device__ __forceinline__ void vm_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
 // One packed 1 KB piece (16 rows x 64 k of 1-byte samples, or 16 rows x 128 k of nibbles) as held by one lane.
 template <int WF> struct BigPiece;
 template <> struct BigPiece<WF_Q8_0_P> {
   u32x4_t q;
-  uint32_t dsel;  // the lane's block scale, duplicated into both halves
+  uint32_t d;  // the lane's block scale (fp16 bits, zero-extended)
   // 16 values of T: row n = lane%16, k = 16*g .. 16*g+15 of the 64-wide K step
   template <typename T> __device__ __forceinline__ void convert(uint32_t out[8]) const {
-    const half2_t dd = as_half2(dsel);
+    const half2_t dd = as_half2(d | (d << 16));
     const half2_t bias = {(f16_t)1152.0f, (f16_t)1152.0f};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -65,6 +82,7 @@ template <> struct BigPiece<WF_Q8_0_P> {
   }
 };
 
+template <int V> struct BigSet { static constexpr int value = V; };
 struct BigTagOn { static constexpr bool value = true; };
 struct BigTagOff { static constexpr bool value = false; };
 
@@ -72,12 +90,13 @@ struct BigTagOff { static constexpr bool value = false; };
 // leaves the register allocator room: a 128 x 128 wavefront tile fills all 256 accumulation registers and made
 // the compiler shuffle accumulators between register files around every MFMA).
 template <typename T, int WF, int MODE, int WN, int WM, int STAGES>
-__global__ void __launch_bounds__(64 * WN * WM, STAGES == 1 ? 2 : 1)
+__global__ void __launch_bounds__(64 * WN * WM, 1)
 grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
   constexpr int NTHR = 64 * WN * WM;
   constexpr int BN = 128 * WN;           // weight rows per workgroup tile (GATEUP: BN/2 gate + BN/2 up)
   constexpr int BM = 64 * WM;            // token rows per workgroup tile
-  constexpr int STAGE = (BN + BM) * BIG_LS;
+  static_assert(STAGES == 2, "two weight stages and three token stages");
+  constexpr int WSTAGE = BN * BIG_LS, XSTAGE = BM * BIG_LS;  // elements
   constexpr int WPIECES = (BN / 16) / (WN * WM);  // packed weight pieces per wavefront per K step
   constexpr int XPIECES = BM * 8 / NTHR;          // 16-byte token pieces per thread per K step
   constexpr int XROWS_PER_PASS = NTHR / 8;
@@ -119,46 +138,70 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
     const int64_t rt = row0 >> 4;
     wq[j] = wv->qs + (rt * kblocks * 64 + lane) * 16;
     wd[j] = reinterpret_cast<const uint16_t*>(wv->d) + (rt * (p.kred >> 8) * 16 + n_in) * 8 + (g >> 1);
+    // the scale of K step kt sits at wd[j] + (kt / 4) * 128 + (kt % 4) * 2
   }
   // Token rows past the end of the expert's rows are clamped to its last row: every output row depends on its
   // own token row only and those outputs are never stored, so no zero fill (and no branch) is needed.
-  const uint16_t* xp[XPIECES];
+  // A direct load puts lane l's 16 bytes at (wave-uniform LDS address) + 16*l, i.e. 8 lanes fill one 128-byte row
+  // in order; the XOR swizzle of the row is therefore applied to the source: LDS unit j of row r receives global
+  // unit j ^ (r & 7).
+  uint32_t xoff[XPIECES];  // byte offsets from p.a (the host checks that the activations span less than 4 GB)
 #pragma unroll
   for (int j = 0; j < XPIECES; ++j) {
-    const int r = min((tid >> 3) + XROWS_PER_PASS * j, rows_here - 1);
+    const int lr = (tid >> 3) + XROWS_PER_PASS * j;  // LDS row
+    const int r = min(lr, rows_here - 1);
     const int i = row_begin + r;
     const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
-    xp[j] = reinterpret_cast<const uint16_t*>(p.a) + src * p.lda + (tid & 7) * 8;
+    xoff[j] = (uint32_t)((src * p.lda + (((tid & 7) ^ (lr & 7)) << 3)) * 2);
   }
 
-  BigPiece<WF> wreg[WPIECES];
-  u32x4_t xreg[XPIECES];
-  auto load_global = [&](int64_t kt) {
+  uint16_t* const Wbase = lds;               // [2][BN][64]
+  uint16_t* const Xbase = lds + 2 * WSTAGE;  // [3][BM][64]
+  const uint32_t lds_addr0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)lds);
+  // LDS byte address of the 8 rows this wavefront fills in pass 0 of token stage 0
+  const uint32_t x_lds0 = __builtin_amdgcn_readfirstlane(lds_addr0 + (2 * WSTAGE + wave * 8 * BIG_LS) * 2);
+
+  // LDS addressing: rows handled by a lane differ from its base row by multiples of 16, so the swizzle term
+  // (unit ^ (row & 7)) depends on the lane (and the K half) only, and everything else is a compile-time offset.
+  const int sw = n_in & 7;
+  uint16_t* const w_st = Wbase + (wave * WPIECES * 16 + n_in) * BIG_LS;  // producer: first row tile of the wavefront
+  const int st_swz0 = ((2 * g) ^ sw) << 3, st_swz1 = ((2 * g + 1) ^ sw) << 3;
+  const uint16_t* a_rd[2];  // consumer, K half ks: weight row (wavefront base + n_in), unit ks*4 + g
+  const uint16_t* b_rd[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    const int u = ((ks * 4 + g) ^ sw) << 3;
+    a_rd[ks] = Wbase + ((MODE == MODE_GATEUP ? wn * 64 : wn * 128) + n_in) * BIG_LS + u;
+    b_rd[ks] = Xbase + (wm * 64 + n_in) * BIG_LS + u;
+  }
+
+  BigPiece<WF> wreg[2][WPIECES];
+  constexpr int WLOADS = 2 * WPIECES;  // vector-memory instructions of one load_w
+  auto load_w = [&](auto set_tag, int64_t kt) {
+    constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
     for (int j = 0; j < WPIECES; ++j) {
       // plain (cacheable) loads: the token tiles of one (expert, feature tile) run back to back on one XCD and
       // share the weight tile in its L2
-      wreg[j].q = *reinterpret_cast<const u32x4_t*>(wq[j] + kt * 1024);
-      const uint32_t d = wd[j][(kt >> 2) * 128 + (kt & 3) * 2];
-      wreg[j].dsel = d | (d << 16);
+      wreg[SET][j].q = *reinterpret_cast<const u32x4_t*>(wq[j] + kt * 1024);
+      wreg[SET][j].d = wd[j][(kt >> 2) * 128 + (kt & 3) * 2];
     }
-#pragma unroll
-    for (int j = 0; j < XPIECES; ++j) xreg[j] = *reinterpret_cast<const u32x4_t*>(xp[j] + kt * BIG_BK);
   };
-  auto store_lds = [&](int stage) {
-    uint16_t* Ws = lds + stage * STAGE;
-    uint16_t* Xs = Ws + BN * BIG_LS;
+  auto store_w = [&](auto set_tag) {  // registers of set s hold a K step of parity s and go to weight stage s
+    constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
     for (int j = 0; j < WPIECES; ++j) {
       uint32_t v[8];
-      wreg[j].template convert<T>(v);
-      const int row = (wave * WPIECES + j) * 16 + n_in;
-      *reinterpret_cast<u32x4_t*>(&Ws[lds_off(row, 2 * g)]) = (u32x4_t){v[0], v[1], v[2], v[3]};
-      *reinterpret_cast<u32x4_t*>(&Ws[lds_off(row, 2 * g + 1)]) = (u32x4_t){v[4], v[5], v[6], v[7]};
+      wreg[SET][j].template convert<T>(v);
+      uint16_t* row = w_st + SET * WSTAGE + j * 16 * BIG_LS;  // constants fold into the instruction's offset field
+      *reinterpret_cast<u32x4_t*>(row + st_swz0) = (u32x4_t){v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<u32x4_t*>(row + st_swz1) = (u32x4_t){v[4], v[5], v[6], v[7]};
     }
+  };
+  auto load_x = [&](int xstage, int64_t kt) {
 #pragma unroll
     for (int j = 0; j < XPIECES; ++j)
-      *reinterpret_cast<u32x4_t*>(&Xs[lds_off((tid >> 3) + XROWS_PER_PASS * j, tid & 7)]) = xreg[j];
+      vm_load16_to_lds(p.a, xoff[j] + (uint32_t)kt * (BIG_BK * 2), x_lds0 + (uint32_t)((xstage * XSTAGE + XROWS_PER_PASS * j * BIG_LS) * 2));
   };
 
   // ---- consumer -----------------------------------------------------------------------------------------
@@ -171,64 +214,102 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
     for (int b = 0; b < 4; ++b) acc[a][b] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
   const bool active = rows_here > wm * 64;  // wavefronts whose token rows are all past the end skip their MFMAs
 
-  auto w_lds_row = [&](int ti) -> int {
-    if (MODE == MODE_GATEUP) return (ti < 4 ? 0 : BN / 2) + wn * 64 + (ti & 3) * 16;
-    return wn * 128 + ti * 16;
-  };
-  auto compute = [&](int stage, int ks) {
-    const uint16_t* Ws = lds + stage * STAGE;
-    const uint16_t* Xs = Ws + BN * BIG_LS;
+  auto compute = [&](auto parity_tag, int xstage, int ks) {
+    constexpr int PAR = decltype(parity_tag)::value;
+    const uint16_t* bp = b_rd[ks] + xstage * XSTAGE;
     u32x4_t bf[4];
 #pragma unroll
-    for (int tj = 0; tj < 4; ++tj)
-      bf[tj] = *reinterpret_cast<const u32x4_t*>(&Xs[lds_off(wm * 64 + tj * 16 + n_in, ks * 4 + g)]);
+    for (int tj = 0; tj < 4; ++tj) bf[tj] = *reinterpret_cast<const u32x4_t*>(bp + tj * 16 * BIG_LS);
 #pragma unroll
     for (int ti = 0; ti < 8; ++ti) {
-      const u32x4_t af = *reinterpret_cast<const u32x4_t*>(&Ws[lds_off(w_lds_row(ti) + n_in, ks * 4 + g)]);
+      const int row_off = MODE == MODE_GATEUP ? (ti < 4 ? 0 : BN / 2) + (ti & 3) * 16 : ti * 16;
+      const u32x4_t af = *reinterpret_cast<const u32x4_t*>(a_rd[ks] + PAR * WSTAGE + row_off * BIG_LS);
 #pragma unroll
       for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = mfma16b<T>(af, bf[tj], acc[ti][tj]);
     }
   };
 
   const int64_t nkt = p.kred >> 6;
-  // ACTIVE is a compile-time tag so that the steady-state loop is one straight-line block (producer and MFMA
-  // instructions can be interleaved by the scheduler); wavefronts whose token rows are all past the end run the
-  // producer-only copy of the loop.
-  auto main_loop = [&](auto active_tag) {
+  // K step kt reads weight stage kt % 2 and token stage kt % 3.  During step kt a wavefront
+  //   converts and stores the weights of step kt + 1 (registers loaded during step kt - 2),
+  //   issues the token loads of step kt + 2 (into the stage last read in step kt - 1),
+  //   issues the weight loads of step kt + 3 (into the registers just freed),
+  // so every global load has about two K steps to arrive.  ACTIVE and LATE are compile-time tags so that a K step is
+  // one straight-line block; LATE wavefronts produce before their MFMAs, the others after.
+  // STEADY steps (kt + 3 < nkt) contain no branch, so two of them form one basic block and the compiler's waits for
+  // the weight registers stay exact; the last steps run the same code with the loads guarded.
+  auto k_step = [&](auto active_tag, auto late_tag, auto parity_tag, auto steady_tag, int64_t kt, int xs) {
     constexpr bool ACTIVE = decltype(active_tag)::value;
-    if constexpr (STAGES == 2) {
-      load_global(0);
-      store_lds(0);
-      __syncthreads();
-      if (nkt > 1) load_global(1);
-      for (int64_t kt = 0; kt < nkt; ++kt) {
-        const int stage = (int)(kt & 1);
-        if constexpr (ACTIVE) compute(stage, 0);
-        if (kt + 1 < nkt) {
-          store_lds(stage ^ 1);
-          if (kt + 2 < nkt) load_global(kt + 2);
-        }
-        if constexpr (ACTIVE) compute(stage, 1);
-        __syncthreads();
-      }
-    } else {
-      // one LDS stage, next K step prefetched into registers; two workgroups share a CU and fill each other's
-      // barrier and load bubbles
-      load_global(0);
-      for (int64_t kt = 0; kt < nkt; ++kt) {
-        store_lds(0);
-        __syncthreads();
-        load_global(kt + 1 < nkt ? kt + 1 : kt);
-        if constexpr (ACTIVE) {
-          compute(0, 0);
-          compute(0, 1);
-        }
-        __syncthreads();
+    constexpr bool LATE = decltype(late_tag)::value;
+    constexpr int PAR = decltype(parity_tag)::value;  // kt % 2
+    constexpr bool STEADY = decltype(steady_tag)::value;
+    using Next = BigSet<PAR ^ 1>;
+    auto produce = [&]() {
+      // the compiler's wait for the registers of step kt + 1 also covers the older token loads of that step
+      if (STEADY || kt + 1 < nkt) store_w(Next{});
+      if (STEADY || kt + 2 < nkt) load_x(xs >= 1 ? xs - 1 : 2, kt + 2);
+      if (STEADY || kt + 3 < nkt) load_w(Next{}, kt + 3);
+    };
+    // scheduling fences: without them the compiler hoists the LDS reads of both K halves and the next step's
+    // conversions across the whole block and runs out of registers
+    if constexpr (LATE) {
+      produce();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (ACTIVE) {
+      compute(parity_tag, xs, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(parity_tag, xs, 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (!LATE) {
+      produce();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // the token loads of step kt + 1 were issued during step kt - 1, before that step's weight loads; in steady state
+    // exactly those weight loads and this step's token and weight loads are younger
+    if constexpr (STEADY) vm_wait<2 * WLOADS + XPIECES>();
+    else vm_wait<0>();
+    __syncthreads();
+  };
+  auto main_loop = [&](auto active_tag, auto late_tag) {
+    load_w(BigSet<0>{}, 0);
+    load_x(0, 0);
+    if (nkt > 1) {
+      load_w(BigSet<1>{}, 1);
+      load_x(1, 1);
+    }
+    vm_wait<0>();
+    store_w(BigSet<0>{});
+    if (nkt > 2) load_w(BigSet<0>{}, 2);
+    __syncthreads();  // everything but the last weight loads has arrived
+    int xs = 0;       // kt % 3
+    int64_t kt = 0;
+    for (; kt + 4 < nkt; kt += 2) {
+      k_step(active_tag, late_tag, BigSet<0>{}, BigTagOn{}, kt, xs);
+      xs = xs == 2 ? 0 : xs + 1;
+      k_step(active_tag, late_tag, BigSet<1>{}, BigTagOn{}, kt + 1, xs);
+      xs = xs == 2 ? 0 : xs + 1;
+    }
+    for (; kt < nkt; kt += 2) {
+      k_step(active_tag, late_tag, BigSet<0>{}, BigTagOff{}, kt, xs);
+      xs = xs == 2 ? 0 : xs + 1;
+      if (kt + 1 < nkt) {
+        k_step(active_tag, late_tag, BigSet<1>{}, BigTagOff{}, kt + 1, xs);
+        xs = xs == 2 ? 0 : xs + 1;
       }
     }
   };
-  if (active) main_loop(BigTagOn{});
-  else main_loop(BigTagOff{});
+  // The two wavefronts that share a SIMD (w and w + 4) run the K step in opposite orders: one converts and stores
+  // the next stage while the other feeds the matrix pipe, then they swap, so the vector-ALU and LDS-write work of
+  // the producer overlaps MFMAs instead of leaving the matrix pipe idle between barriers.
+  const bool late = (wave & 4) != 0;
+  if (active) {
+    if (late) main_loop(BigTagOn{}, BigTagOn{});
+    else main_loop(BigTagOn{}, BigTagOff{});
+  } else {
+    main_loop(BigTagOff{}, BigTagOff{});
+  }
 
   // ---- epilogue -------------------------------------------------------------------------------------------
 #pragma unroll
@@ -258,7 +339,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
 template <typename T, int WF, int MODE, int WN, int WM, int STAGES>
 static int launch_big_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   constexpr int BN = 128 * WN, BM = 64 * WM;
-  constexpr size_t lds_bytes = (size_t)STAGES * (BN + BM) * BIG_LS * 2;
+  constexpr size_t lds_bytes = (size_t)(2 * BN + 3 * BM) * BIG_LS * 2;
   static bool attr_set = false;
   auto kern = grouped_mfma_big_kernel<T, WF, MODE, WN, WM, STAGES>;
   if (!attr_set) {
@@ -295,6 +376,12 @@ int launch_mfma_big(int act_dtype, int wtag, int mode, const GemmParams& p, int6
     return set_error(STMOE_ERR_UNSUPPORTED, "mfma big kernel: needs weights in the packed Q8_0 order");
   if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0 || p.n_out % (mode == MODE_GATEUP ? 64 * STMOE_BIG_WN : 128 * STMOE_BIG_WN) != 0)
     return set_error(STMOE_ERR_UNSUPPORTED, "mfma big kernel: needs K %% 256 == 0 and output features in whole tiles");
+  {
+    // token rows are addressed with 32-bit byte offsets from the activation base
+    const int64_t src_rows = p.perm ? (max_rows + p.k_top - 1) / p.k_top : max_rows;
+    if (src_rows * p.lda * 2 >= (int64_t)1 << 32)
+      return set_error(STMOE_ERR_UNSUPPORTED, "mfma big kernel: activations span 4 GB or more");
+  }
   if (act_dtype == STMOE_F16) return launch_big_t<f16_t, WF_Q8_0_P>(mode, p, max_rows, st);
   if (act_dtype == STMOE_BF16) return launch_big_t<bf16_t, WF_Q8_0_P>(mode, p, max_rows, st);
   return set_error(STMOE_ERR_UNSUPPORTED, "mfma big kernel: activation dtype %d", act_dtype);
