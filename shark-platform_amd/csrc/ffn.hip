@@ -43,13 +43,19 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 }
 
 // variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile, 3 skinny streaming kernel (decode),
-//          4 MFMA 256x256 tile (prefill; packed Q8_0), 5 fp8 matrix cores (fp8 weights and quantised activations)
+//          4 MFMA 256x256 tile (prefill; packed Q8_0), 5 fp8 matrix cores (fp8 weights and quantised activations),
+//          6 MFMA 256x256 tile with specialised producer/consumer wavefronts (prefill; packed Q8_0)
 static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
     else if (p.offsets && p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) variant = 3;
-    else variant = max_rows >= 512 ? 4 : 2;
+    else variant = max_rows >= 512 ? 6 : 2;
+  }
+  if (variant == 6) {
+    int rc = launch_mfma_ws(dtype, wtag, mode, p, max_rows, st);
+    if (rc != STMOE_ERR_UNSUPPORTED) return rc;
+    variant = 4;
   }
   if (variant == 4) {
     int rc = launch_mfma_big(dtype, wtag, mode, p, max_rows, st);

@@ -22,69 +22,9 @@
 // barrier of the K step that precedes their use (s_waitcnt vmcnt(n): loads return in issue order, and per K step a
 // wavefront issues XPIECES token loads followed by WLOADS weight loads, one 16-byte and one 2-byte load per piece).
 // The compiler's own waits for the weight registers do not count the hidden token loads and can only be stricter.
-#include "ffn_kernels.h"
+#include "ffn_mfma_common.h"
 
 namespace stmoe {
-
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float floatx4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-
-template <typename T> __device__ __forceinline__ floatx4_t mfma16b(const u32x4_t& a, const u32x4_t& b, floatx4_t c);
-template <> __device__ __forceinline__ floatx4_t mfma16b<f16_t>(const u32x4_t& a, const u32x4_t& b, floatx4_t c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
-}
-template <> __device__ __forceinline__ floatx4_t mfma16b<bf16_t>(const u32x4_t& a, const u32x4_t& b, floatx4_t c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-}
-
-static constexpr int BIG_BK = 64;
-static constexpr int BIG_LS = BIG_BK;  // LDS row stride (elements): 128 bytes = 8 units of 16 bytes, no padding
-
-// LDS rows are XOR-swizzled: the 16-byte unit u of row r lives at unit u ^ (r & 7).  ds_read_b128 serves lanes
-// in groups {0-3, 20-23}, {32-35, 52-55}, ... (4 rows of one K group and the next 4 rows of the neighbouring
-// K group) and ds_write_b128 in groups of 8 consecutive lanes; with the swizzle every such group touches 8
-// distinct 16-byte bank groups for the operand reads, the weight-row writes and the token-row writes alike.
-__device__ __forceinline__ int lds_off(int row, int unit) { return row * BIG_LS + ((unit ^ (row & 7)) << 3); }
-
-// ---- hand-issued vector-memory operations ------------------------------------------------------------
-// Lane l's 16 bytes at base + byte_off land at LDS byte address lds_addr + 16*l (base and lds_addr wave-uniform).
-__device__ __forceinline__ void vm_load16_to_lds(const void* base, uint32_t byte_off, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(byte_off), "s"(base), "s"(lds_addr)
-               : "memory", "m0");
-}
-template <int N> __device__ __forceinline__ void vm_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-
-// One packed 1 KB piece (16 rows x 64 k of 1-byte samples, or 16 rows x 128 k of nibbles) as held by one lane.
-template <int WF> struct BigPiece;
-template <> struct BigPiece<WF_Q8_0_P> {
-  u32x4_t q;
-  uint32_t d;  // the lane's block scale (fp16 bits, zero-extended)
-  // 16 values of T: row n = lane%16, k = 16*g .. 16*g+15 of the 64-wide K step
-  template <typename T> __device__ __forceinline__ void convert(uint32_t out[8]) const {
-    const half2_t dd = as_half2(d | (d << 16));
-    const half2_t bias = {(f16_t)1152.0f, (f16_t)1152.0f};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t u = q[i] ^ 0x80808080u;
-      const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
-      const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
-      const uint32_t a = as_u32((as_half2(lo) - bias) * dd), b = as_u32((as_half2(hi) - bias) * dd);
-      if constexpr (__is_same(T, f16_t)) {
-        out[2 * i] = a;
-        out[2 * i + 1] = b;
-      } else {
-        out[2 * i] = pack2<bf16_t>(f16_bits_to_f32(a & 0xffffu), f16_bits_to_f32(a >> 16));
-        out[2 * i + 1] = pack2<bf16_t>(f16_bits_to_f32(b & 0xffffu), f16_bits_to_f32(b >> 16));
-      }
-    }
-  }
-};
-
-template <int V> struct BigSet { static constexpr int value = V; };
-struct BigTagOn { static constexpr bool value = true; };
-struct BigTagOff { static constexpr bool value = false; };
 
 // WN x WM wavefronts; each owns 128 weight rows x 64 token rows (32 accumulator tiles = 128 registers, which
 // leaves the register allocator room: a 128 x 128 wavefront tile fills all 256 accumulation registers and made
@@ -106,6 +46,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
   const int wn = wave / WM, wm = wave % WM;
 
   // ---- tile id: XCD-aware remap, token tile fastest -------------------------------------------------
+#ifndef STMOE_BIG_SCHED_OWNER
   int pid = blockIdx.x;
   {
     const int per_xcd = gridDim.x >> 3;  // the host rounds the grid up to a multiple of 8
@@ -113,6 +54,37 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
   }
   const int slot = pid % m_slots, ntile = pid / m_slots;
   if (ntile >= n_tiles) return;
+#else
+  int slot, ntile;
+  {
+    int total_slots = 0;
+    if (p.offsets) {
+      for (int ee = 0; ee < p.E; ++ee) total_slots += (p.offsets[ee + 1] - p.offsets[ee] + BM - 1) / BM;
+    } else {
+      total_slots = (int)((p.fixed_rows + BM - 1) / BM);
+    }
+    const int units = total_slots * n_tiles;
+    const int xcd = blockIdx.x & 7;
+    int j = blockIdx.x >> 3;
+    const int u0 = (int)((int64_t)units * xcd / 8), u1 = (int)((int64_t)units * (xcd + 1) / 8);
+    if (j >= u1 - u0) return;
+    const int s_first = u0 / n_tiles, s_last = (u1 - 1) / n_tiles;
+    slot = -1;
+    ntile = 0;
+    for (int t = 0; t < n_tiles; ++t) {
+      const int s_min = s_first + (s_first * n_tiles + t < u0 ? 1 : 0);
+      const int s_max = s_last - (s_last * n_tiles + t >= u1 ? 1 : 0);
+      const int cnt = s_max - s_min + 1;
+      if (j < cnt) {
+        slot = s_min + j;
+        ntile = t;
+        break;
+      }
+      j -= cnt > 0 ? cnt : 0;
+    }
+    if (slot < 0) return;
+  }
+#endif
   int e, row_begin, row_end;
   if (!find_tile(p, slot, BM, e, row_begin, row_end)) return;
   const int rows_here = row_end - row_begin;
@@ -350,7 +322,7 @@ static int launch_big_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;
-  const int total = (n_tiles * m_slots + 7) / 8 * 8;
+  const int total = ((n_tiles * m_slots + 7) / 8 + 1) * 8;
   kern<<<dim3((unsigned)total), 64 * WN * WM, lds_bytes, st>>>(p, n_tiles, m_slots);
   return check_launch("grouped_mfma_big");
 }

@@ -1,0 +1,269 @@
+// Prefill kernel with specialised wavefronts: 256 x 256 workgroup tile, 8 consumer + 4 producer wavefronts.
+//
+//   consumers (wavefronts 0-7, 2 x 4): 128 weight rows x 64 token rows each (GATEUP: 64 gate + the same 64 up rows);
+//             a K step is nothing but LDS operand reads and 64 MFMAs, so both consumers of a SIMD keep the matrix
+//             pipe fed all the time
+//   producers (wavefronts 8-11, one per SIMD): per K step each loads 4 packed 1 KB weight pieces into registers
+//             (two K steps ahead), dequantises them and writes 16-bit rows into the next weight stage, and issues 8
+//             direct global->LDS loads of token rows (also two K steps ahead)
+//   LDS (160 KB): 2 weight stages + 3 token stages of 32 KB, rows of 128 bytes XOR-swizzled in 16-byte units;
+//             one barrier per K step
+//   registers: 12 wavefronts leave 168 per lane; the consumers hold 128 accumulators and 20 operand registers
+//
+// The direct loads are inline assembly and are awaited by hand (see ffn_mfma_common.h); per K step a producer
+// issues XLOADS token loads followed by WLOADS weight loads, always in this order.
+#include "ffn_mfma_common.h"
+
+namespace stmoe {
+
+template <int V> struct WsInt { static constexpr int value = V; };
+
+template <typename T, int WF, int MODE>
+__global__ void __launch_bounds__(768, 1)
+grouped_mfma_ws_kernel(GemmParams p, int n_tiles, int m_slots) {
+  constexpr int BN = 256, BM = 256;
+  constexpr int WSTAGE = BN * BIG_LS, XSTAGE = BM * BIG_LS;  // elements
+  constexpr int WPIECES = 4;   // packed weight pieces per producer per K step (16 row tiles / 4 producers)
+  constexpr int XLOADS = 8;    // direct token loads per producer per K step (32 blocks of 8 rows / 4 producers)
+  constexpr int WLOADS = 2 * WPIECES;
+  extern __shared__ __align__(16) uint16_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane >> 4, n_in = lane & 15;
+
+  // ---- tile id: XCD-aware remap, token tile fastest ---------------------------------------------------
+  int pid = blockIdx.x;
+  {
+    const int per_xcd = gridDim.x >> 3;  // the host rounds the grid up to a multiple of 8
+    pid = (pid & 7) * per_xcd + (pid >> 3);
+  }
+  const int slot = pid % m_slots, ntile = pid / m_slots;
+  if (ntile >= n_tiles) return;
+  int e, row_begin, row_end;
+  if (!find_tile(p, slot, BM, e, row_begin, row_end)) return;
+  const int rows_here = row_end - row_begin;
+  const int64_t nkt = p.kred >> 6;
+
+  uint16_t* const Wbase = lds;               // [2][BN][64]
+  uint16_t* const Xbase = lds + 2 * WSTAGE;  // [3][BM][64]
+  const int sw = n_in & 7;
+
+  if (wave >= 8) {
+    // =================================== producer ===================================
+    const int pw = wave - 8;
+    const uint8_t* wq[WPIECES];
+    const uint16_t* wd[WPIECES];
+    const int64_t kblocks = p.kred >> 6;
+#pragma unroll
+    for (int j = 0; j < WPIECES; ++j) {
+      const int rtl = pw * WPIECES + j;  // row tile (16 rows) inside the workgroup tile
+      int64_t row0;
+      const WeightView* wv;
+      if (MODE == MODE_GATEUP) {
+        const bool up = rtl >= BN / 32;
+        wv = up ? &p.w1 : &p.w0;
+        row0 = (int64_t)e * wv->rows + (int64_t)ntile * (BN / 2) + (rtl % (BN / 32)) * 16;
+      } else {
+        wv = &p.w0;
+        row0 = (int64_t)e * wv->rows + (int64_t)ntile * BN + rtl * 16;
+      }
+      const int64_t rt = row0 >> 4;
+      wq[j] = wv->qs + (rt * kblocks * 64 + lane) * 16;
+      wd[j] = reinterpret_cast<const uint16_t*>(wv->d) + (rt * (p.kred >> 8) * 16 + n_in) * 8 + (g >> 1);
+    }
+    // token rows: lane l of direct load j fills LDS row pw*8 + 32*j + l/8, unit l%8, from global unit (l%8) ^ (row & 7);
+    // rows past the end of the expert's rows re-read its last row (their outputs are never stored)
+    uint32_t xoff[XLOADS];
+#pragma unroll
+    for (int j = 0; j < XLOADS; ++j) {
+      const int lr = pw * 8 + 32 * j + (lane >> 3);
+      const int r = min(lr, rows_here - 1);
+      const int i = row_begin + r;
+      const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
+      xoff[j] = (uint32_t)((src * p.lda + (((lane & 7) ^ (lr & 7)) << 3)) * 2);
+    }
+    const uint32_t lds_addr0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)lds);
+    const uint32_t x_lds0 = __builtin_amdgcn_readfirstlane(lds_addr0 + (2 * WSTAGE + pw * 8 * BIG_LS) * 2);
+    uint16_t* const w_st = Wbase + (pw * WPIECES * 16 + n_in) * BIG_LS;
+    const int st_swz0 = ((2 * g) ^ sw) << 3, st_swz1 = ((2 * g + 1) ^ sw) << 3;
+
+    BigPiece<WF> wreg[2][WPIECES];
+    auto load_w = [&](auto set_tag, int64_t kt) {
+      constexpr int SET = decltype(set_tag)::value;
+#pragma unroll
+      for (int j = 0; j < WPIECES; ++j) {
+        wreg[SET][j].q = *reinterpret_cast<const u32x4_t*>(wq[j] + kt * 1024);
+        wreg[SET][j].d = wd[j][(kt >> 2) * 128 + (kt & 3) * 2];
+      }
+    };
+    auto store_w = [&](auto set_tag) {  // registers of set s hold a K step of parity s and go to weight stage s
+      constexpr int SET = decltype(set_tag)::value;
+#pragma unroll
+      for (int j = 0; j < WPIECES; ++j) {
+        uint32_t v[8];
+        wreg[SET][j].template convert<T>(v);
+        uint16_t* row = w_st + SET * WSTAGE + j * 16 * BIG_LS;
+        *reinterpret_cast<u32x4_t*>(row + st_swz0) = (u32x4_t){v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<u32x4_t*>(row + st_swz1) = (u32x4_t){v[4], v[5], v[6], v[7]};
+      }
+    };
+    auto load_x = [&](int xstage, int64_t kt) {
+#pragma unroll
+      for (int j = 0; j < XLOADS; ++j)
+        vm_load16_to_lds(p.a, xoff[j] + (uint32_t)kt * (BIG_BK * 2), x_lds0 + (uint32_t)((xstage * XSTAGE + 32 * j * BIG_LS) * 2));
+    };
+    // During K step kt: store the weights of step kt + 1 (loaded during step kt - 2), issue the token loads of step
+    // kt + 2 and the weight loads of step kt + 3; before the barrier the token loads of step kt + 1 (issued during
+    // step kt - 1, followed by that step's weight loads) must have landed.
+    auto k_step = [&](auto parity_tag, auto steady_tag, int64_t kt, int xs) {
+      constexpr int PAR = decltype(parity_tag)::value;
+      constexpr bool STEADY = decltype(steady_tag)::value;
+      using Next = WsInt<PAR ^ 1>;
+      if (STEADY || kt + 1 < nkt) store_w(Next{});
+      if (STEADY || kt + 2 < nkt) load_x(xs >= 1 ? xs - 1 : 2, kt + 2);
+      if (STEADY || kt + 3 < nkt) load_w(Next{}, kt + 3);
+      if constexpr (STEADY) vm_wait<2 * WLOADS + XLOADS>();
+      else vm_wait<0>();
+      __syncthreads();
+    };
+    load_w(WsInt<0>{}, 0);
+    load_x(0, 0);
+    if (nkt > 1) {
+      load_w(WsInt<1>{}, 1);
+      load_x(1, 1);
+    }
+    vm_wait<0>();
+    store_w(WsInt<0>{});
+    if (nkt > 2) load_w(WsInt<0>{}, 2);
+    __syncthreads();
+    int xs = 0;
+    int64_t kt = 0;
+    for (; kt + 4 < nkt; kt += 2) {
+      k_step(WsInt<0>{}, WsInt<1>{}, kt, xs);
+      xs = xs == 2 ? 0 : xs + 1;
+      k_step(WsInt<1>{}, WsInt<1>{}, kt + 1, xs);
+      xs = xs == 2 ? 0 : xs + 1;
+    }
+    for (; kt < nkt; kt += 2) {
+      k_step(WsInt<0>{}, WsInt<0>{}, kt, xs);
+      xs = xs == 2 ? 0 : xs + 1;
+      if (kt + 1 < nkt) {
+        k_step(WsInt<1>{}, WsInt<0>{}, kt + 1, xs);
+        xs = xs == 2 ? 0 : xs + 1;
+      }
+    }
+    return;
+  }
+
+  // =================================== consumer ===================================
+  const int wn = wave >> 2, wm = wave & 3;
+  const uint16_t* a_rd[2];  // K half ks: weight row (wavefront base + n_in), unit ks*4 + g
+  const uint16_t* b_rd[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    const int u = ((ks * 4 + g) ^ sw) << 3;
+    a_rd[ks] = Wbase + ((MODE == MODE_GATEUP ? wn * 64 : wn * 128) + n_in) * BIG_LS + u;
+    b_rd[ks] = Xbase + (wm * 64 + n_in) * BIG_LS + u;
+  }
+  floatx4_t acc[8][4];
+#pragma unroll
+  for (int a = 0; a < 8; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[a][b] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+  const bool active = rows_here > wm * 64;  // wavefronts whose token rows are all past the end skip their MFMAs
+
+  auto compute = [&](auto parity_tag, int xstage, int ks) {
+    constexpr int PAR = decltype(parity_tag)::value;
+    const uint16_t* bp = b_rd[ks] + xstage * XSTAGE;
+    u32x4_t bf[4];
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) bf[tj] = *reinterpret_cast<const u32x4_t*>(bp + tj * 16 * BIG_LS);
+#pragma unroll
+    for (int ti = 0; ti < 8; ++ti) {
+      const int row_off = MODE == MODE_GATEUP ? (ti < 4 ? 0 : BN / 2) + (ti & 3) * 16 : ti * 16;
+      const u32x4_t af = *reinterpret_cast<const u32x4_t*>(a_rd[ks] + PAR * WSTAGE + row_off * BIG_LS);
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = mfma16b<T>(af, bf[tj], acc[ti][tj]);
+    }
+  };
+  __syncthreads();  // first stage filled
+  if (active) {
+    int xs = 0;
+    for (int64_t kt = 0; kt < nkt; kt += 2) {
+      compute(WsInt<0>{}, xs, 0);
+      compute(WsInt<0>{}, xs, 1);
+      __syncthreads();
+      xs = xs == 2 ? 0 : xs + 1;
+      if (kt + 1 < nkt) {
+        compute(WsInt<1>{}, xs, 0);
+        compute(WsInt<1>{}, xs, 1);
+        __syncthreads();
+        xs = xs == 2 ? 0 : xs + 1;
+      }
+    }
+  } else {
+    for (int64_t kt = 0; kt < nkt; ++kt) __syncthreads();
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------------
+#pragma unroll
+  for (int tj = 0; tj < 4; ++tj) {
+    const int r = wm * 64 + tj * 16 + n_in;
+    if (r < rows_here) {
+      T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo;
+      if (MODE == MODE_GATEUP) {
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti) {
+          float v[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = gateup_epilogue<T>(p.act, acc[ti][tj][q], acc[ti + 4][tj][q], 1.0f);
+          *reinterpret_cast<uint2*>(orow + (int64_t)ntile * (BN / 2) + wn * 64 + ti * 16 + 4 * g) =
+              make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
+        }
+      } else {
+#pragma unroll
+        for (int ti = 0; ti < 8; ++ti)
+          *reinterpret_cast<uint2*>(orow + (int64_t)ntile * BN + wn * 128 + ti * 16 + 4 * g) =
+              make_uint2(pack2<T>(acc[ti][tj][0], acc[ti][tj][1]), pack2<T>(acc[ti][tj][2], acc[ti][tj][3]));
+      }
+    }
+  }
+}
+
+template <typename T, int WF, int MODE>
+static int launch_ws_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
+  constexpr int BN = 256, BM = 256;
+  constexpr size_t lds_bytes = (size_t)(2 * BN + 3 * BM) * BIG_LS * 2;
+  static bool attr_set = false;
+  auto kern = grouped_mfma_ws_kernel<T, WF, MODE>;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+      return set_error(STMOE_ERR_LAUNCH, "mfma ws kernel: cannot reserve %zu bytes of LDS", lds_bytes);
+    attr_set = true;
+  }
+  const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
+  const int experts = p.offsets ? p.E : 1;
+  const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;
+  const int total = (n_tiles * m_slots + 7) / 8 * 8;
+  kern<<<dim3((unsigned)total), 768, lds_bytes, st>>>(p, n_tiles, m_slots);
+  return check_launch("grouped_mfma_ws");
+}
+
+int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
+  if (max_rows == 0) return STMOE_OK;
+  if (wtag != WF_Q8_0_P)
+    return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs weights in the packed Q8_0 order");
+  if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0 || p.n_out % (mode == MODE_GATEUP ? 128 : 256) != 0)
+    return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs K %% 256 == 0 and output features in whole tiles");
+  {
+    const int64_t src_rows = p.perm ? (max_rows + p.k_top - 1) / p.k_top : max_rows;
+    if (src_rows * p.lda * 2 >= (int64_t)1 << 32)
+      return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: activations span 4 GB or more");
+  }
+  if (act_dtype == STMOE_F16)
+    return mode == MODE_GATEUP ? launch_ws_m<f16_t, WF_Q8_0_P, MODE_GATEUP>(p, max_rows, st) : launch_ws_m<f16_t, WF_Q8_0_P, MODE_DOWN>(p, max_rows, st);
+  if (act_dtype == STMOE_BF16)
+    return mode == MODE_GATEUP ? launch_ws_m<bf16_t, WF_Q8_0_P, MODE_GATEUP>(p, max_rows, st) : launch_ws_m<bf16_t, WF_Q8_0_P, MODE_DOWN>(p, max_rows, st);
+  return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: activation dtype %d", act_dtype);
+}
+
+}  // namespace stmoe

@@ -301,7 +301,8 @@ def test_packed_weights_match_planar(device, fmt, dtype, variant, T):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("T,E,act", [(700, 8, "silu"), (700, 2, "gelu"), (130, 1, "silu")])
 def test_ffn_mfma_big_kernel(device, dtype, T, E, act):
-    """The 256 x 256 prefill kernel (packed Q8_0): ragged tiles, several token tiles per expert, one expert."""
+    """The 256 x 256 prefill kernels (packed Q8_0; one with every wavefront producing and consuming, one with
+    specialised producer and consumer wavefronts): ragged tiles, several token tiles per expert, one expert."""
     hip = _hip()
     from sharktank_amd.ops import device_weight
 
@@ -319,8 +320,10 @@ def test_ffn_mfma_big_kernel(device, dtype, T, E, act):
     _, offsets, perm, inv = hip.dispatch_build(idx.to(torch.int32).to(device), E)
     act_e = hip.ACT_SILU if act == "silu" else hip.ACT_GELU_ERF
     outs = {}
-    for variant in (hip.VARIANT_MFMA_BIG, hip.VARIANT_MFMA_TILE):
+    for variant in (hip.VARIANT_MFMA_BIG, hip.VARIANT_MFMA_WS, hip.VARIANT_MFMA_TILE):
         y = hip.grouped_ffn(case.planes["h"].to(device), dws[0], dws[1], dws[2], act_e, offsets, perm, case.k, variant=variant)
         outs[variant] = hip.combine(y, gate.to(device), inv, T, case.k).cpu()
         assert O.rel_l2(outs[variant], want) < tol
     assert O.rel_l2(outs[hip.VARIANT_MFMA_BIG], outs[hip.VARIANT_MFMA_TILE]) < tol
+    # both 256 x 256 kernels accumulate every output in the same order
+    assert torch.equal(outs[hip.VARIANT_MFMA_BIG], outs[hip.VARIANT_MFMA_WS])
