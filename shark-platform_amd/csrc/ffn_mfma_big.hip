@@ -14,8 +14,7 @@
 //   the two wavefronts of a SIMD run producer and consumer halves of a K step in opposite orders, so that one
 //             converts and stores while the other feeds the matrix pipe
 //   ragged tiles: wavefronts whose 64 token rows are all past the end of the expert's rows skip their MFMAs
-//   scheduling: workgroup ids are remapped so that consecutive logical tiles run on the same XCD (one L2),
-//               with the token tiles of one (expert, feature tile) adjacent so they share its weights in L2.
+//   scheduling: see big_tile_id (equal shares per XCD, partial token tiles last).
 //
 // The direct loads are written as inline assembly: given the builtin, the compiler waits for every outstanding load
 // before each LDS read, which would undo the prefetch.  Their completion is therefore awaited by hand before the
@@ -31,7 +30,7 @@ namespace stmoe {
 // the compiler shuffle accumulators between register files around every MFMA).
 template <typename T, int WF, int MODE, int WN, int WM, int STAGES>
 __global__ void __launch_bounds__(64 * WN * WM, 1)
-grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
+grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
   constexpr int NTHR = 64 * WN * WM;
   constexpr int BN = 128 * WN;           // weight rows per workgroup tile (GATEUP: BN/2 gate + BN/2 up)
   constexpr int BM = 64 * WM;            // token rows per workgroup tile
@@ -45,48 +44,9 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles, int m_slots) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wn = wave / WM, wm = wave % WM;
 
-  // ---- tile id: XCD-aware remap, token tile fastest -------------------------------------------------
-#ifndef STMOE_BIG_SCHED_OWNER
-  int pid = blockIdx.x;
-  {
-    const int per_xcd = gridDim.x >> 3;  // the host rounds the grid up to a multiple of 8
-    pid = (pid & 7) * per_xcd + (pid >> 3);
-  }
-  const int slot = pid % m_slots, ntile = pid / m_slots;
-  if (ntile >= n_tiles) return;
-#else
-  int slot, ntile;
-  {
-    int total_slots = 0;
-    if (p.offsets) {
-      for (int ee = 0; ee < p.E; ++ee) total_slots += (p.offsets[ee + 1] - p.offsets[ee] + BM - 1) / BM;
-    } else {
-      total_slots = (int)((p.fixed_rows + BM - 1) / BM);
-    }
-    const int units = total_slots * n_tiles;
-    const int xcd = blockIdx.x & 7;
-    int j = blockIdx.x >> 3;
-    const int u0 = (int)((int64_t)units * xcd / 8), u1 = (int)((int64_t)units * (xcd + 1) / 8);
-    if (j >= u1 - u0) return;
-    const int s_first = u0 / n_tiles, s_last = (u1 - 1) / n_tiles;
-    slot = -1;
-    ntile = 0;
-    for (int t = 0; t < n_tiles; ++t) {
-      const int s_min = s_first + (s_first * n_tiles + t < u0 ? 1 : 0);
-      const int s_max = s_last - (s_last * n_tiles + t >= u1 ? 1 : 0);
-      const int cnt = s_max - s_min + 1;
-      if (j < cnt) {
-        slot = s_min + j;
-        ntile = t;
-        break;
-      }
-      j -= cnt > 0 ? cnt : 0;
-    }
-    if (slot < 0) return;
-  }
-#endif
-  int e, row_begin, row_end;
-  if (!find_tile(p, slot, BM, e, row_begin, row_end)) return;
+  BigTile tile;
+  if (!big_tile_id(p, BM, n_tiles, tile)) return;
+  const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
 
   // ---- producer assignment ---------------------------------------------------------------------------
@@ -322,8 +282,7 @@ static int launch_big_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;
-  const int total = ((n_tiles * m_slots + 7) / 8 + 1) * 8;
-  kern<<<dim3((unsigned)total), 64 * WN * WM, lds_bytes, st>>>(p, n_tiles, m_slots);
+  kern<<<dim3((unsigned)big_grid(n_tiles, m_slots)), 64 * WN * WM, lds_bytes, st>>>(p, n_tiles);
   return check_launch("grouped_mfma_big");
 }
 

@@ -27,6 +27,79 @@ static constexpr int BIG_LS = BIG_BK;  // LDS row stride (elements): 128 bytes =
 // distinct 16-byte bank groups for the operand reads, the weight-row writes and the token-row writes alike.
 __device__ __forceinline__ int lds_off(int row, int unit) { return row * BIG_LS + ((unit ^ (row & 7)) << 3); }
 
+// ---- work distribution ---------------------------------------------------------------------------------
+// Token tiles are the full ones (BM rows) and the partial ones (the last rows of an expert).  A unit is one token
+// tile times one feature tile.  Workgroup ids are dealt round-robin to the 8 XCDs; XCD i takes the i-th eighth of
+// the full units and then the i-th eighth of the partial units, so every XCD gets the same amount of work (within
+// one unit) and the short partial units run last, where they fill the end of the launch instead of delaying full
+// units.  Inside each class the token tile index runs fastest, so the token tiles of one expert work on the same
+// weight slab at the same time and share it in the XCD's L2.
+struct BigTile {
+  int e, row_begin, row_end, ntile;
+};
+__device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_tiles, BigTile& t) {
+  int F = 0, R = 0;
+  if (p.offsets) {
+    for (int e = 0; e < p.E; ++e) {
+      const int rows = p.offsets[e + 1] - p.offsets[e];
+      F += rows / BM;
+      R += (rows % BM) != 0;
+    }
+  } else {
+    F = (int)(p.fixed_rows / BM);
+    R = (p.fixed_rows % BM) != 0;
+  }
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  const int UF = F * n_tiles, UR = R * n_tiles;
+  const int f0 = (int)((int64_t)UF * xcd / 8), f1 = (int)((int64_t)UF * (xcd + 1) / 8);
+  const int r0 = (int)((int64_t)UR * xcd / 8), r1 = (int)((int64_t)UR * (xcd + 1) / 8);
+  int u, cnt;
+  bool partial;
+  if (j < f1 - f0) {
+    u = f0 + j;
+    cnt = F;
+    partial = false;
+  } else if (j - (f1 - f0) < r1 - r0) {
+    u = r0 + j - (f1 - f0);
+    cnt = R;
+    partial = true;
+  } else {
+    return false;
+  }
+  t.ntile = u / cnt;
+  int s = u - t.ntile * cnt;
+  if (!p.offsets) {
+    t.e = 0;
+    t.row_begin = partial ? F * BM : s * BM;
+    t.row_end = partial ? (int)p.fixed_rows : t.row_begin + BM;
+    return true;
+  }
+  for (int e = 0; e < p.E; ++e) {
+    const int b = p.offsets[e], rows = p.offsets[e + 1] - b;
+    if (!partial) {
+      const int c = rows / BM;
+      if (s < c) {
+        t.e = e;
+        t.row_begin = b + s * BM;
+        t.row_end = t.row_begin + BM;
+        return true;
+      }
+      s -= c;
+    } else if (rows % BM) {
+      if (s == 0) {
+        t.e = e;
+        t.row_begin = b + rows / BM * BM;
+        t.row_end = b + rows;
+        return true;
+      }
+      --s;
+    }
+  }
+  return false;
+}
+// Grid size that covers every XCD's share for at most `slots_bound` token tiles.
+static inline int big_grid(int n_tiles, int slots_bound) { return 8 * ((n_tiles * slots_bound + 7) / 8 + 2); }
+
 // ---- hand-issued vector-memory operations ------------------------------------------------------------
 // Lane l's 16 bytes at base + byte_off land at LDS byte address lds_addr + 16*l (base and lds_addr wave-uniform).
 __device__ __forceinline__ void vm_load16_to_lds(const void* base, uint32_t byte_off, uint32_t lds_addr) {

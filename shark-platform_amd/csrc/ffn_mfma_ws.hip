@@ -4,8 +4,8 @@
 //             a K step is nothing but LDS operand reads and 64 MFMAs, so both consumers of a SIMD keep the matrix
 //             pipe fed all the time
 //   producers (wavefronts 8-11, one per SIMD): per K step each loads 4 packed 1 KB weight pieces into registers
-//             (two K steps ahead), dequantises them and writes 16-bit rows into the next weight stage, and issues 8
-//             direct global->LDS loads of token rows (also two K steps ahead)
+//             (three K steps before they are needed), dequantises them and writes 16-bit rows into the next weight
+//             stage, and issues 8 direct global->LDS loads of token rows (two K steps ahead)
 //   LDS (160 KB): 2 weight stages + 3 token stages of 32 KB, rows of 128 bytes XOR-swizzled in 16-byte units;
 //             one barrier per K step
 //   registers: 12 wavefronts leave 168 per lane; the consumers hold 128 accumulators and 20 operand registers
@@ -20,7 +20,7 @@ template <int V> struct WsInt { static constexpr int value = V; };
 
 template <typename T, int WF, int MODE>
 __global__ void __launch_bounds__(768, 1)
-grouped_mfma_ws_kernel(GemmParams p, int n_tiles, int m_slots) {
+grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
   constexpr int BN = 256, BM = 256;
   constexpr int WSTAGE = BN * BIG_LS, XSTAGE = BM * BIG_LS;  // elements
   constexpr int WPIECES = 4;   // packed weight pieces per producer per K step (16 row tiles / 4 producers)
@@ -30,16 +30,9 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, int m_slots) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, n_in = lane & 15;
 
-  // ---- tile id: XCD-aware remap, token tile fastest ---------------------------------------------------
-  int pid = blockIdx.x;
-  {
-    const int per_xcd = gridDim.x >> 3;  // the host rounds the grid up to a multiple of 8
-    pid = (pid & 7) * per_xcd + (pid >> 3);
-  }
-  const int slot = pid % m_slots, ntile = pid / m_slots;
-  if (ntile >= n_tiles) return;
-  int e, row_begin, row_end;
-  if (!find_tile(p, slot, BM, e, row_begin, row_end)) return;
+  BigTile tile;
+  if (!big_tile_id(p, BM, n_tiles, tile)) return;
+  const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
   const int64_t nkt = p.kred >> 6;
 
@@ -86,7 +79,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, int m_slots) {
     uint16_t* const w_st = Wbase + (pw * WPIECES * 16 + n_in) * BIG_LS;
     const int st_swz0 = ((2 * g) ^ sw) << 3, st_swz1 = ((2 * g + 1) ^ sw) << 3;
 
-    BigPiece<WF> wreg[2][WPIECES];
+    BigPiece<WF> wreg[3][WPIECES];  // three register sets: weights are loaded three K steps before their conversion
     auto load_w = [&](auto set_tag, int64_t kt) {
       constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
@@ -95,60 +88,67 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, int m_slots) {
         wreg[SET][j].d = wd[j][(kt >> 2) * 128 + (kt & 3) * 2];
       }
     };
-    auto store_w = [&](auto set_tag) {  // registers of set s hold a K step of parity s and go to weight stage s
-      constexpr int SET = decltype(set_tag)::value;
+    auto store_w = [&](auto set_tag, auto stage_tag) {
+      constexpr int SET = decltype(set_tag)::value, STAGE = decltype(stage_tag)::value;
 #pragma unroll
       for (int j = 0; j < WPIECES; ++j) {
         uint32_t v[8];
         wreg[SET][j].template convert<T>(v);
-        uint16_t* row = w_st + SET * WSTAGE + j * 16 * BIG_LS;
+        uint16_t* row = w_st + STAGE * WSTAGE + j * 16 * BIG_LS;
         *reinterpret_cast<u32x4_t*>(row + st_swz0) = (u32x4_t){v[0], v[1], v[2], v[3]};
         *reinterpret_cast<u32x4_t*>(row + st_swz1) = (u32x4_t){v[4], v[5], v[6], v[7]};
       }
     };
-    auto load_x = [&](int xstage, int64_t kt) {
+    auto load_x = [&](auto xstage_tag, int64_t kt) {
+      constexpr int XS = decltype(xstage_tag)::value;
 #pragma unroll
       for (int j = 0; j < XLOADS; ++j)
-        vm_load16_to_lds(p.a, xoff[j] + (uint32_t)kt * (BIG_BK * 2), x_lds0 + (uint32_t)((xstage * XSTAGE + 32 * j * BIG_LS) * 2));
+        vm_load16_to_lds(p.a, xoff[j] + (uint32_t)kt * (BIG_BK * 2), x_lds0 + (uint32_t)((XS * XSTAGE + 32 * j * BIG_LS) * 2));
     };
-    // During K step kt: store the weights of step kt + 1 (loaded during step kt - 2), issue the token loads of step
-    // kt + 2 and the weight loads of step kt + 3; before the barrier the token loads of step kt + 1 (issued during
-    // step kt - 1, followed by that step's weight loads) must have landed.
-    auto k_step = [&](auto parity_tag, auto steady_tag, int64_t kt, int xs) {
-      constexpr int PAR = decltype(parity_tag)::value;
+    // K step kt (R = kt % 6 fixes every stage and register set at compile time): store the weights of step kt + 1
+    // (register set (kt+1) % 3, loaded during step kt - 3) into weight stage (kt+1) % 2, issue the token loads of step
+    // kt + 2 into token stage (kt+2) % 3 and the weight loads of step kt + 4 into the register set just freed.  Before
+    // the barrier the token loads of step kt + 1 must have landed: they were issued during step kt - 1, followed by
+    // that step's weight loads and this step's token and weight loads.  STEADY steps (kt + 4 < nkt) have no branch.
+    auto k_step = [&](auto r_tag, auto steady_tag, int64_t kt) {
+      constexpr int R = decltype(r_tag)::value;
       constexpr bool STEADY = decltype(steady_tag)::value;
-      using Next = WsInt<PAR ^ 1>;
-      if (STEADY || kt + 1 < nkt) store_w(Next{});
-      if (STEADY || kt + 2 < nkt) load_x(xs >= 1 ? xs - 1 : 2, kt + 2);
-      if (STEADY || kt + 3 < nkt) load_w(Next{}, kt + 3);
+      using Set = WsInt<(R + 1) % 3>;
+      if (STEADY || kt + 1 < nkt) store_w(Set{}, WsInt<(R + 1) % 2>{});
+      if (STEADY || kt + 2 < nkt) load_x(WsInt<(R + 2) % 3>{}, kt + 2);
+      if (STEADY || kt + 4 < nkt) load_w(Set{}, kt + 4);
       if constexpr (STEADY) vm_wait<2 * WLOADS + XLOADS>();
       else vm_wait<0>();
       __syncthreads();
     };
     load_w(WsInt<0>{}, 0);
-    load_x(0, 0);
+    load_x(WsInt<0>{}, 0);
     if (nkt > 1) {
       load_w(WsInt<1>{}, 1);
-      load_x(1, 1);
+      load_x(WsInt<1>{}, 1);
     }
+    if (nkt > 2) load_w(WsInt<2>{}, 2);
+    store_w(WsInt<0>{}, WsInt<0>{});
+    if (nkt > 3) load_w(WsInt<0>{}, 3);
     vm_wait<0>();
-    store_w(WsInt<0>{});
-    if (nkt > 2) load_w(WsInt<0>{}, 2);
     __syncthreads();
-    int xs = 0;
     int64_t kt = 0;
-    for (; kt + 4 < nkt; kt += 2) {
-      k_step(WsInt<0>{}, WsInt<1>{}, kt, xs);
-      xs = xs == 2 ? 0 : xs + 1;
-      k_step(WsInt<1>{}, WsInt<1>{}, kt + 1, xs);
-      xs = xs == 2 ? 0 : xs + 1;
+    for (; kt + 9 < nkt; kt += 6) {
+      k_step(WsInt<0>{}, WsInt<1>{}, kt);
+      k_step(WsInt<1>{}, WsInt<1>{}, kt + 1);
+      k_step(WsInt<2>{}, WsInt<1>{}, kt + 2);
+      k_step(WsInt<3>{}, WsInt<1>{}, kt + 3);
+      k_step(WsInt<4>{}, WsInt<1>{}, kt + 4);
+      k_step(WsInt<5>{}, WsInt<1>{}, kt + 5);
     }
-    for (; kt < nkt; kt += 2) {
-      k_step(WsInt<0>{}, WsInt<0>{}, kt, xs);
-      xs = xs == 2 ? 0 : xs + 1;
-      if (kt + 1 < nkt) {
-        k_step(WsInt<1>{}, WsInt<0>{}, kt + 1, xs);
-        xs = xs == 2 ? 0 : xs + 1;
+    for (int r = 0; kt < nkt; ++kt, ++r) {  // kt % 6 == r here: the steady loop advances in sixes
+      switch (r % 6) {
+        case 0: k_step(WsInt<0>{}, WsInt<0>{}, kt); break;
+        case 1: k_step(WsInt<1>{}, WsInt<0>{}, kt); break;
+        case 2: k_step(WsInt<2>{}, WsInt<0>{}, kt); break;
+        case 3: k_step(WsInt<3>{}, WsInt<0>{}, kt); break;
+        case 4: k_step(WsInt<4>{}, WsInt<0>{}, kt); break;
+        default: k_step(WsInt<5>{}, WsInt<0>{}, kt); break;
       }
     }
     return;
@@ -243,8 +243,7 @@ static int launch_ws_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;
-  const int total = (n_tiles * m_slots + 7) / 8 * 8;
-  kern<<<dim3((unsigned)total), 768, lds_bytes, st>>>(p, n_tiles, m_slots);
+  kern<<<dim3((unsigned)big_grid(n_tiles, m_slots)), 768, lds_bytes, st>>>(p, n_tiles);
   return check_launch("grouped_mfma_ws");
 }
 
