@@ -66,8 +66,13 @@ __device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_t
   } else {
     return false;
   }
+#ifdef STMOE_BIG_SLOT_MAJOR
+  int s = u / n_tiles;
+  t.ntile = u - s * n_tiles;
+#else
   t.ntile = u / cnt;
   int s = u - t.ntile * cnt;
+#endif
   if (!p.offsets) {
     t.e = 0;
     t.row_begin = partial ? F * BM : s * BM;

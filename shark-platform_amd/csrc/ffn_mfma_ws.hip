@@ -1,6 +1,6 @@
 // Prefill kernel with specialised wavefronts: 256 x 256 workgroup tile, 8 consumer + 4 producer wavefronts.
 //
-//   consumers (wavefronts 0-7, 2 x 4): 128 weight rows x 64 token rows each (GATEUP: 64 gate + the same 64 up rows);
+//   consumers (wavefronts 0-7: 2 weight-row halves x 4 token-row groups): 128 weight rows x 64 token rows each (GATEUP: 64 gate + the same 64 up rows);
 //             a K step is nothing but LDS operand reads and 64 MFMAs, so both consumers of a SIMD keep the matrix
 //             pipe fed all the time
 //   producers (wavefronts 8-11, one per SIMD): per K step each loads 4 packed 1 KB weight pieces into registers
@@ -155,7 +155,9 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
   }
 
   // =================================== consumer ===================================
-  const int wn = wave >> 2, wm = wave & 3;
+  // Wavefront w runs on SIMD w % 4.  Token-row groups (wm) are spread so that a partial tile, where only the first
+  // groups have rows, still uses several SIMDs: wm 0 -> SIMDs 0,1; wm 1 -> SIMDs 2,3; wm 2 -> 0,1; wm 3 -> 2,3.
+  const int wn = wave & 1, wm = wave >> 1;
   const uint16_t* a_rd[2];  // K half ks: weight row (wavefront base + n_in), unit ks*4 + g
   const uint16_t* b_rd[2];
 #pragma unroll
