@@ -45,11 +45,15 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 // variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile, 3 skinny streaming kernel (decode),
 //          4 MFMA 256x256 tile (prefill; packed Q8_0), 5 fp8 matrix cores (fp8 weights and quantised activations),
 //          6 MFMA 256x256 tile with specialised producer/consumer wavefronts (prefill; packed Q8_0)
+// The streaming kernel is chosen when no expert can get more than 32 rows, or when experts get 40 rows or fewer on
+// average (it then walks an expert's rows in passes of 32, re-reading the expert's weights for every pass).
 static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
+static constexpr int64_t kSkinnyMaxAvgRows = 40;
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
-    else if (p.offsets && p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) variant = 3;
+    else if (p.offsets && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
+                           max_rows <= kSkinnyMaxAvgRows * p.E)) variant = 3;
     else variant = max_rows >= 512 ? 6 : 2;
   }
   if (variant == 6) {
@@ -142,7 +146,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   // runs unchanged; otherwise both operands go to the fp8 matrix cores as bytes (variant 5).
   const bool fp8_w_in = w_gate->format == STMOE_W_FP8 || w_gate->format == STMOE_W_FP8_PACKED;
   const bool fp8_w_out = w_down->format == STMOE_W_FP8 || w_down->format == STMOE_W_FP8_PACKED;
-  const bool few_rows = T <= kSkinnyMaxRowsPerExpert;
+  const bool few_rows = T <= kSkinnyMaxRowsPerExpert || T * k <= kSkinnyMaxAvgRows * E;
   STMOE_REQUIRE(variant != 5 || (x_scale && z_scale), STMOE_ERR_UNSUPPORTED, "grouped_ffn: variant 5 (fp8 matrix cores) needs x_scale and z_scale");
   const bool t16 = dtype == STMOE_F16 || dtype == STMOE_BF16;
   const bool mfma8_in = t16 && x_scale && fp8_w_in && w_gate->dtype == STMOE_F32 && K % 16 == 0 && (variant == 5 || (variant == 0 && !few_rows));

@@ -25,6 +25,10 @@
 
 namespace stmoe {
 
+template <int V> struct BigSet { static constexpr int value = V; };
+struct BigTagOn { static constexpr bool value = true; };
+struct BigTagOff { static constexpr bool value = false; };
+
 // WN x WM wavefronts; each owns 128 weight rows x 64 token rows (32 accumulator tiles = 128 registers, which
 // leaves the register allocator room: a 128 x 128 wavefront tile fills all 256 accumulation registers and made
 // the compiler shuffle accumulators between register files around every MFMA).
@@ -51,9 +55,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
 
   // ---- producer assignment ---------------------------------------------------------------------------
   const int g = lane >> 4, n_in = lane & 15;
-  const uint8_t* wq[WPIECES];
-  const uint16_t* wd[WPIECES];
-  const int64_t kblocks = p.kred >> 6;
+  BigAddr<WF> waddr[WPIECES];
 #pragma unroll
   for (int j = 0; j < WPIECES; ++j) {
     const int rtl = wave * WPIECES + j;  // row tile (16 rows) inside the workgroup tile
@@ -67,10 +69,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
       wv = &p.w0;
       row0 = (int64_t)e * wv->rows + (int64_t)ntile * BN + rtl * 16;
     }
-    const int64_t rt = row0 >> 4;
-    wq[j] = wv->qs + (rt * kblocks * 64 + lane) * 16;
-    wd[j] = reinterpret_cast<const uint16_t*>(wv->d) + (rt * (p.kred >> 8) * 16 + n_in) * 8 + (g >> 1);
-    // the scale of K step kt sits at wd[j] + (kt / 4) * 128 + (kt % 4) * 2
+    waddr[j].init(*wv, row0 >> 4, e, lane, p.kred);
   }
   // Token rows past the end of the expert's rows are clamped to its last row: every output row depends on its
   // own token row only and those outputs are never stored, so no zero fill (and no branch) is needed.
@@ -108,15 +107,14 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
   }
 
   BigPiece<WF> wreg[2][WPIECES];
-  constexpr int WLOADS = 2 * WPIECES;  // vector-memory instructions of one load_w
+  constexpr int WLOADS = BigPiece<WF>::LOADS * WPIECES;  // vector-memory instructions of one load_w
   auto load_w = [&](auto set_tag, int64_t kt) {
     constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
     for (int j = 0; j < WPIECES; ++j) {
       // plain (cacheable) loads: the token tiles of one (expert, feature tile) run back to back on one XCD and
       // share the weight tile in its L2
-      wreg[SET][j].q = *reinterpret_cast<const u32x4_t*>(wq[j] + kt * 1024);
-      wreg[SET][j].d = wd[j][(kt >> 2) * 128 + (kt & 3) * 2];
+      wreg[SET][j].load(waddr[j], kt);
     }
   };
   auto store_w = [&](auto set_tag) {  // registers of set s hold a K step of parity s and go to weight stage s
@@ -124,7 +122,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
 #pragma unroll
     for (int j = 0; j < WPIECES; ++j) {
       uint32_t v[8];
-      wreg[SET][j].template convert<T>(v);
+      wreg[SET][j].template convert<T>(waddr[j], v);
       uint16_t* row = w_st + SET * WSTAGE + j * 16 * BIG_LS;  // constants fold into the instruction's offset field
       *reinterpret_cast<u32x4_t*>(row + st_swz0) = (u32x4_t){v[0], v[1], v[2], v[3]};
       *reinterpret_cast<u32x4_t*>(row + st_swz1) = (u32x4_t){v[4], v[5], v[6], v[7]};

@@ -113,34 +113,114 @@ __device__ __forceinline__ void vm_load16_to_lds(const void* base, uint32_t byte
 }
 template <int N> __device__ __forceinline__ void vm_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
-// One packed 1 KB piece (16 rows x 64 k of 1-byte samples, or 16 rows x 128 k of nibbles) as held by one lane.
+// ---- packed weight pieces -----------------------------------------------------------------------------
+// Per K step (64 reduction elements) and row tile (16 rows), lane (n = lane % 16, g = lane / 16) fetches the samples
+// of row n, k = 16*g .. 16*g + 15 and their block scale, and later converts them to 16 values of T (8 dwords) that
+// go to LDS units 2g and 2g + 1 of row n.  BigAddr holds what does not change along K, BigPiece what is in flight.
+template <int WF> struct BigAddr;
 template <int WF> struct BigPiece;
+
+// (q + 1152) built by byte permutation as 0x6400 | u8, minus 1152, times d: f16(d * q) with one rounding
+__device__ __forceinline__ void q8x16_to_f16(const u32x4_t& q, uint32_t dbits, uint32_t out[8]) {
+  const half2_t dd = as_half2(dbits | (dbits << 16));
+  const half2_t bias = {(f16_t)1152.0f, (f16_t)1152.0f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t u = q[i] ^ 0x80808080u;
+    const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
+    const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
+    out[2 * i] = as_u32((as_half2(lo) - bias) * dd);
+    out[2 * i + 1] = as_u32((as_half2(hi) - bias) * dd);
+  }
+}
+template <typename T> __device__ __forceinline__ void f16x16_to_T(uint32_t v[8]) {
+  if constexpr (!__is_same(T, f16_t)) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = pack2<T>(f16_bits_to_f32(v[i] & 0xffffu), f16_bits_to_f32(v[i] >> 16));
+  }
+}
+
+// Q8_0: 1 KB piece = 16 rows x 64 k; scales d_p[rt][K/256][16][8]
+template <> struct BigAddr<WF_Q8_0_P> {
+  const uint8_t* q;
+  const uint16_t* d;
+  __device__ __forceinline__ void init(const WeightView& w, int64_t rt, int64_t, int lane, int64_t kred) {
+    q = w.qs + (rt * (kred >> 6) * 64 + lane) * 16;
+    d = reinterpret_cast<const uint16_t*>(w.d) + (rt * (kred >> 8) * 16 + (lane & 15)) * 8 + (lane >> 5);
+  }
+};
 template <> struct BigPiece<WF_Q8_0_P> {
+  static constexpr int LOADS = 2;
   u32x4_t q;
-  uint32_t d;  // the lane's block scale (fp16 bits, zero-extended)
-  // 16 values of T: row n = lane%16, k = 16*g .. 16*g+15 of the 64-wide K step
-  template <typename T> __device__ __forceinline__ void convert(uint32_t out[8]) const {
-    const half2_t dd = as_half2(d | (d << 16));
-    const half2_t bias = {(f16_t)1152.0f, (f16_t)1152.0f};
+  uint32_t d;  // fp16 bits, zero-extended
+  __device__ __forceinline__ void load(const BigAddr<WF_Q8_0_P>& a, int64_t kt) {
+    q = *reinterpret_cast<const u32x4_t*>(a.q + kt * 1024);
+    d = a.d[(kt >> 2) * 128 + (kt & 3) * 2];
+  }
+  template <typename T> __device__ __forceinline__ void convert(const BigAddr<WF_Q8_0_P>&, uint32_t out[8]) const {
+    q8x16_to_f16(q, d, out);
+    f16x16_to_T<T>(out);
+  }
+};
+
+// fp8 e4m3fn with one fp32 scale per tensor or per expert: pieces as Q8_0, T(f32(q) * d)
+template <> struct BigAddr<WF_FP8_F32D_P> {
+  const uint8_t* q;
+  float dv;
+  __device__ __forceinline__ void init(const WeightView& w, int64_t rt, int64_t e, int lane, int64_t kred) {
+    q = w.qs + (rt * (kred >> 6) * 64 + lane) * 16;
+    dv = reinterpret_cast<const float*>(w.d)[w.d_count > 1 ? e : 0];
+  }
+};
+template <> struct BigPiece<WF_FP8_F32D_P> {
+  static constexpr int LOADS = 1;
+  u32x4_t q;
+  __device__ __forceinline__ void load(const BigAddr<WF_FP8_F32D_P>& a, int64_t kt) {
+    q = *reinterpret_cast<const u32x4_t*>(a.q + kt * 1024);
+  }
+  template <typename T> __device__ __forceinline__ void convert(const BigAddr<WF_FP8_F32D_P>& a, uint32_t out[8]) const {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const uint32_t u = q[i] ^ 0x80808080u;
-      const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
-      const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
-      const uint32_t a = as_u32((as_half2(lo) - bias) * dd), b = as_u32((as_half2(hi) - bias) * dd);
-      if constexpr (__is_same(T, f16_t)) {
-        out[2 * i] = a;
-        out[2 * i + 1] = b;
-      } else {
-        out[2 * i] = pack2<bf16_t>(f16_bits_to_f32(a & 0xffffu), f16_bits_to_f32(a >> 16));
-        out[2 * i + 1] = pack2<bf16_t>(f16_bits_to_f32(b & 0xffffu), f16_bits_to_f32(b >> 16));
-      }
+      float f[4];
+      fp8x4_to_f32(q[i], f);
+      out[2 * i] = pack2<T>(__fmul_rn(f[0], a.dv), __fmul_rn(f[1], a.dv));
+      out[2 * i + 1] = pack2<T>(__fmul_rn(f[2], a.dv), __fmul_rn(f[3], a.dv));
     }
   }
 };
 
-template <int V> struct BigSet { static constexpr int value = V; };
-struct BigTagOn { static constexpr bool value = true; };
-struct BigTagOff { static constexpr bool value = false; };
+// Q4_1: 1 KB piece = 16 rows x 128 k (lane (n, g') holds block g' of row n, nibbles in the packed order); a K step
+// takes half of it: the lane's 16 samples are 8 bytes of block 2*(kt % 2) + g/2, half g % 2
+template <> struct BigAddr<WF_Q4_1_P> {
+  const uint8_t* q;
+  const uint16_t* d;
+  const uint16_t* m;
+  __device__ __forceinline__ void init(const WeightView& w, int64_t rt, int64_t, int lane, int64_t kred) {
+    const int n = lane & 15, g = lane >> 4;
+    q = w.qs + rt * (kred >> 7) * 1024 + (((g >> 1) * 16 + n) * 16 + (g & 1) * 8);
+    const int64_t s = (rt * (kred >> 8) * 16 + n) * 8 + (g >> 1);
+    d = reinterpret_cast<const uint16_t*>(w.d) + s;
+    m = reinterpret_cast<const uint16_t*>(w.m) + s;
+  }
+};
+template <> struct BigPiece<WF_Q4_1_P> {
+  static constexpr int LOADS = 3;
+  uint2 q;
+  uint32_t d, m;
+  __device__ __forceinline__ void load(const BigAddr<WF_Q4_1_P>& a, int64_t kt) {
+    q = *reinterpret_cast<const uint2*>(a.q + (kt >> 1) * 1024 + (kt & 1) * 512);
+    const int64_t s = (kt >> 2) * 128 + (kt & 3) * 2;
+    d = a.d[s];
+    m = a.m[s];
+  }
+  template <typename T> __device__ __forceinline__ void convert(const BigAddr<WF_Q4_1_P>&, uint32_t out[8]) const {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      out[b] = q4_pair_dequant(q4_pair_packed(q.x, b), d, m);
+      out[4 + b] = q4_pair_dequant(q4_pair_packed(q.y, b), d, m);
+    }
+    f16x16_to_T<T>(out);
+  }
+};
 
 }  // namespace stmoe

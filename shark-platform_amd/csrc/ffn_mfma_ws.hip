@@ -25,7 +25,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
   constexpr int WSTAGE = BN * BIG_LS, XSTAGE = BM * BIG_LS;  // elements
   constexpr int WPIECES = 4;   // packed weight pieces per producer per K step (16 row tiles / 4 producers)
   constexpr int XLOADS = 8;    // direct token loads per producer per K step (32 blocks of 8 rows / 4 producers)
-  constexpr int WLOADS = 2 * WPIECES;
+  constexpr int WLOADS = BigPiece<WF>::LOADS * WPIECES;
   extern __shared__ __align__(16) uint16_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, n_in = lane & 15;
@@ -43,9 +43,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
   if (wave >= 8) {
     // =================================== producer ===================================
     const int pw = wave - 8;
-    const uint8_t* wq[WPIECES];
-    const uint16_t* wd[WPIECES];
-    const int64_t kblocks = p.kred >> 6;
+    BigAddr<WF> waddr[WPIECES];
 #pragma unroll
     for (int j = 0; j < WPIECES; ++j) {
       const int rtl = pw * WPIECES + j;  // row tile (16 rows) inside the workgroup tile
@@ -59,9 +57,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
         wv = &p.w0;
         row0 = (int64_t)e * wv->rows + (int64_t)ntile * BN + rtl * 16;
       }
-      const int64_t rt = row0 >> 4;
-      wq[j] = wv->qs + (rt * kblocks * 64 + lane) * 16;
-      wd[j] = reinterpret_cast<const uint16_t*>(wv->d) + (rt * (p.kred >> 8) * 16 + n_in) * 8 + (g >> 1);
+      waddr[j].init(*wv, row0 >> 4, e, lane, p.kred);
     }
     // token rows: lane l of direct load j fills LDS row pw*8 + 32*j + l/8, unit l%8, from global unit (l%8) ^ (row & 7);
     // rows past the end of the expert's rows re-read its last row (their outputs are never stored)
@@ -84,8 +80,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
       constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
       for (int j = 0; j < WPIECES; ++j) {
-        wreg[SET][j].q = *reinterpret_cast<const u32x4_t*>(wq[j] + kt * 1024);
-        wreg[SET][j].d = wd[j][(kt >> 2) * 128 + (kt & 3) * 2];
+        wreg[SET][j].load(waddr[j], kt);
       }
     };
     auto store_w = [&](auto set_tag, auto stage_tag) {
@@ -93,7 +88,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
 #pragma unroll
       for (int j = 0; j < WPIECES; ++j) {
         uint32_t v[8];
-        wreg[SET][j].template convert<T>(v);
+        wreg[SET][j].template convert<T>(waddr[j], v);
         uint16_t* row = w_st + STAGE * WSTAGE + j * 16 * BIG_LS;
         *reinterpret_cast<u32x4_t*>(row + st_swz0) = (u32x4_t){v[0], v[1], v[2], v[3]};
         *reinterpret_cast<u32x4_t*>(row + st_swz1) = (u32x4_t){v[4], v[5], v[6], v[7]};
@@ -249,21 +244,33 @@ static int launch_ws_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   return check_launch("grouped_mfma_ws");
 }
 
+template <typename T, int WF>
+static int launch_ws_t(int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
+  return mode == MODE_GATEUP ? launch_ws_m<T, WF, MODE_GATEUP>(p, max_rows, st) : launch_ws_m<T, WF, MODE_DOWN>(p, max_rows, st);
+}
+
 int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (max_rows == 0) return STMOE_OK;
-  if (wtag != WF_Q8_0_P)
-    return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs weights in the packed Q8_0 order");
+  if (wtag != WF_Q8_0_P && wtag != WF_Q4_1_P && wtag != WF_FP8_F32D_P)
+    return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs weights in a packed streaming order");
   if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0 || p.n_out % (mode == MODE_GATEUP ? 128 : 256) != 0)
     return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs K %% 256 == 0 and output features in whole tiles");
   {
+    // token rows are addressed with 32-bit byte offsets from the activation base
     const int64_t src_rows = p.perm ? (max_rows + p.k_top - 1) / p.k_top : max_rows;
     if (src_rows * p.lda * 2 >= (int64_t)1 << 32)
       return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: activations span 4 GB or more");
   }
-  if (act_dtype == STMOE_F16)
-    return mode == MODE_GATEUP ? launch_ws_m<f16_t, WF_Q8_0_P, MODE_GATEUP>(p, max_rows, st) : launch_ws_m<f16_t, WF_Q8_0_P, MODE_DOWN>(p, max_rows, st);
-  if (act_dtype == STMOE_BF16)
-    return mode == MODE_GATEUP ? launch_ws_m<bf16_t, WF_Q8_0_P, MODE_GATEUP>(p, max_rows, st) : launch_ws_m<bf16_t, WF_Q8_0_P, MODE_DOWN>(p, max_rows, st);
+  if (act_dtype == STMOE_F16) {
+    if (wtag == WF_Q8_0_P) return launch_ws_t<f16_t, WF_Q8_0_P>(mode, p, max_rows, st);
+    if (wtag == WF_Q4_1_P) return launch_ws_t<f16_t, WF_Q4_1_P>(mode, p, max_rows, st);
+    return launch_ws_t<f16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
+  }
+  if (act_dtype == STMOE_BF16) {
+    if (wtag == WF_Q8_0_P) return launch_ws_t<bf16_t, WF_Q8_0_P>(mode, p, max_rows, st);
+    if (wtag == WF_Q4_1_P) return launch_ws_t<bf16_t, WF_Q4_1_P>(mode, p, max_rows, st);
+    return launch_ws_t<bf16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
+  }
   return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: activation dtype %d", act_dtype);
 }
 

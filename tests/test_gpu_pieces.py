@@ -327,3 +327,33 @@ def test_ffn_mfma_big_kernel(device, dtype, T, E, act):
     assert O.rel_l2(outs[hip.VARIANT_MFMA_BIG], outs[hip.VARIANT_MFMA_TILE]) < tol
     # both 256 x 256 kernels accumulate every output in the same order
     assert torch.equal(outs[hip.VARIANT_MFMA_BIG], outs[hip.VARIANT_MFMA_WS])
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("fmt", ["q4_1", "fp8"])
+def test_ffn_mfma_ws_kernel_formats(device, dtype, fmt):
+    """The specialised-wavefront prefill kernel on packed Q4_1 and fp8 weights: same values as the 128 x 128 tile
+    kernel (both dequantise every weight to the activation dtype before the product) and the oracle."""
+    hip = _hip()
+    from sharktank_amd.ops import device_weight
+
+    T, E = 600, 4
+    tol = 1e-3 if dtype == torch.float16 else 8e-3
+    case = MC.build(MC.Case(T=T, K=512, N=768, E=E, k=2, fmt=fmt, dtype=dtype, seed=62))
+    K, N = case.K, case.N
+    g = torch.Generator().manual_seed(63)
+    idx = torch.stack([torch.randperm(E, generator=g)[: case.k] for _ in range(T)])
+    gate = torch.rand(T, case.k, generator=g)
+    gate = (gate / gate.sum(-1, keepdim=True)).to(dtype)
+    wg, wu, wd = MC.dense_weights(case)
+    want = O.grouped_ffn_moe(case.planes["h"], idx, gate, wg, wu, wd, case.activation)
+    dws = [device_weight(MC.to_inference_tensor(fmt, case.planes[n], shp, n, device), stacked=True, prepack=True)
+           for n, shp in (("gate", [E, N, K]), ("up", [E, N, K]), ("down", [E, K, N]))]
+    assert all(w.is_packed for w in dws)
+    _, offsets, perm, inv = hip.dispatch_build(idx.to(torch.int32).to(device), E)
+    outs = {}
+    for variant in (hip.VARIANT_MFMA_WS, hip.VARIANT_MFMA_TILE):
+        y = hip.grouped_ffn(case.planes["h"].to(device), dws[0], dws[1], dws[2], hip.ACT_SILU, offsets, perm, case.k, variant=variant)
+        outs[variant] = hip.combine(y, gate.to(device), inv, T, case.k).cpu()
+        assert O.rel_l2(outs[variant], want) < tol
+    assert O.rel_l2(outs[hip.VARIANT_MFMA_WS], outs[hip.VARIANT_MFMA_TILE]) < tol
