@@ -37,7 +37,7 @@ class PreGatherFFNMOE(ThetaLayer):
         self.ffn_up = theta.tensor("ffn_up_exps", "weight")
         self.ffn_down = theta.tensor("ffn_down_exps", "weight")
         # Optional static per-tensor fp8 quantizers of the activations, named as LinearLayer names its input quantizer
-        # (sharktank/sharktank/layers/linear.py:49): `ffn_gate_exps.q_input` quantises h for the gate and up
+        # (sharktank/sharktank/layers/linear.py:57): `ffn_gate_exps.q_input` quantises h for the gate and up
         # projections, `ffn_down_exps.q_input` the gated intermediate for the down projection.  The values are the
         # reference's quantise-then-dequantise ones (linear.py:72-78).
         self.q_input = theta.optional_tensor("ffn_gate_exps", "q_input")
