@@ -11,21 +11,29 @@ import torch.nn.functional as F
 
 from oracle import moe_oracle as O
 
+import json
+import os
+
+with open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")) as _f:
+    GOLDEN = json.load(_f)
+
 
 # ---- i4 nibble utilities: sharktank/tests/types/layout_utils_test.py:15-65 ---------------------------------
 def test_linearize_and_interleave_known_answer():
-    inter = torch.tensor([[0x80, 0x91, 0xA2, 0xB3, 0xC4, 0xD5, 0xE6, 0xF7]], dtype=torch.uint8)
+    v = GOLDEN["i4_interleaved_to_linear"]
+    inter = torch.tensor([v["interleaved"]], dtype=torch.uint8)
     linear = O.linearize_interleaved_i4_block(inter)
-    assert linear.tolist() == [[0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]]
+    assert linear.tolist() == [v["linear"]]
     assert O.interleave_linear_i4_block(linear).tolist() == inter.tolist()
 
 
 def test_promote_i4_known_answer():
-    linear = torch.tensor([[0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]], dtype=torch.uint8)
+    v = GOLDEN["i4_promote"]
+    linear = torch.tensor([v["linear"]], dtype=torch.uint8)
     u = O.promote_linear_i4_block_to_i8(linear)
-    assert u.dtype == torch.uint8 and u.tolist() == [list(range(16))]
+    assert u.dtype == torch.uint8 and u.tolist() == [v["unsigned"]]
     s = O.promote_linear_i4_block_to_i8(linear, signed=True)
-    assert s.dtype == torch.int8 and s.tolist() == [[0, 1, 2, 3, 4, 5, 6, 7, -8, -7, -6, -5, -4, -3, -2, -1]]
+    assert s.dtype == torch.int8 and s.tolist() == [v["signed"]]
 
 
 def test_linearize_is_a_permutation_of_nibbles():
@@ -39,8 +47,9 @@ def test_linearize_is_a_permutation_of_nibbles():
 
 # ---- TensorScaledLayout: sharktank/tests/types/layouts_test.py:107-125 ---------------------------------------
 def test_tensor_scaled_known_answer():
-    got = O.dequant_tensor_scaled(torch.tensor(2.0), torch.tensor([2.0, 3.0, 4.0], dtype=torch.float16), torch.tensor(5.0))
-    assert got.dtype == torch.float32 and got.tolist() == [-6.0, -4.0, -2.0]
+    v = GOLDEN["tensor_scaled_dequant"]
+    got = O.dequant_tensor_scaled(torch.tensor(v["d"]), torch.tensor(v["qs"], dtype=torch.float16), torch.tensor(v["m"]))
+    assert got.dtype == torch.float32 and got.tolist() == v["want"]
 
 
 # ---- block-scaled dequant: exact rational arithmetic with a hand-written round-to-nearest-even -----------------
@@ -127,8 +136,7 @@ def test_dynamic_quantizer_roundtrip(dtype):  # :133-170
     torch.testing.assert_close(orig, got, atol=1e-1, rtol=1e-1)
 
 
-QUARK_FP8 = [-58, -48, -70, 53, -53, 76, -71, -90, 50, 77, 62, -98, 66, -54, 55, -80, -66, -62, -61, -56, 56, -67, 79,
-             -60, -71, 42, 72, -73, 91, 63, 124, -128]
+QUARK_FP8 = GOLDEN["quark_fp8"]["int8_bit_patterns"]
 
 
 def test_quark_fp8_vector():  # :172-244
