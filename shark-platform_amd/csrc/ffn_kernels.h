@@ -67,6 +67,39 @@ template <typename T> __device__ __forceinline__ float gateup_epilogue(int act, 
   return round_to<T>(__fmul_rn(a, ur));
 }
 
+// Epilogue of the prefill kernels for one accumulator quad (4 consecutive features of one token): the same rounding
+// points as gateup_epilogue, with the activation fixed at compile time.  SiLU is x * rcp(1 + exp2(-x * log2 e)) on the
+// hardware exp2 / rcp (about 1 ulp of fp32 each, far below the rounding to the 16-bit activation dtype that
+// follows); for fp16 the last product is a packed fp16 multiply, which rounds the exact product once like the fp32
+// multiply followed by the conversion.
+template <int ACT> __device__ __forceinline__ float act_fast(float v) {
+  if constexpr (ACT == STMOE_ACT_SILU)
+    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.44269504088896340736f));
+  else
+    return act_gelu_erf(v);
+}
+template <typename T, int ACT>
+__device__ __forceinline__ uint2 gateup_quad(const float (&g)[4], const float (&u)[4]) {
+  if constexpr (__is_same(T, f16_t)) {
+    uint32_t out[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const half2_t a = {(f16_t)act_fast<ACT>((float)(f16_t)g[2 * h]), (f16_t)act_fast<ACT>((float)(f16_t)g[2 * h + 1])};
+      const half2_t uu = {(f16_t)u[2 * h], (f16_t)u[2 * h + 1]};
+      out[h] = as_u32(a * uu);
+    }
+    return make_uint2(out[0], out[1]);
+  } else {
+    float v[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float a = round_to<T>(act_fast<ACT>(round_to<T>(g[q])));
+      v[q] = round_to<T>(__fmul_rn(a, round_to<T>(u[q])));
+    }
+    return make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
+  }
+}
+
 }  // namespace stmoe
 
 namespace stmoe {

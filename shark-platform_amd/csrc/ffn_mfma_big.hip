@@ -241,22 +241,32 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
     main_loop(BigTagOff{}, BigTagOff{});
   }
 
-  // ---- epilogue -------------------------------------------------------------------------------------------
+  // ---- epilogue ---------------------------------------------------------------------------------------
+  auto store_gateup = [&](auto act_tag) {
+    constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
-  for (int tj = 0; tj < 4; ++tj) {
-    const int r = wm * 64 + tj * 16 + n_in;
-    if (r < rows_here) {
-      T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo;
-      if (MODE == MODE_GATEUP) {
+    for (int tj = 0; tj < 4; ++tj) {
+      const int r = wm * 64 + tj * 16 + n_in;
+      if (r < rows_here) {
+        T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo + (int64_t)ntile * (BN / 2) + wn * 64 + 4 * g;
 #pragma unroll
         for (int ti = 0; ti < 4; ++ti) {
-          float v[4];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) v[q] = gateup_epilogue<T>(p.act, acc[ti][tj][q], acc[ti + 4][tj][q], 1.0f);
-          *reinterpret_cast<uint2*>(orow + (int64_t)ntile * (BN / 2) + wn * 64 + ti * 16 + 4 * g) =
-              make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
+          const float gq[4] = {acc[ti][tj][0], acc[ti][tj][1], acc[ti][tj][2], acc[ti][tj][3]};
+          const float uq[4] = {acc[ti + 4][tj][0], acc[ti + 4][tj][1], acc[ti + 4][tj][2], acc[ti + 4][tj][3]};
+          *reinterpret_cast<uint2*>(orow + ti * 16) = gateup_quad<T, ACT>(gq, uq);
         }
-      } else {
+      }
+    }
+  };
+  if (MODE == MODE_GATEUP) {
+    if (p.act == STMOE_ACT_SILU) store_gateup(EpiAct<STMOE_ACT_SILU>{});
+    else store_gateup(EpiAct<STMOE_ACT_GELU_ERF>{});
+  } else {
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) {
+      const int r = wm * 64 + tj * 16 + n_in;
+      if (r < rows_here) {
+        T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo;
 #pragma unroll
         for (int ti = 0; ti < 8; ++ti)
           *reinterpret_cast<uint2*>(orow + (int64_t)ntile * BN + wn * 128 + ti * 16 + 4 * g) =

@@ -27,6 +27,8 @@ static constexpr int BIG_LS = BIG_BK;  // LDS row stride (elements): 128 bytes =
 // distinct 16-byte bank groups for the operand reads, the weight-row writes and the token-row writes alike.
 __device__ __forceinline__ int lds_off(int row, int unit) { return row * BIG_LS + ((unit ^ (row & 7)) << 3); }
 
+template <int A> struct EpiAct { static constexpr int value = A; };
+
 // ---- work distribution ---------------------------------------------------------------------------------
 // Token tiles are the full ones (BM rows) and the partial ones (the last rows of an expert).  A unit is one token
 // tile times one feature tile.  Workgroup ids are dealt round-robin to the 8 XCDs; XCD i takes the i-th eighth of
