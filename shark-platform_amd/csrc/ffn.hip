@@ -57,7 +57,7 @@ static int run_projection(int variant, int dtype, int wtag, int mode, const Gemm
     else variant = max_rows >= 512 ? 6 : 2;
   }
   if (variant == 6) {
-    int rc = launch_mfma_ws(dtype, wtag, mode, p, max_rows, st);
+    int rc = launch_mfma_ws(dtype, wtag, mode, p, max_rows, p.split_scratch, st);
     if (rc != STMOE_ERR_UNSUPPORTED) return rc;
     variant = 4;
   }
@@ -87,7 +87,7 @@ using namespace stmoe;
 // Workspace of the grouped FFN: the intermediate z [T*k, N] in `dtype`, then (used only with quantised activations)
 // the quantised or re-dequantised copy of x [T, K] and the quantised intermediate [T*k, N] bytes.
 struct FfnWs {
-  size_t z, xa, zq, total;
+  size_t z, xa, zq, split, total;
 };
 static FfnWs carve_ffn(int64_t T, int k, int64_t K, int64_t N, int dtype) {
   FfnWs w{};
@@ -95,7 +95,9 @@ static FfnWs carve_ffn(int64_t T, int k, int64_t K, int64_t N, int dtype) {
   w.z = 0;
   w.xa = align_up((size_t)T * k * N * es, 256);
   w.zq = w.xa + align_up((size_t)T * K * es, 256);
-  w.total = w.zq + align_up((size_t)T * k * N, 256);
+  w.split = w.zq + align_up((size_t)T * k * N, 256);
+  // fp32 partial tiles of split reductions (prefill kernels only)
+  w.total = w.split + (T * k >= 512 ? align_up(mfma_ws_partial_bytes(), 256) : 0);
   return w;
 }
 
@@ -178,6 +180,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   q.a = z; q.lda = N; q.perm = nullptr; q.k_top = 1; q.offsets = offsets; q.E = E; q.fixed_rows = 0;
   q.w0 = make_view(w_down); q.w1 = q.w0;
   q.out = y_sorted; q.ldo = K; q.n_out = K; q.kred = N; q.act = act; q.x_scale = nullptr; q.expert_rows_bound = T;
+  q.split_scratch = ws.total > ws.split ? reinterpret_cast<float*>(base + ws.split) : nullptr;
   mark(events, 2, st);
   if (z_scale) {
     if (mfma8_out && !mfma8_in) rc = stmoe_quantize_fp8(z, dtype, z_scale, rows * N, zq, stream);

@@ -30,6 +30,7 @@ struct GemmParams {
   const float* x_scale;   // optional scale applied to the fp32 dot products (fp8 activations)
   const float* out_scale; // fp8 kernel only: quantise the result with this reciprocal scale and store e4m3fn bytes
   int64_t expert_rows_bound;  // host-side bound of rows per expert (a token gives an expert at most one row)
+  float* split_scratch;       // optional fp32 scratch for split reductions (mfma_ws_partial_bytes() bytes)
 };
 
 // (expert, first row, end row) of m-tile `slot` when every expert's rows are cut into tiles of BM.
@@ -109,7 +110,8 @@ namespace stmoe {
 int launch_generic(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_mfma_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_mfma_big(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
-int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
+int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, float* partial, hipStream_t st);
+size_t mfma_ws_partial_bytes();
 int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_fp8_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 }  // namespace stmoe

@@ -49,7 +49,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
   const int wn = wave / WM, wm = wave % WM;
 
   BigTile tile;
-  if (!big_tile_id(p, BM, n_tiles, tile)) return;
+  if (!big_tile_id(p, BM, n_tiles, false, tile)) return;
   const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
 
@@ -290,7 +290,7 @@ static int launch_big_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;
-  kern<<<dim3((unsigned)big_grid(n_tiles, m_slots)), 64 * WN * WM, lds_bytes, st>>>(p, n_tiles);
+  kern<<<dim3((unsigned)big_grid(n_tiles, m_slots, false)), 64 * WN * WM, lds_bytes, st>>>(p, n_tiles);
   return check_launch("grouped_mfma_big");
 }
 

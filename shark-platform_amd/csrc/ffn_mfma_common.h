@@ -38,46 +38,73 @@ template <int A> struct EpiAct { static constexpr int value = A; };
 // weight slab at the same time and share it in the XCD's L2.
 struct BigTile {
   int e, row_begin, row_end, ntile;
+  int chunk, nchunks;  // this workgroup's part of the reduction (0 of 1 unless the unit is split)
+  int chunk_slot;      // index of the fp32 partial tile of a split unit's chunk
 };
-__device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_tiles, BigTile& t) {
-  int F = 0, R = 0;
+// A launch whose units do not fill a whole number of rounds over the 32 CUs of an XCD leaves most CUs idle while the
+// last few units run.  With `allow_split` those last units (the partial token tiles come last) are cut along the
+// reduction into 4 (at most 8 left over) or 2 (at most 16) chunks that run on separate CUs and write fp32 partial
+// tiles; big_reduce_kernel adds the chunks in order.  Everything is a pure function of the offsets, so the result is
+// the same on every run.
+static constexpr int kBigCusPerXcd = 32;
+static constexpr int kBigChunkSlotsPerXcd = 32;  // rest * chunks <= 32
+struct BigPlan {
+  int F, R, f0, f1, r0, r1, whole, rest, chunks;
+};
+__device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int BM, int n_tiles, int xcd, bool allow_split) {
+  BigPlan pl;
+  pl.F = 0;
+  pl.R = 0;
   if (p.offsets) {
     for (int e = 0; e < p.E; ++e) {
       const int rows = p.offsets[e + 1] - p.offsets[e];
-      F += rows / BM;
-      R += (rows % BM) != 0;
+      pl.F += rows / BM;
+      pl.R += (rows % BM) != 0;
     }
   } else {
-    F = (int)(p.fixed_rows / BM);
-    R = (p.fixed_rows % BM) != 0;
+    pl.F = (int)(p.fixed_rows / BM);
+    pl.R = (p.fixed_rows % BM) != 0;
   }
-  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
-  const int UF = F * n_tiles, UR = R * n_tiles;
-  const int f0 = (int)((int64_t)UF * xcd / 8), f1 = (int)((int64_t)UF * (xcd + 1) / 8);
-  const int r0 = (int)((int64_t)UR * xcd / 8), r1 = (int)((int64_t)UR * (xcd + 1) / 8);
+  const int UF = pl.F * n_tiles, UR = pl.R * n_tiles;
+  pl.f0 = (int)((int64_t)UF * xcd / 8);
+  pl.f1 = (int)((int64_t)UF * (xcd + 1) / 8);
+  pl.r0 = (int)((int64_t)UR * xcd / 8);
+  pl.r1 = (int)((int64_t)UR * (xcd + 1) / 8);
+  const int n = (pl.f1 - pl.f0) + (pl.r1 - pl.r0);
+  pl.whole = n;
+  pl.rest = 0;
+  pl.chunks = 1;
+  if (allow_split) {
+    const int rest = n % kBigCusPerXcd;
+    const int chunks = rest == 0 ? 1 : (rest <= 8 ? 4 : (rest <= 16 ? 2 : 1));
+    if (chunks > 1) {
+      pl.whole = n - rest;
+      pl.rest = rest;
+      pl.chunks = chunks;
+    }
+  }
+  return pl;
+}
+// Unit number `unit` of the XCD's list (full units, then partial ones; token tile index fastest inside each class).
+__device__ __forceinline__ bool big_unit(const GemmParams& p, int BM, int n_tiles, const BigPlan& pl, int unit, BigTile& t) {
   int u, cnt;
   bool partial;
-  if (j < f1 - f0) {
-    u = f0 + j;
-    cnt = F;
+  if (unit < pl.f1 - pl.f0) {
+    u = pl.f0 + unit;
+    cnt = pl.F;
     partial = false;
-  } else if (j - (f1 - f0) < r1 - r0) {
-    u = r0 + j - (f1 - f0);
-    cnt = R;
+  } else if (unit - (pl.f1 - pl.f0) < pl.r1 - pl.r0) {
+    u = pl.r0 + unit - (pl.f1 - pl.f0);
+    cnt = pl.R;
     partial = true;
   } else {
     return false;
   }
-#ifdef STMOE_BIG_SLOT_MAJOR
-  int s = u / n_tiles;
-  t.ntile = u - s * n_tiles;
-#else
   t.ntile = u / cnt;
   int s = u - t.ntile * cnt;
-#endif
   if (!p.offsets) {
     t.e = 0;
-    t.row_begin = partial ? F * BM : s * BM;
+    t.row_begin = partial ? pl.F * BM : s * BM;
     t.row_end = partial ? (int)p.fixed_rows : t.row_begin + BM;
     return true;
   }
@@ -104,8 +131,30 @@ __device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_t
   }
   return false;
 }
-// Grid size that covers every XCD's share for at most `slots_bound` token tiles.
-static inline int big_grid(int n_tiles, int slots_bound) { return 8 * ((n_tiles * slots_bound + 7) / 8 + 2); }
+__device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_tiles, bool allow_split, BigTile& t) {
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  const BigPlan pl = big_plan(p, BM, n_tiles, xcd, allow_split);
+  int unit;
+  if (j < pl.whole) {
+    unit = j;
+    t.chunk = 0;
+    t.nchunks = 1;
+    t.chunk_slot = 0;
+  } else {
+    const int c = j - pl.whole;
+    if (c >= pl.rest * pl.chunks) return false;
+    unit = pl.whole + c / pl.chunks;
+    t.chunk = c % pl.chunks;
+    t.nchunks = pl.chunks;
+    t.chunk_slot = xcd * kBigChunkSlotsPerXcd + c;
+  }
+  return big_unit(p, BM, n_tiles, pl, unit, t);
+}
+// Grid size that covers every XCD's share for at most `slots_bound` token tiles (a split adds up to 24 workgroups).
+static inline int big_grid(int n_tiles, int slots_bound, bool allow_split) {
+  return 8 * ((n_tiles * slots_bound + 7) / 8 + 2 + (allow_split ? 24 : 0));
+}
+static inline size_t big_partial_bytes(int BN, int BM) { return (size_t)8 * kBigChunkSlotsPerXcd * BN * BM * sizeof(float); }
 
 // ---- hand-issued vector-memory operations ------------------------------------------------------------
 // Lane l's 16 bytes at base + byte_off land at LDS byte address lds_addr + 16*l (base and lds_addr wave-uniform).

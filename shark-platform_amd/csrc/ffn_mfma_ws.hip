@@ -20,7 +20,7 @@ template <int V> struct WsInt { static constexpr int value = V; };
 
 template <typename T, int WF, int MODE>
 __global__ void __launch_bounds__(768, 1)
-grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
+grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   constexpr int BN = 256, BM = 256;
   constexpr int WSTAGE = BN * BIG_LS, XSTAGE = BM * BIG_LS;  // elements
   constexpr int WPIECES = 4;   // packed weight pieces per producer per K step (16 row tiles / 4 producers)
@@ -31,10 +31,12 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
   const int g = lane >> 4, n_in = lane & 15;
 
   BigTile tile;
-  if (!big_tile_id(p, BM, n_tiles, tile)) return;
+  if (!big_tile_id(p, BM, n_tiles, partial != nullptr, tile)) return;
   const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
-  const int64_t nkt = p.kred >> 6;
+  // this workgroup's K steps: all of them, or one chunk of a split unit
+  const int64_t kt0 = (p.kred >> 6) * tile.chunk / tile.nchunks;
+  const int64_t nkt = (p.kred >> 6) * (tile.chunk + 1) / tile.nchunks - kt0;
 
   uint16_t* const Wbase = lds;               // [2][BN][64]
   uint16_t* const Xbase = lds + 2 * WSTAGE;  // [3][BM][64]
@@ -80,7 +82,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
       constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
       for (int j = 0; j < WPIECES; ++j) {
-        wreg[SET][j].load(waddr[j], kt);
+        wreg[SET][j].load(waddr[j], kt0 + kt);
       }
     };
     auto store_w = [&](auto set_tag, auto stage_tag) {
@@ -98,7 +100,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
       constexpr int XS = decltype(xstage_tag)::value;
 #pragma unroll
       for (int j = 0; j < XLOADS; ++j)
-        vm_load16_to_lds(p.a, xoff[j] + (uint32_t)kt * (BIG_BK * 2), x_lds0 + (uint32_t)((XS * XSTAGE + 32 * j * BIG_LS) * 2));
+        vm_load16_to_lds(p.a, xoff[j] + (uint32_t)(kt0 + kt) * (BIG_BK * 2), x_lds0 + (uint32_t)((XS * XSTAGE + 32 * j * BIG_LS) * 2));
     };
     // K step kt (R = kt % 6 fixes every stage and register set at compile time): store the weights of step kt + 1
     // (register set (kt+1) % 3, loaded during step kt - 3) into weight stage (kt+1) % 2, issue the token loads of step
@@ -218,7 +220,21 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
       }
     }
   };
-  if (MODE == MODE_GATEUP) {
+  if (tile.nchunks > 1) {
+    // chunk of a split unit: fp32 partial tile [BM][BN], added to the other chunks by big_reduce_kernel
+    float* pt = partial + (size_t)tile.chunk_slot * (BN * BM);
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) {
+      const int r = wm * 64 + tj * 16 + n_in;
+      if (r < rows_here) {
+#pragma unroll
+        for (int ti = 0; ti < 8; ++ti) {
+          const int col = (MODE == MODE_GATEUP ? (ti < 4 ? 0 : BN / 2) + wn * 64 + (ti & 3) * 16 : wn * 128 + ti * 16) + 4 * g;
+          *reinterpret_cast<floatx4_t*>(pt + r * BN + col) = acc[ti][tj];
+        }
+      }
+    }
+  } else if (MODE == MODE_GATEUP) {
     if (p.act == STMOE_ACT_SILU) store_gateup(EpiAct<STMOE_ACT_SILU>{});
     else store_gateup(EpiAct<STMOE_ACT_GELU_ERF>{});
   } else {
@@ -236,8 +252,32 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles) {
   }
 }
 
+// Adds the chunks of every split unit in chunk order and writes the rows (DOWN only).  Grid: (8 XCDs x 16 split units,
+// 8 blocks of 32 rows); the unit list is recomputed with the same plan as the main kernel.
+template <typename T>
+__global__ void __launch_bounds__(256) big_reduce_kernel(GemmParams p, int n_tiles, const float* partial) {
+  constexpr int BN = 256, BM = 256;
+  const int xcd = blockIdx.x >> 4, su = blockIdx.x & 15;
+  const BigPlan pl = big_plan(p, BM, n_tiles, xcd, true);
+  if (su >= pl.rest) return;
+  BigTile t;
+  if (!big_unit(p, BM, n_tiles, pl, pl.whole + su, t)) return;
+  const int rows_here = t.row_end - t.row_begin;
+  const int r = blockIdx.y * 32 + (threadIdx.x >> 3);
+  if (r >= rows_here) return;
+  const float* base = partial + (size_t)(xcd * kBigChunkSlotsPerXcd + su * pl.chunks) * (BN * BM) + r * BN;
+  T* orow = reinterpret_cast<T*>(p.out) + out_row(p, t.row_begin + r) * p.ldo + (int64_t)t.ntile * BN;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int col = ((threadIdx.x & 7) + 8 * j) * 4;
+    floatx4_t sum = *reinterpret_cast<const floatx4_t*>(base + col);
+    for (int c = 1; c < pl.chunks; ++c) sum = sum + *reinterpret_cast<const floatx4_t*>(base + (size_t)c * (BN * BM) + col);
+    *reinterpret_cast<uint2*>(orow + col) = make_uint2(pack2<T>(sum[0], sum[1]), pack2<T>(sum[2], sum[3]));
+  }
+}
+
 template <typename T, int WF, int MODE>
-static int launch_ws_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
+static int launch_ws_m(const GemmParams& p, int64_t max_rows, float* partial, hipStream_t st) {
   constexpr int BN = 256, BM = 256;
   constexpr size_t lds_bytes = (size_t)(2 * BN + 3 * BM) * BIG_LS * 2;
   static bool attr_set = false;
@@ -250,16 +290,25 @@ static int launch_ws_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;
-  kern<<<dim3((unsigned)big_grid(n_tiles, m_slots)), 768, lds_bytes, st>>>(p, n_tiles);
-  return check_launch("grouped_mfma_ws");
+  if (MODE == MODE_GATEUP) partial = nullptr;  // the gated product needs complete sums
+  kern<<<dim3((unsigned)big_grid(n_tiles, m_slots, partial != nullptr)), 768, lds_bytes, st>>>(p, n_tiles, partial);
+  int rc = check_launch("grouped_mfma_ws");
+  if (rc || !partial) return rc;
+  big_reduce_kernel<T><<<dim3(8 * 16, BM / 32), 256, 0, st>>>(p, n_tiles, partial);
+  return check_launch("big_reduce");
 }
 
 template <typename T, int WF>
-static int launch_ws_t(int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
-  return mode == MODE_GATEUP ? launch_ws_m<T, WF, MODE_GATEUP>(p, max_rows, st) : launch_ws_m<T, WF, MODE_DOWN>(p, max_rows, st);
+static int launch_ws_t(int mode, const GemmParams& p, int64_t max_rows, float* partial, hipStream_t st) {
+  return mode == MODE_GATEUP ? launch_ws_m<T, WF, MODE_GATEUP>(p, max_rows, partial, st)
+                             : launch_ws_m<T, WF, MODE_DOWN>(p, max_rows, partial, st);
 }
 
-int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
+size_t mfma_ws_partial_bytes() { return big_partial_bytes(256, 256); }
+
+// `partial`: optional fp32 scratch of mfma_ws_partial_bytes() bytes; with it the last units of a down projection that
+// would run on a few CUs only are split along the reduction.
+int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, float* partial, hipStream_t st) {
   if (max_rows == 0) return STMOE_OK;
   if (wtag != WF_Q8_0_P && wtag != WF_Q4_1_P && wtag != WF_FP8_F32D_P)
     return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs weights in a packed streaming order");
@@ -272,14 +321,14 @@ int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64
       return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: activations span 4 GB or more");
   }
   if (act_dtype == STMOE_F16) {
-    if (wtag == WF_Q8_0_P) return launch_ws_t<f16_t, WF_Q8_0_P>(mode, p, max_rows, st);
-    if (wtag == WF_Q4_1_P) return launch_ws_t<f16_t, WF_Q4_1_P>(mode, p, max_rows, st);
-    return launch_ws_t<f16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
+    if (wtag == WF_Q8_0_P) return launch_ws_t<f16_t, WF_Q8_0_P>(mode, p, max_rows, partial, st);
+    if (wtag == WF_Q4_1_P) return launch_ws_t<f16_t, WF_Q4_1_P>(mode, p, max_rows, partial, st);
+    return launch_ws_t<f16_t, WF_FP8_F32D_P>(mode, p, max_rows, partial, st);
   }
   if (act_dtype == STMOE_BF16) {
-    if (wtag == WF_Q8_0_P) return launch_ws_t<bf16_t, WF_Q8_0_P>(mode, p, max_rows, st);
-    if (wtag == WF_Q4_1_P) return launch_ws_t<bf16_t, WF_Q4_1_P>(mode, p, max_rows, st);
-    return launch_ws_t<bf16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
+    if (wtag == WF_Q8_0_P) return launch_ws_t<bf16_t, WF_Q8_0_P>(mode, p, max_rows, partial, st);
+    if (wtag == WF_Q4_1_P) return launch_ws_t<bf16_t, WF_Q4_1_P>(mode, p, max_rows, partial, st);
+    return launch_ws_t<bf16_t, WF_FP8_F32D_P>(mode, p, max_rows, partial, st);
   }
   return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: activation dtype %d", act_dtype);
 }

@@ -4,7 +4,8 @@ The CPU oracle cannot run these shapes in full in reasonable time, so each case 
   * routing indices of every token against the oracle (bit-exact; the router is cheap on the CPU),
   * the layer output of a sample of tokens against the oracle (tokens are independent given their own routing,
     so the oracle on a subset of rows is the full oracle restricted to those rows), within the stated tolerance,
-  * size-independent properties on all tokens: token-permutation equivariance (bit-exact), agreement of two
+  * size-independent properties on all tokens: token-permutation equivariance (routing bit-exact; outputs equal up to
+    the fp32 summation grouping of the few rows whose down-projection tile is split along the reduction), agreement of two
     kernel families, and run-to-run bit-identity (no float atomics).
 """
 
@@ -140,11 +141,15 @@ def test_config2_mixtral_q8_0_prefill_and_decode(device):
     y, idx, gate, block = run_layer(theta, pc, device)
     rows = list(range(0, 2048, 171))
     check_against_oracle(y, idx, pc, rows, 1e-3)
-    # permutation equivariance, bit-exact: every output row depends on its own token only and has a fixed k-order
+    # permutation equivariance: every output row depends on its own token only.  Routing is bit-exact; an output row
+    # changes in its last bits only if its down-projection tile is one of the last units of the launch in one order and
+    # not in the other (those units add four fp32 partial sums instead of one running sum)
     perm = torch.randperm(2048, generator=torch.Generator().manual_seed(1))
     y2, idx2, _ = block(pc["h"][perm].reshape(1, 2048, 4096).to(device), return_routing=True)
     assert torch.equal(idx2.cpu(), idx.cpu()[perm])
-    assert torch.equal(y2.reshape(2048, 4096).cpu().view(torch.int16), y.cpu()[perm].view(torch.int16))
+    a, b = y2.reshape(2048, 4096).cpu(), y.cpu()[perm]
+    assert O.rel_l2(a, b) < 1e-4
+    assert (a != b).float().mean().item() < 0.02
     # run-to-run identity
     y3 = block(pc["h"].reshape(1, 2048, 4096).to(device))
     assert torch.equal(y3.reshape(2048, 4096).view(torch.int16), y.view(torch.int16))
