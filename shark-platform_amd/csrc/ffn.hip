@@ -159,6 +159,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   p.a = x; p.lda = K; p.perm = perm; p.k_top = k; p.offsets = offsets; p.E = E; p.fixed_rows = 0;
   p.w0 = make_view(w_gate); p.w1 = make_view(w_up);
   p.out = z; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr; p.expert_rows_bound = T;
+  p.split_scratch = ws.total > ws.split ? reinterpret_cast<float*>(base + ws.split) : nullptr;
   mark(events, 0, st);
   if (x_scale) {
     if (mfma8_in) rc = stmoe_quantize_fp8(x, dtype, x_scale, T * K, xa, stream);

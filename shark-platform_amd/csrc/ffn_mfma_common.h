@@ -43,8 +43,8 @@ struct BigTile {
 };
 // A launch whose units do not fill a whole number of rounds over the 32 CUs of an XCD leaves most CUs idle while the
 // last few units run.  With `allow_split` those last units (the partial token tiles come last) are cut along the
-// reduction into 4 (at most 8 left over) or 2 (at most 16) chunks that run on separate CUs and write fp32 partial
-// tiles; big_reduce_kernel adds the chunks in order.  Everything is a pure function of the offsets, so the result is
+// reduction into up to 4 chunks (as many as keep units x chunks within the 32 CUs) that run on separate CUs and write
+// fp32 partial tiles; big_reduce_kernel adds the chunks in order.  Everything is a pure function of the offsets, so the result is
 // the same on every run.
 static constexpr int kBigCusPerXcd = 32;
 static constexpr int kBigChunkSlotsPerXcd = 32;  // rest * chunks <= 32
@@ -76,7 +76,7 @@ __device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int BM, int n_t
   pl.chunks = 1;
   if (allow_split) {
     const int rest = n % kBigCusPerXcd;
-    const int chunks = rest == 0 ? 1 : (rest <= 8 ? 4 : (rest <= 16 ? 2 : 1));
+    const int chunks = rest == 0 ? 1 : (kBigCusPerXcd / rest > 4 ? 4 : kBigCusPerXcd / rest);
     if (chunks > 1) {
       pl.whole = n - rest;
       pl.rest = rest;

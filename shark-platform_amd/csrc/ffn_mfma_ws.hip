@@ -252,9 +252,10 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   }
 }
 
-// Adds the chunks of every split unit in chunk order and writes the rows (DOWN only).  Grid: (8 XCDs x 16 split units,
-// 8 blocks of 32 rows); the unit list is recomputed with the same plan as the main kernel.
-template <typename T>
+// Adds the chunks of every split unit in chunk order and writes the rows: DOWN: the sums; GATEUP: the gated product of
+// the gate sums (columns 0..127 of the partial tile) and the up sums (columns 128..255).  Grid: (8 XCDs x 16 split
+// units, 8 blocks of 32 rows); the unit list is recomputed with the same plan as the main kernel.
+template <typename T, int MODE>
 __global__ void __launch_bounds__(256) big_reduce_kernel(GemmParams p, int n_tiles, const float* partial) {
   constexpr int BN = 256, BM = 256;
   const int xcd = blockIdx.x >> 4, su = blockIdx.x & 15;
@@ -266,13 +267,29 @@ __global__ void __launch_bounds__(256) big_reduce_kernel(GemmParams p, int n_til
   const int r = blockIdx.y * 32 + (threadIdx.x >> 3);
   if (r >= rows_here) return;
   const float* base = partial + (size_t)(xcd * kBigChunkSlotsPerXcd + su * pl.chunks) * (BN * BM) + r * BN;
-  T* orow = reinterpret_cast<T*>(p.out) + out_row(p, t.row_begin + r) * p.ldo + (int64_t)t.ntile * BN;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int col = ((threadIdx.x & 7) + 8 * j) * 4;
+  auto total = [&](int col) {
     floatx4_t sum = *reinterpret_cast<const floatx4_t*>(base + col);
     for (int c = 1; c < pl.chunks; ++c) sum = sum + *reinterpret_cast<const floatx4_t*>(base + (size_t)c * (BN * BM) + col);
-    *reinterpret_cast<uint2*>(orow + col) = make_uint2(pack2<T>(sum[0], sum[1]), pack2<T>(sum[2], sum[3]));
+    return sum;
+  };
+  T* orow = reinterpret_cast<T*>(p.out) + out_row(p, t.row_begin + r) * p.ldo;
+  if (MODE == MODE_GATEUP) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = ((threadIdx.x & 7) + 8 * j) * 4;
+      const floatx4_t gs = total(col), us = total(BN / 2 + col);
+      const float gq[4] = {gs[0], gs[1], gs[2], gs[3]}, uq[4] = {us[0], us[1], us[2], us[3]};
+      uint2* dst = reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * (BN / 2) + col);
+      if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq);
+      else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int col = ((threadIdx.x & 7) + 8 * j) * 4;
+      const floatx4_t sum = total(col);
+      *reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * BN + col) = make_uint2(pack2<T>(sum[0], sum[1]), pack2<T>(sum[2], sum[3]));
+    }
   }
 }
 
@@ -290,11 +307,10 @@ static int launch_ws_m(const GemmParams& p, int64_t max_rows, float* partial, hi
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;
-  if (MODE == MODE_GATEUP) partial = nullptr;  // the gated product needs complete sums
   kern<<<dim3((unsigned)big_grid(n_tiles, m_slots, partial != nullptr)), 768, lds_bytes, st>>>(p, n_tiles, partial);
   int rc = check_launch("grouped_mfma_ws");
   if (rc || !partial) return rc;
-  big_reduce_kernel<T><<<dim3(8 * 16, BM / 32), 256, 0, st>>>(p, n_tiles, partial);
+  big_reduce_kernel<T, MODE><<<dim3(8 * 16, BM / 32), 256, 0, st>>>(p, n_tiles, partial);
   return check_launch("big_reduce");
 }
 
@@ -306,8 +322,8 @@ static int launch_ws_t(int mode, const GemmParams& p, int64_t max_rows, float* p
 
 size_t mfma_ws_partial_bytes() { return big_partial_bytes(256, 256); }
 
-// `partial`: optional fp32 scratch of mfma_ws_partial_bytes() bytes; with it the last units of a down projection that
-// would run on a few CUs only are split along the reduction.
+// `partial`: optional fp32 scratch of mfma_ws_partial_bytes() bytes; with it the last units of a launch, which would
+// run on a few CUs only, are split along the reduction.
 int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, float* partial, hipStream_t st) {
   if (max_rows == 0) return STMOE_OK;
   if (wtag != WF_Q8_0_P && wtag != WF_Q4_1_P && wtag != WF_FP8_F32D_P)

@@ -326,8 +326,8 @@ def test_ffn_mfma_big_kernel(device, dtype, T, E, act):
         assert O.rel_l2(outs[variant], want) < tol
     assert O.rel_l2(outs[hip.VARIANT_MFMA_BIG], outs[hip.VARIANT_MFMA_TILE]) < tol
     # both 256 x 256 kernels accumulate every output in the same order, except that the specialised one splits the
-    # reduction of the last down-projection units of a launch into fp32 partial sums
-    assert O.rel_l2(outs[hip.VARIANT_MFMA_BIG], outs[hip.VARIANT_MFMA_WS]) < 1e-4
+    # reduction of the last units of a launch into fp32 partial sums (a different rounding of a few sums)
+    assert O.rel_l2(outs[hip.VARIANT_MFMA_BIG], outs[hip.VARIANT_MFMA_WS]) < tol / 4
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
