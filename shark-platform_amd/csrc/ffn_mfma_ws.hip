@@ -34,6 +34,10 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   if (!big_tile_id(p, BM, n_tiles, partial != nullptr, tile)) return;
   const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
+  // Rows per token-row group: the rows of a partial tile are spread evenly (in multiples of 16) over the four groups,
+  // so all consumers share the work and each only multiplies the 16-row column blocks it really has.  Tile row
+  // grp * rpg + i (i < rpg) lives in LDS row grp * 64 + i.  Full tiles: rpg = 64, the identity.
+  const int rpg = min(64, ((rows_here + 3) / 4 + 15) / 16 * 16);
   // this workgroup's K steps: all of them, or one chunk of a split unit
   const int64_t kt0 = (p.kred >> 6) * tile.chunk / tile.nchunks;
   const int64_t nkt = (p.kred >> 6) * (tile.chunk + 1) / tile.nchunks - kt0;
@@ -62,12 +66,12 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
       waddr[j].init(*wv, row0 >> 4, e, lane, p.kred);
     }
     // token rows: lane l of direct load j fills LDS row pw*8 + 32*j + l/8, unit l%8, from global unit (l%8) ^ (row & 7);
-    // rows past the end of the expert's rows re-read its last row (their outputs are never stored)
+    // LDS rows that hold no tile row re-read a valid row (their outputs are never stored)
     uint32_t xoff[XLOADS];
 #pragma unroll
     for (int j = 0; j < XLOADS; ++j) {
       const int lr = pw * 8 + 32 * j + (lane >> 3);
-      const int r = min(lr, rows_here - 1);
+      const int r = min((lr >> 6) * rpg + min(lr & 63, rpg - 1), rows_here - 1);
       const int i = row_begin + r;
       const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
       xoff[j] = (uint32_t)((src * p.lda + (((lane & 7) ^ (lr & 7)) << 3)) * 2);
@@ -168,39 +172,49 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   for (int a = 0; a < 8; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
-  const bool active = rows_here > wm * 64;  // wavefronts whose token rows are all past the end skip their MFMAs
+  const int my_rows = min(rpg, rows_here - wm * rpg);  // tile rows of this wavefront's group (<= 0: none)
+  const bool active = my_rows > 0;                     // wavefronts without rows skip their MFMAs
+  const int ntj = (my_rows + 15) >> 4;                 // 16-row column blocks that hold rows
 
-  auto compute = [&](auto parity_tag, int xstage, int ks) {
+  auto compute = [&](auto parity_tag, auto ntj_tag, int xstage, int ks) {
     constexpr int PAR = decltype(parity_tag)::value;
+    constexpr int NTJ = decltype(ntj_tag)::value;
     const uint16_t* bp = b_rd[ks] + xstage * XSTAGE;
-    u32x4_t bf[4];
+    u32x4_t bf[NTJ];
 #pragma unroll
-    for (int tj = 0; tj < 4; ++tj) bf[tj] = *reinterpret_cast<const u32x4_t*>(bp + tj * 16 * BIG_LS);
+    for (int tj = 0; tj < NTJ; ++tj) bf[tj] = *reinterpret_cast<const u32x4_t*>(bp + tj * 16 * BIG_LS);
 #pragma unroll
     for (int ti = 0; ti < 8; ++ti) {
       const int row_off = MODE == MODE_GATEUP ? (ti < 4 ? 0 : BN / 2) + (ti & 3) * 16 : ti * 16;
       const u32x4_t af = *reinterpret_cast<const u32x4_t*>(a_rd[ks] + PAR * WSTAGE + row_off * BIG_LS);
 #pragma unroll
-      for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = mfma16b<T>(af, bf[tj], acc[ti][tj]);
+      for (int tj = 0; tj < NTJ; ++tj) acc[ti][tj] = mfma16b<T>(af, bf[tj], acc[ti][tj]);
     }
   };
   __syncthreads();  // first stage filled
-  if (active) {
+  auto k_loop = [&](auto ntj_tag) {
     int xs = 0;
     for (int64_t kt = 0; kt < nkt; kt += 2) {
-      compute(WsInt<0>{}, xs, 0);
-      compute(WsInt<0>{}, xs, 1);
+      compute(WsInt<0>{}, ntj_tag, xs, 0);
+      compute(WsInt<0>{}, ntj_tag, xs, 1);
       __syncthreads();
       xs = xs == 2 ? 0 : xs + 1;
       if (kt + 1 < nkt) {
-        compute(WsInt<1>{}, xs, 0);
-        compute(WsInt<1>{}, xs, 1);
+        compute(WsInt<1>{}, ntj_tag, xs, 0);
+        compute(WsInt<1>{}, ntj_tag, xs, 1);
         __syncthreads();
         xs = xs == 2 ? 0 : xs + 1;
       }
     }
-  } else {
+  };
+  if (!active) {
     for (int64_t kt = 0; kt < nkt; ++kt) __syncthreads();
+  } else if (ntj == 1) {
+    k_loop(WsInt<1>{});
+  } else if (ntj == 2) {
+    k_loop(WsInt<2>{});
+  } else {
+    k_loop(WsInt<4>{});
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------------
@@ -208,8 +222,8 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
-      const int r = wm * 64 + tj * 16 + n_in;
-      if (r < rows_here) {
+      const int r = wm * rpg + tj * 16 + n_in;
+      if (tj * 16 + n_in < my_rows) {
         T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo + (int64_t)ntile * (BN / 2) + wn * 64 + 4 * g;
 #pragma unroll
         for (int ti = 0; ti < 4; ++ti) {
@@ -225,8 +239,8 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     float* pt = partial + (size_t)tile.chunk_slot * (BN * BM);
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
-      const int r = wm * 64 + tj * 16 + n_in;
-      if (r < rows_here) {
+      const int r = wm * rpg + tj * 16 + n_in;
+      if (tj * 16 + n_in < my_rows) {
 #pragma unroll
         for (int ti = 0; ti < 8; ++ti) {
           const int col = (MODE == MODE_GATEUP ? (ti < 4 ? 0 : BN / 2) + wn * 64 + (ti & 3) * 16 : wn * 128 + ti * 16) + 4 * g;
@@ -240,8 +254,8 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   } else {
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
-      const int r = wm * 64 + tj * 16 + n_in;
-      if (r < rows_here) {
+      const int r = wm * rpg + tj * 16 + n_in;
+      if (tj * 16 + n_in < my_rows) {
         T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo;
 #pragma unroll
         for (int ti = 0; ti < 8; ++ti)
