@@ -311,6 +311,7 @@ static int launch_big_t(int mode, const GemmParams& p, int64_t max_rows, hipStre
 
 int launch_mfma_big(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (max_rows == 0) return STMOE_OK;
+  if (p.offsets && p.E >= 64) return set_error(STMOE_ERR_UNSUPPORTED, "mfma big kernel: at most 63 experts");
   if (wtag != WF_Q8_0_P)
     return set_error(STMOE_ERR_UNSUPPORTED, "mfma big kernel: needs weights in the packed Q8_0 order");
   if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0 || p.n_out % (mode == MODE_GATEUP ? 64 * STMOE_BIG_WN : 128 * STMOE_BIG_WN) != 0)

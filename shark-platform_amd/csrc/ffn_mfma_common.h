@@ -51,13 +51,19 @@ static constexpr int kBigChunkSlotsPerXcd = 32;  // rest * chunks <= 32
 struct BigPlan {
   int F, R, f0, f1, r0, r1, whole, rest, chunks;
 };
-__device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int BM, int n_tiles, int xcd, bool allow_split) {
+// The offsets are fetched with one vector load (lane l holds offsets[l]) and read back with readlane: walking them with
+// scalar loads costs one memory latency per expert, twice per workgroup.  Needs E < 64 (checked by the launchers).
+__device__ __forceinline__ int big_lane_offsets(const GemmParams& p) {
+  const int lane = threadIdx.x & 63;
+  return (p.offsets && lane <= p.E) ? p.offsets[lane] : 0;
+}
+__device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int lane_off, int BM, int n_tiles, int xcd, bool allow_split) {
   BigPlan pl;
   pl.F = 0;
   pl.R = 0;
   if (p.offsets) {
     for (int e = 0; e < p.E; ++e) {
-      const int rows = p.offsets[e + 1] - p.offsets[e];
+      const int rows = __builtin_amdgcn_readlane(lane_off, e + 1) - __builtin_amdgcn_readlane(lane_off, e);
       pl.F += rows / BM;
       pl.R += (rows % BM) != 0;
     }
@@ -86,7 +92,7 @@ __device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int BM, int n_t
   return pl;
 }
 // Unit number `unit` of the XCD's list (full units, then partial ones; token tile index fastest inside each class).
-__device__ __forceinline__ bool big_unit(const GemmParams& p, int BM, int n_tiles, const BigPlan& pl, int unit, BigTile& t) {
+__device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int BM, int n_tiles, const BigPlan& pl, int unit, BigTile& t) {
   int u, cnt;
   bool partial;
   if (unit < pl.f1 - pl.f0) {
@@ -109,7 +115,7 @@ __device__ __forceinline__ bool big_unit(const GemmParams& p, int BM, int n_tile
     return true;
   }
   for (int e = 0; e < p.E; ++e) {
-    const int b = p.offsets[e], rows = p.offsets[e + 1] - b;
+    const int b = __builtin_amdgcn_readlane(lane_off, e), rows = __builtin_amdgcn_readlane(lane_off, e + 1) - b;
     if (!partial) {
       const int c = rows / BM;
       if (s < c) {
@@ -133,7 +139,8 @@ __device__ __forceinline__ bool big_unit(const GemmParams& p, int BM, int n_tile
 }
 __device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_tiles, bool allow_split, BigTile& t) {
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
-  const BigPlan pl = big_plan(p, BM, n_tiles, xcd, allow_split);
+  const int lane_off = big_lane_offsets(p);
+  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, allow_split);
   int unit;
   if (j < pl.whole) {
     unit = j;
@@ -148,7 +155,7 @@ __device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_t
     t.nchunks = pl.chunks;
     t.chunk_slot = xcd * kBigChunkSlotsPerXcd + c;
   }
-  return big_unit(p, BM, n_tiles, pl, unit, t);
+  return big_unit(p, lane_off, BM, n_tiles, pl, unit, t);
 }
 // Grid size that covers every XCD's share for at most `slots_bound` token tiles (a split adds up to 24 workgroups).
 static inline int big_grid(int n_tiles, int slots_bound, bool allow_split) {

@@ -273,10 +273,11 @@ template <typename T, int MODE>
 __global__ void __launch_bounds__(256) big_reduce_kernel(GemmParams p, int n_tiles, const float* partial) {
   constexpr int BN = 256, BM = 256;
   const int xcd = blockIdx.x >> 4, su = blockIdx.x & 15;
-  const BigPlan pl = big_plan(p, BM, n_tiles, xcd, true);
+  const int lane_off = big_lane_offsets(p);
+  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, true);
   if (su >= pl.rest) return;
   BigTile t;
-  if (!big_unit(p, BM, n_tiles, pl, pl.whole + su, t)) return;
+  if (!big_unit(p, lane_off, BM, n_tiles, pl, pl.whole + su, t)) return;
   const int rows_here = t.row_end - t.row_begin;
   const int r = blockIdx.y * 32 + (threadIdx.x >> 3);
   if (r >= rows_here) return;
@@ -340,6 +341,7 @@ size_t mfma_ws_partial_bytes() { return big_partial_bytes(256, 256); }
 // run on a few CUs only, are split along the reduction.
 int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, float* partial, hipStream_t st) {
   if (max_rows == 0) return STMOE_OK;
+  if (p.offsets && p.E >= 64) return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: at most 63 experts");
   if (wtag != WF_Q8_0_P && wtag != WF_Q4_1_P && wtag != WF_FP8_F32D_P)
     return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs weights in a packed streaming order");
   if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0 || p.n_out % (mode == MODE_GATEUP ? 128 : 256) != 0)
