@@ -75,20 +75,12 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
 }
 
 // ---- Q4_1 helpers ------------------------------------------------------------------------------------
-// f16(f16(d*q) + m) for a pair of nibbles given as fp16 numbers 1024 + q (bits 0x6400 | q).  d*q is formed as
-// fma(1024 + q, d, -1024*d): the fma rounds the exact value d*q once, like the multiply of the reference.  -1024*d
-// must be finite for that, so scales of magnitude >= 32 take the subtract-then-multiply form.
+// f16(f16(d*q) + m) for a pair of nibbles given as fp16 numbers 1024 + q (bits 0x6400 | q): the subtraction is exact,
+// the product of an fp16 scale and an integer below 16 rounds once like the reference's multiply, then the add.
 __device__ __forceinline__ uint32_t q4_pair_dequant(uint32_t pair_bits, uint32_t dbits, uint32_t mbits) {
   const half2_t dd = as_half2(dbits | (dbits << 16)), mm = as_half2(mbits | (mbits << 16));
-  half2_t v;
-  if (__builtin_expect((dbits & 0x7fffu) >= 0x5000u, 0)) {
-    const half2_t bias = {(f16_t)1024.0f, (f16_t)1024.0f};
-    v = (as_half2(pair_bits) - bias) * dd;
-  } else {
-    const half2_t nb = as_half2((dbits | (dbits << 16)) ^ 0x80008000u) * (half2_t){(f16_t)1024.0f, (f16_t)1024.0f};
-    v = __builtin_elementwise_fma(as_half2(pair_bits), dd, nb);
-  }
-  return as_u32(v + mm);
+  const half2_t bias = {(f16_t)1024.0f, (f16_t)1024.0f};
+  return as_u32((as_half2(pair_bits) - bias) * dd + mm);
 }
 // Pair p (elements 2p, 2p+1) of the 8 nibbles of a dword, as two fp16 numbers 1024 + q.
 //   linear order (planar planes): element i is nibble i
