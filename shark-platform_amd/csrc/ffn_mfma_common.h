@@ -166,6 +166,7 @@ static inline size_t big_partial_bytes(int BN, int BM) { return (size_t)8 * kBig
 // ---- hand-issued vector-memory operations ------------------------------------------------------------
 // Lane l's 16 bytes at base + byte_off land at LDS byte address lds_addr + 16*l (base and lds_addr wave-uniform).
 __device__ __forceinline__ void vm_load16_to_lds(const void* base, uint32_t byte_off, uint32_t lds_addr) {
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);  // the compiler cannot always prove it uniform
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(byte_off), "s"(base), "s"(lds_addr)
                : "memory", "m0");
 }

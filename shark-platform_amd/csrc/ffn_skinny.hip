@@ -16,7 +16,7 @@
 //   Q4_1 (1/2 byte):       lane (n, g) load i covers block 4*i + g (32 k); steps 4i .. 4i+3 take 4 bytes each.
 //                          Token operand: x[m][128*i + 32*g .. +31].
 //   16-bit dense:          as the 1-byte case with 32-byte loads.
-#include "ffn_kernels.h"
+#include "ffn_mfma_common.h"
 
 namespace stmoe {
 
@@ -61,6 +61,7 @@ template <int WF> __device__ __forceinline__ int x_offset(int s, int g) {
 template <> struct SkinnyW<WF_Q8_0> {
   u32x4_t q[4];
   u32x4_t d;  // the chunk's 8 block scales
+  __device__ __forceinline__ void touch() { asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]), "+v"(d)); }
   __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
     const uint8_t* base = w.qs + row * w.cols + c * 256 + 16 * g;
 #pragma unroll
@@ -89,6 +90,7 @@ template <> struct SkinnyW<WF_Q8_0> {
 template <> struct SkinnyW<WF_Q4_1> {
   u32x4_t q[2];
   uint16_t d[2], m[2];  // scale / offset of the lane's own two blocks (4*i + g, i = 0, 1)
+  __device__ __forceinline__ void touch() { asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(d[0]), "+v"(d[1]), "+v"(m[0]), "+v"(m[1])); }
   __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
     const uint8_t* base = w.qs + ((row * w.cols + c * 256) >> 1) + 16 * g;
 #pragma unroll
@@ -117,6 +119,7 @@ template <> struct SkinnyW<WF_Q4_1> {
 template <> struct SkinnyW<WF_FP8_F32D> {
   u32x4_t q[4];
   float dv;
+  __device__ __forceinline__ void touch() { asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]), "+v"(dv)); }
   __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
     const uint8_t* base = w.qs + row * w.cols + c * 256 + 16 * g;
 #pragma unroll
@@ -177,6 +180,7 @@ template <> struct SkinnyW<WF_FP8_F32D_P> : SkinnyW<WF_FP8_F32D> {
 
 template <bool BF> struct SkinnyWDense16 {
   u32x4_t q[8];
+  __device__ __forceinline__ void touch() {}
   __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
     const uint8_t* base = w.qs + (row * w.cols + c * 256 + 16 * g) * 2;
 #pragma unroll
@@ -324,6 +328,9 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
   }
 }
 
+// The packed formats use the LDS-shared variant.
+template <int WF> struct SkinnyUsesLds { static constexpr bool value = WF == WF_Q8_0_P || WF == WF_Q4_1_P || WF == WF_FP8_F32D_P; };
+
 // Workgroups resident per CU (two wavefronts per SIMD: the double-buffered chunks need about 200 registers).
 template <int WF> struct SkinnyOcc { static constexpr int value = 2; };
 
@@ -378,6 +385,155 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
   }
 }
 
+// ---- variant with the token rows shared through LDS ------------------------------------------------------
+// Feeding the token operand straight from global memory costs one cache-line access per token row and MFMA step pair
+// in every wavefront, and those accesses, not HBM, bound the kernel above.  Here the four wavefronts of a workgroup
+// take four neighbouring items of one expert (the same token rows): per chunk of 256 reduction elements the rows
+// go global -> LDS once per workgroup with fully coalesced direct loads (global_load_lds_dwordx4, one chunk ahead,
+// two LDS stages, one barrier per chunk) and every wavefront reads its MFMA operands from LDS.  LDS rows are 512 bytes;
+// the 16-byte unit u of row r lives at unit u ^ (r & 15), which makes the operand reads of 16 rows conflict-free and
+// is applied on the source side of the direct loads.  Weights are handled as above (registers, one chunk ahead).
+template <typename T, int WF, int MODE, int MT>
+__device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64_t (&wrow)[2], int tile, int r0, int re,
+                                                int64_t nch, int lane, int wave, uint16_t* xs, uint32_t xs_addr) {
+  constexpr int NT = 2;
+  constexpr int XROWS = 16 * MT, XSTAGE = XROWS * 256;  // elements
+  constexpr int XL = XROWS / 8;                         // direct loads (2 rows each) per wavefront per chunk
+  const int g = lane >> 4, n_in = lane & 15;
+  uint32_t xoff[XL];  // byte offsets from p.a (the host checks that the activations span less than 4 GB)
+#pragma unroll
+  for (int j = 0; j < XL; ++j) {
+    const int lr = 2 * (wave * XL + j) + (lane >> 5);  // LDS row; rows past the end re-read the last row (never stored)
+    const int i = min(r0 + lr, re - 1);
+    const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
+    xoff[j] = (uint32_t)((src * p.lda + (((lane & 31) ^ (lr & 15)) << 3)) * 2);
+  }
+  auto load_x = [&](int stage, int64_t c) {
+#pragma unroll
+    for (int j = 0; j < XL; ++j)
+      vm_load16_to_lds(p.a, xoff[j] + (uint32_t)c * 512u, xs_addr + (uint32_t)((stage * XSTAGE + 2 * (wave * XL + j) * 256) * 2));
+  };
+  floatx4_t acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[mt][t] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+  SkinnyW<WF> w0[NT], w1[NT];
+  auto load_w = [&](SkinnyW<WF>* w, int64_t c) {
+    w[0].load(p.w0, wrow[0], c, g);
+    w[1].load(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1], c, g);
+  };
+  auto compute = [&](const SkinnyW<WF>* w, int stage) {
+    const uint16_t* xb = xs + stage * XSTAGE + n_in * 256;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      u32x4_t xf[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        xf[mt] = *reinterpret_cast<const u32x4_t*>(xb + mt * 16 * 256 + (((x_offset<WF>(s, g) >> 3) ^ n_in) << 3));
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const u32x4_t wf = w[t].template frag<T>(s, g);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[mt][t] = mfma16s<T>(wf, xf[mt], acc[mt][t]);
+      }
+    }
+  };
+  // After the hand-written wait every load has landed; naming the weight registers as operands of an empty statement
+  // makes the compiler place its own waits for them here, where they cost nothing, instead of in front of the next
+  // chunk's MFMAs, where they would also wait for the token loads issued in between.
+  auto arrived = [&](SkinnyW<WF>* w) {
+    vm_wait<0>();
+#pragma unroll
+    for (int t = 0; t < NT; ++t) w[t].touch();
+    __syncthreads();
+  };
+  load_x(0, 0);
+  load_w(w0, 0);
+  arrived(w0);
+  for (int64_t c = 0; c < nch; c += 2) {
+    if (c + 1 < nch) {
+      load_x(1, c + 1);
+      load_w(w1, c + 1);
+    }
+    compute(w0, 0);
+    arrived(w1);
+    if (c + 1 < nch) {
+      if (c + 2 < nch) {
+        load_x(0, c + 2);
+        load_w(w0, c + 2);
+      }
+      compute(w1, 1);
+      arrived(w0);
+    }
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int i = r0 + mt * 16 + n_in;
+    if (i < re) {
+      T* orow = reinterpret_cast<T*>(p.out) + out_row(p, i) * p.ldo;
+      if (MODE == MODE_GATEUP) {
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = gateup_epilogue<T>(p.act, acc[mt][0][r], acc[mt][1][r], 1.0f);
+        *reinterpret_cast<uint2*>(orow + tile * 16 + 4 * g) = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
+      } else {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          *reinterpret_cast<uint2*>(orow + tile * 32 + t * 16 + 4 * g) =
+              make_uint2(pack2<T>(acc[mt][t][0], acc[mt][t][1]), pack2<T>(acc[mt][t][2], acc[mt][t][3]));
+      }
+    }
+  }
+}
+
+// A workgroup takes groups of four neighbouring items (tiles 4q .. 4q+3 of one expert), strided by the grid size.
+template <typename T, int WF, int MODE>
+__global__ void __launch_bounds__(256, 2)
+grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
+  __shared__ __align__(16) uint16_t xs[2 * 32 * 256];  // two stages of up to 32 token rows x 256 reduction elements
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n_in = lane & 15;
+  const int64_t nch = p.kred >> 8;
+  const uint32_t xs_addr = __builtin_amdgcn_readfirstlane(
+      (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)xs));
+  int n_active = 0;
+  uint64_t active_mask = 0;
+  for (int e = 0; e < p.E; ++e)
+    if (p.offsets[e + 1] > p.offsets[e]) {
+      active_mask |= 1ull << e;
+      ++n_active;
+    }
+  const int groups_per_expert = tiles_per_expert >> 2;
+  const int n_groups = n_active * groups_per_expert;
+  for (int grp = blockIdx.x; grp < n_groups; grp += gridDim.x) {
+    const int a_idx = grp / groups_per_expert, tile = (grp - a_idx * groups_per_expert) * 4 + wave;
+    int e = 0;
+    {
+      int seen = 0;
+      for (int ee = 0; ee < p.E; ++ee)
+        if ((active_mask >> ee) & 1ull) {
+          if (seen == a_idx) { e = ee; break; }
+          ++seen;
+        }
+    }
+    const int rb = p.offsets[e], re = p.offsets[e + 1];
+    int64_t wrow[2];
+    if (MODE == MODE_GATEUP) {
+      wrow[0] = (int64_t)e * p.w0.rows + tile * 16 + n_in;
+      wrow[1] = (int64_t)e * p.w1.rows + tile * 16 + n_in;
+    } else {
+      wrow[0] = (int64_t)e * p.w0.rows + tile * 32 + n_in;
+      wrow[1] = wrow[0] + 16;
+    }
+    if (re - rb <= 16) {
+      skinny_lds_pass<T, WF, MODE, 1>(p, wrow, tile, rb, re, nch, lane, wave, xs, xs_addr);
+    } else {
+      for (int r0 = rb; r0 < re; r0 += 32) skinny_lds_pass<T, WF, MODE, 2>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
+    }
+  }
+}
+
 static int pick_waves(int64_t items, int wg_per_cu) {
   // 256 CUs x resident workgroups x 4 wavefronts; give every wavefront the same number of items
   const int64_t capacity = 1024 * wg_per_cu;
@@ -399,6 +555,21 @@ static int launch_skinny_t(int mode, const GemmParams& p, int64_t max_rows, hipS
     if (mode == MODE_GATEUP) grouped_skinny_kernel<T, WF, MODE_GATEUP, 4><<<grid, 256, 0, st>>>(p, tiles, (int)items_bound);
     else grouped_skinny_kernel<T, WF, MODE_DOWN, 4><<<grid, 256, 0, st>>>(p, tiles, (int)items_bound);
     return check_launch("grouped_skinny(split)");
+  }
+  {
+    // token rows shared through LDS: needs whole groups of four tiles and 32-bit token offsets.  The down projection
+    // has four times fewer groups than the gate/up projection; with few rows per expert (one token tile, few loads to
+    // share) it is better off with independent wavefronts.
+    const int64_t src_rows = p.perm ? (max_rows + p.k_top - 1) / p.k_top : max_rows;
+    const bool worth = mode == MODE_GATEUP || max_rows > 12 * (int64_t)p.E;
+    if constexpr (SkinnyUsesLds<WF>::value) if (worth && tiles % 4 == 0 && src_rows * p.lda * 2 < ((int64_t)1 << 32)) {
+      const int64_t groups = (int64_t)(tiles / 4) * p.E, capacity = 256 * 2;
+      const int64_t per_wg = (groups + capacity - 1) / capacity;
+      dim3 grid((unsigned)((groups + per_wg - 1) / per_wg));
+      if (mode == MODE_GATEUP) grouped_skinny_lds_kernel<T, WF, MODE_GATEUP><<<grid, 256, 0, st>>>(p, tiles);
+      else grouped_skinny_lds_kernel<T, WF, MODE_DOWN><<<grid, 256, 0, st>>>(p, tiles);
+      return check_launch("grouped_skinny_lds");
+    }
   }
   const int waves = pick_waves((int64_t)tiles * p.E, SkinnyOcc<WF>::value);
   dim3 grid((unsigned)(waves / 4));
