@@ -393,12 +393,14 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
 // two LDS stages, one barrier per chunk) and every wavefront reads its MFMA operands from LDS.  LDS rows are 512 bytes;
 // the 16-byte unit u of row r lives at unit u ^ (r & 15), which makes the operand reads of 16 rows conflict-free and
 // is applied on the source side of the direct loads.  Weights are handled as above (registers, one chunk ahead).
-template <typename T, int WF, int MODE, int MT>
+template <typename T, int WF, int MODE, int MT, int G>
 __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64_t (&wrow)[2], int tile, int r0, int re,
                                                 int64_t nch, int lane, int wave, uint16_t* xs, uint32_t xs_addr) {
+  // G chunks of 256 reduction elements form one pipeline step (G = 2 for the 4-bit format, whose chunks are half
+  // as many bytes, so that as many bytes are in flight per wavefront as for the 8-bit formats)
   constexpr int NT = 2;
-  constexpr int XROWS = 16 * MT, XSTAGE = XROWS * 256;  // elements
-  constexpr int XL = XROWS / 8;                         // direct loads (2 rows each) per wavefront per chunk
+  constexpr int XROWS = 16 * MT, XCHUNK = XROWS * 256, XSTAGE = G * XCHUNK;  // elements
+  constexpr int XL = XROWS / 8;                                             // direct loads (2 rows each) per wavefront per chunk
   const int g = lane >> 4, n_in = lane & 15;
   uint32_t xoff[XL];  // byte offsets from p.a (the host checks that the activations span less than 4 GB)
 #pragma unroll
@@ -408,60 +410,71 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
     const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
     xoff[j] = (uint32_t)((src * p.lda + (((lane & 31) ^ (lr & 15)) << 3)) * 2);
   }
-  auto load_x = [&](int stage, int64_t c) {
+  auto load_x = [&](int stage, int64_t c) {  // chunks c .. c + G - 1
 #pragma unroll
-    for (int j = 0; j < XL; ++j)
-      vm_load16_to_lds(p.a, xoff[j] + (uint32_t)c * 512u, xs_addr + (uint32_t)((stage * XSTAGE + 2 * (wave * XL + j) * 256) * 2));
+    for (int q = 0; q < G; ++q)
+#pragma unroll
+      for (int j = 0; j < XL; ++j)
+        vm_load16_to_lds(p.a, xoff[j] + (uint32_t)(c + q) * 512u,
+                         xs_addr + (uint32_t)((stage * XSTAGE + q * XCHUNK + 2 * (wave * XL + j) * 256) * 2));
   };
   floatx4_t acc[MT][NT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[mt][t] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
-  SkinnyW<WF> w0[NT], w1[NT];
-  auto load_w = [&](SkinnyW<WF>* w, int64_t c) {
-    w[0].load(p.w0, wrow[0], c, g);
-    w[1].load(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1], c, g);
+  SkinnyW<WF> w0[G][NT], w1[G][NT];
+  auto load_w = [&](SkinnyW<WF> (*w)[NT], int64_t c) {
+#pragma unroll
+    for (int q = 0; q < G; ++q) {
+      w[q][0].load(p.w0, wrow[0], c + q, g);
+      w[q][1].load(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1], c + q, g);
+    }
   };
-  auto compute = [&](const SkinnyW<WF>* w, int stage) {
-    const uint16_t* xb = xs + stage * XSTAGE + n_in * 256;
+  auto compute = [&](const SkinnyW<WF> (*w)[NT], int stage) {
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      u32x4_t xf[MT];
+    for (int q = 0; q < G; ++q) {
+      const uint16_t* xb = xs + stage * XSTAGE + q * XCHUNK + n_in * 256;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        xf[mt] = *reinterpret_cast<const u32x4_t*>(xb + mt * 16 * 256 + (((x_offset<WF>(s, g) >> 3) ^ n_in) << 3));
+      for (int s = 0; s < 8; ++s) {
+        u32x4_t xf[MT];
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const u32x4_t wf = w[t].template frag<T>(s, g);
+        for (int mt = 0; mt < MT; ++mt)
+          xf[mt] = *reinterpret_cast<const u32x4_t*>(xb + mt * 16 * 256 + (((x_offset<WF>(s, g) >> 3) ^ n_in) << 3));
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc[mt][t] = mfma16s<T>(wf, xf[mt], acc[mt][t]);
+        for (int t = 0; t < NT; ++t) {
+          const u32x4_t wf = w[q][t].template frag<T>(s, g);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[mt][t] = mfma16s<T>(wf, xf[mt], acc[mt][t]);
+        }
       }
     }
   };
   // After the hand-written wait every load has landed; naming the weight registers as operands of an empty statement
   // makes the compiler place its own waits for them here, where they cost nothing, instead of in front of the next
-  // chunk's MFMAs, where they would also wait for the token loads issued in between.
-  auto arrived = [&](SkinnyW<WF>* w) {
+  // step's MFMAs, where they would also wait for the token loads issued in between.
+  auto arrived = [&](SkinnyW<WF> (*w)[NT]) {
     vm_wait<0>();
 #pragma unroll
-    for (int t = 0; t < NT; ++t) w[t].touch();
+    for (int q = 0; q < G; ++q)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) w[q][t].touch();
     __syncthreads();
   };
   load_x(0, 0);
   load_w(w0, 0);
   arrived(w0);
-  for (int64_t c = 0; c < nch; c += 2) {
-    if (c + 1 < nch) {
-      load_x(1, c + 1);
-      load_w(w1, c + 1);
+  for (int64_t c = 0; c < nch; c += 2 * G) {
+    if (c + G < nch) {
+      load_x(1, c + G);
+      load_w(w1, c + G);
     }
     compute(w0, 0);
     arrived(w1);
-    if (c + 1 < nch) {
-      if (c + 2 < nch) {
-        load_x(0, c + 2);
-        load_w(w0, c + 2);
+    if (c + G < nch) {
+      if (c + 2 * G < nch) {
+        load_x(0, c + 2 * G);
+        load_w(w0, c + 2 * G);
       }
       compute(w1, 1);
       arrived(w0);
@@ -487,11 +500,15 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
   }
 }
 
+// Workgroups per CU (three for the 4-bit format, which needs fewer registers, measured no faster).
+template <int WF> struct SkinnyLdsOcc { static constexpr int value = 2; };
+
 // A workgroup takes groups of four neighbouring items (tiles 4q .. 4q+3 of one expert), strided by the grid size.
 template <typename T, int WF, int MODE>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(256, SkinnyLdsOcc<WF>::value)
 grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
-  __shared__ __align__(16) uint16_t xs[2 * 32 * 256];  // two stages of up to 32 token rows x 256 reduction elements
+  constexpr int G = 1;                                     // chunks per pipeline step (the host checks K % (256 G) == 0)
+  __shared__ __align__(16) uint16_t xs[2 * G * 32 * 256];  // two stages of up to 32 token rows x 256 G reduction elements
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n_in = lane & 15;
   const int64_t nch = p.kred >> 8;
@@ -527,9 +544,9 @@ grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
       wrow[1] = wrow[0] + 16;
     }
     if (re - rb <= 16) {
-      skinny_lds_pass<T, WF, MODE, 1>(p, wrow, tile, rb, re, nch, lane, wave, xs, xs_addr);
+      skinny_lds_pass<T, WF, MODE, 1, G>(p, wrow, tile, rb, re, nch, lane, wave, xs, xs_addr);
     } else {
-      for (int r0 = rb; r0 < re; r0 += 32) skinny_lds_pass<T, WF, MODE, 2>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
+      for (int r0 = rb; r0 < re; r0 += 32) skinny_lds_pass<T, WF, MODE, 2, G>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
     }
   }
 }
@@ -561,9 +578,9 @@ static int launch_skinny_t(int mode, const GemmParams& p, int64_t max_rows, hipS
     // has four times fewer groups than the gate/up projection; with few rows per expert (one token tile, few loads to
     // share) it is better off with independent wavefronts.
     const int64_t src_rows = p.perm ? (max_rows + p.k_top - 1) / p.k_top : max_rows;
-    const bool worth = mode == MODE_GATEUP || max_rows > 12 * (int64_t)p.E;
+    const bool worth = (mode == MODE_GATEUP || max_rows > 12 * (int64_t)p.E) ;
     if constexpr (SkinnyUsesLds<WF>::value) if (worth && tiles % 4 == 0 && src_rows * p.lda * 2 < ((int64_t)1 << 32)) {
-      const int64_t groups = (int64_t)(tiles / 4) * p.E, capacity = 256 * 2;
+      const int64_t groups = (int64_t)(tiles / 4) * p.E, capacity = 256 * SkinnyLdsOcc<WF>::value;
       const int64_t per_wg = (groups + capacity - 1) / capacity;
       dim3 grid((unsigned)((groups + per_wg - 1) / per_wg));
       if (mode == MODE_GATEUP) grouped_skinny_lds_kernel<T, WF, MODE_GATEUP><<<grid, 256, 0, st>>>(p, tiles);
