@@ -1,0 +1,128 @@
+"""Edge cases of the grouped FFN path through the C ABI: empty inputs, experts without rows, one expert, k = E, rows per
+expert that need several passes or several token tiles, shapes that fall off the fast kernels, strided inputs."""
+
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+import moe_cases as MC
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(device, case, idx, *, prepack=True, variant=0):
+    """grouped_ffn + combine with the given routing; returns (got, want)."""
+    from sharktank_amd import _hip as hip
+    from sharktank_amd.ops import device_weight
+
+    x = case.planes["h"]
+    T, k = idx.shape
+    g = torch.Generator().manual_seed(case.seed + 7)
+    gate = torch.rand(T, k, generator=g)
+    gate = (gate / gate.sum(-1, keepdim=True)).to(case.dtype)
+    wg, wu, wd = MC.dense_weights(case)
+    want = O.grouped_ffn_moe(x, idx, gate, wg, wu, wd, case.activation)
+    E, N, K = case.E, case.N, case.K
+    dws = [device_weight(MC.to_inference_tensor(case.fmt, case.planes[n], shp, n, device), stacked=True, prepack=prepack)
+           for n, shp in (("gate", [E, N, K]), ("up", [E, N, K]), ("down", [E, K, N]))]
+    _, offsets, perm, inv = hip.dispatch_build(idx.to(torch.int32).to(device), E)
+    act = hip.ACT_SILU if case.act == "silu" else hip.ACT_GELU_ERF
+    y = hip.grouped_ffn(x.to(device), dws[0], dws[1], dws[2], act, offsets, perm, k, variant=variant)
+    got = hip.combine(y, gate.to(device), inv, T, k).cpu()
+    return got, want
+
+
+def test_empty_batch(device):
+    from sharktank_amd.layers import MoeBlock
+
+    case = MC.build(MC.Case(T=4, K=256, N=512, fmt="q8_0", dtype=torch.float16, seed=70))
+    block = MoeBlock(MC.make_theta(case, device), case.E, case.k, case.eps)
+    y = block(torch.empty(1, 0, case.K, dtype=torch.float16, device=device))
+    assert tuple(y.shape) == (1, 0, case.K)
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8"])
+def test_prefill_with_experts_that_get_no_rows(device, fmt):
+    """600 tokens all routed to experts 2 and 5 of 8: two experts with 600 rows (three token tiles, the last one
+    partial), six without rows; the launch is small enough that units are split along the reduction."""
+    case = MC.build(MC.Case(T=600, K=512, N=768, E=8, k=2, fmt=fmt, dtype=torch.float16, seed=71))
+    idx = torch.tensor([[2, 5]]).repeat(600, 1)
+    idx[::2] = torch.tensor([5, 2])
+    got, want = _run(device, case, idx)
+    assert O.rel_l2(got, want) < 1e-3
+
+
+def test_prefill_single_expert_top1(device):
+    case = MC.build(MC.Case(T=700, K=512, N=512, E=1, k=1, fmt="q8_0", dtype=torch.bfloat16, seed=72))
+    got, want = _run(device, case, torch.zeros(700, 1, dtype=torch.long))
+    assert O.rel_l2(got, want) < 8e-3
+
+
+def test_every_expert_selected(device):
+    """k = E: every token visits every expert (one full and one partial token tile per expert)."""
+    case = MC.build(MC.Case(T=300, K=256, N=512, E=4, k=4, fmt="q4_1", dtype=torch.float16, seed=73))
+    idx = torch.stack([torch.randperm(4, generator=torch.Generator().manual_seed(t)) for t in range(300)])
+    got, want = _run(device, case, idx)
+    assert O.rel_l2(got, want) < 1e-3
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_streaming_kernel_packed_rows_per_expert(device, fmt, dtype):
+    """The packed streaming kernels (token rows shared through LDS) with 3, 16, 17, 40 and 70 rows on the experts: one
+    token tile, two tiles, and several passes over an expert's weights."""
+    E, T, k = 8, 73, 2
+    case = MC.build(MC.Case(T=T, K=512, N=1024, E=E, k=k, fmt=fmt, dtype=dtype, seed=74))
+    rows = {0: 3, 1: 16, 2: 17, 3: 40, 4: 70}
+    pairs = [e for e, n in rows.items() for _ in range(n)]  # 146 = T * k pairs
+    assert len(pairs) == T * k
+    # deal the pairs so that a token never gets the same expert twice
+    idx = torch.empty(T, k, dtype=torch.long)
+    order = sorted(range(len(pairs)), key=lambda i: (i % T, i // T))
+    by_token = [[] for _ in range(T)]
+    for i, e in enumerate(sorted(pairs, key=lambda e: -rows[e])):
+        by_token[i % T].append(e)
+    for t in range(T):
+        assert len(set(by_token[t])) == k
+        idx[t] = torch.tensor(by_token[t])
+    got, want = _run(device, case, idx, variant=3)
+    assert O.rel_l2(got, want) < (1e-3 if dtype == torch.float16 else 8e-3)
+
+
+@pytest.mark.parametrize("N,K", [(96, 512), (992, 256), (512, 528)])
+def test_shapes_off_the_fast_paths(device, N, K):
+    """Feature counts that are not whole tiles or groups of four tiles, and a reduction length that is not a multiple
+    of 256: the launchers fall back to kernels that take them (planar order when the packed one does not apply)."""
+    for T in (5, 300):
+        case = MC.build(MC.Case(T=T, K=K, N=N, E=4, k=2, fmt="q8_0" if K % 32 == 0 else "dense", dtype=torch.float16, seed=75))
+        g = torch.Generator().manual_seed(76)
+        idx = torch.stack([torch.randperm(4, generator=g)[:2] for _ in range(T)])
+        from sharktank_amd.ops import device_weight
+
+        can = N % 16 == 0 and K % 256 == 0
+        got, want = _run(device, case, idx, prepack=can)
+        assert O.rel_l2(got, want) < 1e-3, (N, K, T)
+
+
+def test_strided_input_view(device):
+    """h given as a non-contiguous view (every other row of a larger buffer)."""
+    from sharktank_amd.layers import MoeBlock
+
+    case = MC.build(MC.Case(T=40, K=256, N=512, fmt="q8_0", dtype=torch.float16, seed=77))
+    block = MoeBlock(MC.make_theta(case, device), case.E, case.k, case.eps)
+    big = torch.zeros(80, case.K, dtype=torch.float16, device=device)
+    big[::2] = case.planes["h"].to(device)
+    y = block(big[::2].reshape(1, 40, case.K))
+    want, _, _ = MC.oracle_block(case)
+    assert O.rel_l2(y.reshape(40, case.K).cpu(), want) < 1e-3
+
+
+def test_three_experts_top3_router(device):
+    from sharktank_amd.layers import MoeBlock
+
+    case = MC.build(MC.Case(T=33, K=256, N=256, E=3, k=3, fmt="q8_0", dtype=torch.float16, seed=78))
+    block = MoeBlock(MC.make_theta(case, device), case.E, case.k, case.eps)
+    y, idx, gate = block(case.planes["h"].reshape(1, 33, case.K).to(device), return_routing=True)
+    want, want_idx, want_gate = MC.oracle_block(case)
+    assert torch.equal(idx.cpu().long(), want_idx)
+    assert O.rel_l2(y.reshape(33, case.K).cpu(), want) < 1e-3
