@@ -164,9 +164,9 @@ size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int64_t K, int
  * per-tensor e4m3fn quantizers (StaticScaledQuantizer, quantizers.py:153-183) applied to x before the gate/up
  * projections and to the intermediate before the down projection.  The reference semantics is quantise then
  * dequantise (`quantize(x).unpack().dequant()`, sharktank/sharktank/layers/linear.py:72-78) followed by the
- * floating-point path.  With FP8 weights and more than 32 tokens both operands are fed to the fp8 matrix cores as
- * bytes and the fp32 dot product is scaled once by scale_x * d_w; otherwise the re-dequantised values go through the
- * 16-bit kernels.  x itself is always given unquantised in `dtype`.
+ * floating-point path, and that is what variant 0 computes (quantise, dequantise, 16-bit kernels).  Variant 5 with FP8
+ * weights feeds both operands to the fp8 matrix cores as bytes and scales the fp32 dot product once by scale_x * d_w.
+ * x itself is always given unquantised in `dtype`.
  * `variant` 0 picks the kernel by shape; other values force one (see the kernel list in ffn.hip). */
 int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                       const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,

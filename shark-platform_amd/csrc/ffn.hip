@@ -143,16 +143,17 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   void* xa = base + ws.xa;
   void* zq = base + ws.zq;
 
-  // Quantised activations (fp8 e4m3fn, static per-tensor scale).  With few rows per expert the projections are bound
-  // by the weight stream, so the samples are re-dequantised (the reference's own formulation) and the streaming kernel
-  // runs unchanged; otherwise both operands go to the fp8 matrix cores as bytes (variant 5).
+  // Quantised activations (fp8 e4m3fn, static per-tensor scale).  By default the samples are re-dequantised (the
+  // reference's own formulation: quantize, dequantize, multiply in the activation dtype) and the 16-bit kernels run
+  // unchanged: the streaming kernel is bound by the weight stream anyway, and the 16-bit prefill kernel with its
+  // producer/consumer pipeline is currently faster than the fp8 matrix-core kernel.  Variant 5 sends both operands to
+  // the fp8 matrix cores as bytes and scales the fp32 dot product once.
   const bool fp8_w_in = w_gate->format == STMOE_W_FP8 || w_gate->format == STMOE_W_FP8_PACKED;
   const bool fp8_w_out = w_down->format == STMOE_W_FP8 || w_down->format == STMOE_W_FP8_PACKED;
-  const bool few_rows = T <= kSkinnyMaxRowsPerExpert || T * k <= kSkinnyMaxAvgRows * E;
   STMOE_REQUIRE(variant != 5 || (x_scale && z_scale), STMOE_ERR_UNSUPPORTED, "grouped_ffn: variant 5 (fp8 matrix cores) needs x_scale and z_scale");
   const bool t16 = dtype == STMOE_F16 || dtype == STMOE_BF16;
-  const bool mfma8_in = t16 && x_scale && fp8_w_in && w_gate->dtype == STMOE_F32 && K % 16 == 0 && (variant == 5 || (variant == 0 && !few_rows));
-  const bool mfma8_out = t16 && z_scale && fp8_w_out && w_down->dtype == STMOE_F32 && N % 16 == 0 && (variant == 5 || (variant == 0 && !few_rows));
+  const bool mfma8_in = t16 && x_scale && fp8_w_in && w_gate->dtype == STMOE_F32 && K % 16 == 0 && variant == 5;
+  const bool mfma8_out = t16 && z_scale && fp8_w_out && w_down->dtype == STMOE_F32 && N % 16 == 0 && variant == 5;
   const int v16 = variant == 5 ? 0 : variant;
 
   GemmParams p{};

@@ -208,9 +208,9 @@ def test_config5_mixtral_fp8_weights(device):
 
 
 def test_config5_mixtral_fp8_weights_and_activations(device):
-    """Config 5 with static e4m3fn quantizers on the FFN input and on the gated intermediate: the 4096-token prefill
-    runs both operands on the fp8 matrix cores, the 1-token decode re-dequantises and streams the weights.  Both are
-    held to the fp8 tolerance against the reference's quantise-dequantise-then-multiply arithmetic."""
+    """Config 5 with static e4m3fn quantizers on the FFN input and on the gated intermediate.  By default prefill and
+    decode quantise, dequantise and multiply in the activation dtype (the reference's arithmetic); with kernel
+    variant 5 the prefill runs both operands on the fp8 matrix cores.  All are held to the fp8 tolerance."""
     theta, pc = build_device_case(device, 4096, 4096, 14336, "fp8", torch.float16, seed=5, act_quant=True)
     y, idx, gate, block = run_layer(theta, pc, device)
     check_against_oracle(y, idx, pc, [0, 2047, 4095], 2e-2)
@@ -218,6 +218,13 @@ def test_config5_mixtral_fp8_weights_and_activations(device):
     assert torch.equal(idx1.cpu(), idx.cpu()[:1])
     want1, _, _ = oracle_rows(pc, [0])
     assert O.rel_l2(y1.reshape(1, 4096).cpu(), want1) < 1e-3  # the decode path follows the reference's arithmetic
-    # run-to-run bit identity of the matrix-core path
+    # run-to-run bit identity
     y2, _, _, _ = run_layer(theta, pc, device)
     assert torch.equal(y2, y)
+    # fp8 matrix cores
+    from sharktank_amd import _hip
+
+    y8, idx8, _, _ = run_layer(theta, pc, device, variant=_hip.VARIANT_FP8_MFMA)
+    check_against_oracle(y8, idx8, pc, [0, 2047, 4095], 2e-2)
+    y8b, _, _, _ = run_layer(theta, pc, device, variant=_hip.VARIANT_FP8_MFMA)
+    assert torch.equal(y8b, y8)
