@@ -128,6 +128,18 @@ int stmoe_fake_quant_fp8(const void* x, int dtype, const float* rscale, int64_t 
 int stmoe_prepack(const stmoe_weight* planar, const stmoe_weight* packed_out, stmoe_stream_t stream);
 int stmoe_unpack(const stmoe_weight* packed, const stmoe_weight* planar_out, stmoe_stream_t stream);
 
+typedef enum {
+  STMOE_GGUF_Q8_0 = 0, /* ggml block_q8_0 {f16 d; i8 qs[32]}, 34 bytes */
+  STMOE_GGUF_Q4_1 = 1  /* ggml block_q4_1 {f16 d; f16 m; u8 qs[16]}, 20 bytes; byte i = element i (low nibble), i + 16 (high) */
+} stmoe_gguf_type;
+
+/* Raw GGUF blocks -> weight planes in one pass: Q8_0.unpack (sharktank/sharktank/types/gguf_interop/layouts.py:51-60)
+ * and Q4_1.unpack (:285-300) with linearize_interleaved_i4_block (sharktank/sharktank/types/layout_utils.py:20-44).
+ * `raw_blocks` holds experts*rows*cols/32 blocks, row-major, 2-byte aligned.  `out` describes caller-owned planes of
+ * format STMOE_W_Q8_0 / STMOE_W_Q4_1 (the reference's planar planes, bit for bit) or of the matching _PACKED format
+ * (the streaming order of stmoe_prepack, written directly: rows % 16 == 0 and cols % 256 == 0). */
+int stmoe_gguf_ingest(const void* raw_blocks, int gguf_type, const stmoe_weight* out, stmoe_stream_t stream);
+
 /* ---- layer pieces ----------------------------------------------------------------------------- */
 
 /* RMSNormLayer.forward (sharktank/sharktank/layers/norm.py:34-41) with rms_norm_default
@@ -165,7 +177,8 @@ size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int64_t K, int
  * projections and to the intermediate before the down projection.  The reference semantics is quantise then
  * dequantise (`quantize(x).unpack().dequant()`, sharktank/sharktank/layers/linear.py:72-78) followed by the
  * floating-point path, and that is what variant 0 computes (quantise, dequantise, 16-bit kernels).  Variant 5 with FP8
- * weights feeds both operands to the fp8 matrix cores as bytes and scales the fp32 dot product once by scale_x * d_w.
+ * weights feeds both operands to the fp8 matrix cores as bytes and scales the fp32 dot product once by scale_x * d_w
+ * (variant 7: the same arithmetic on the general 128x128 tile kernel only).
  * x itself is always given unquantised in `dtype`.
  * `variant` 0 picks the kernel by shape; other values force one (see the kernel list in ffn.hip). */
 int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,

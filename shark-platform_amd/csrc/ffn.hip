@@ -44,11 +44,22 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 
 // variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile, 3 skinny streaming kernel (decode),
 //          4 MFMA 256x256 tile (prefill; packed Q8_0), 5 fp8 matrix cores (fp8 weights and quantised activations),
-//          6 MFMA 256x256 tile with specialised producer/consumer wavefronts (prefill; packed Q8_0)
+//          6 MFMA 256x256 tile with specialised producer/consumer wavefronts (prefill; packed formats),
+//          7 fp8 matrix cores, 128x128 tile kernel only (5 uses the 256x256 LDS-direct kernel where it applies)
 // The streaming kernel is chosen when no expert can get more than 32 rows, or when experts get 40 rows or fewer on
 // average (it then walks an expert's rows in passes of 32, re-reading the expert's weights for every pass).
 static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
 static constexpr int64_t kSkinnyMaxAvgRows = 40;
+// fp8 activations x fp8 weights on the fp8 matrix cores: the 256 x 256 kernel for packed weights and launches with
+// enough rows to fill its tiles (variant 5), the 128 x 128 kernel otherwise (and always with variant 7).
+static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
+  const bool ws_ok = variant == 5 && wtag == WF_FP8_F32D_P && max_rows >= 512 && p.kred % 256 == 0 && p.lda % 16 == 0 &&
+                     p.ldo % 4 == 0 && p.n_out % (mode == MODE_GATEUP ? 128 : 256) == 0 && (!p.offsets || p.E < 64) &&
+                     max_rows * p.lda < ((int64_t)1 << 32);
+  if (ws_ok) return launch_fp8_ws(dtype, wtag, mode, p, max_rows, st);
+  return launch_fp8_tile(dtype, wtag, mode, p, max_rows, st);
+}
+
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
@@ -150,11 +161,12 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   // the fp8 matrix cores as bytes and scales the fp32 dot product once.
   const bool fp8_w_in = w_gate->format == STMOE_W_FP8 || w_gate->format == STMOE_W_FP8_PACKED;
   const bool fp8_w_out = w_down->format == STMOE_W_FP8 || w_down->format == STMOE_W_FP8_PACKED;
-  STMOE_REQUIRE(variant != 5 || (x_scale && z_scale), STMOE_ERR_UNSUPPORTED, "grouped_ffn: variant 5 (fp8 matrix cores) needs x_scale and z_scale");
+  const bool want_mfma8 = variant == 5 || variant == 7;
+  STMOE_REQUIRE(!want_mfma8 || (x_scale && z_scale), STMOE_ERR_UNSUPPORTED, "grouped_ffn: variants 5 and 7 (fp8 matrix cores) need x_scale and z_scale");
   const bool t16 = dtype == STMOE_F16 || dtype == STMOE_BF16;
-  const bool mfma8_in = t16 && x_scale && fp8_w_in && w_gate->dtype == STMOE_F32 && K % 16 == 0 && variant == 5;
-  const bool mfma8_out = t16 && z_scale && fp8_w_out && w_down->dtype == STMOE_F32 && N % 16 == 0 && variant == 5;
-  const int v16 = variant == 5 ? 0 : variant;
+  const bool mfma8_in = t16 && x_scale && fp8_w_in && w_gate->dtype == STMOE_F32 && K % 16 == 0 && want_mfma8;
+  const bool mfma8_out = t16 && z_scale && fp8_w_out && w_down->dtype == STMOE_F32 && N % 16 == 0 && want_mfma8;
+  const int v16 = want_mfma8 ? 0 : variant;
 
   GemmParams p{};
   p.a = x; p.lda = K; p.perm = perm; p.k_top = k; p.offsets = offsets; p.E = E; p.fixed_rows = 0;
@@ -171,7 +183,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   if (mfma8_in) {
     p.x_scale = x_scale;
     if (mfma8_out) { p.out = zq; p.out_scale = z_scale; }
-    rc = launch_fp8_tile(dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
+    rc = run_fp8_projection(variant, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
   } else {
     rc = run_projection(v16, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
   }
@@ -193,7 +205,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   if (mfma8_out) {
     q.a = zq;
     q.x_scale = z_scale;
-    rc = launch_fp8_tile(dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
+    rc = run_fp8_projection(variant, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
   } else {
     rc = run_projection(v16, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
   }

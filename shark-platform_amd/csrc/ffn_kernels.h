@@ -114,4 +114,5 @@ int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64
 size_t mfma_ws_partial_bytes();
 int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_fp8_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
+int launch_fp8_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 }  // namespace stmoe

@@ -88,7 +88,107 @@ static int repack_weight(const stmoe_weight* src, const stmoe_weight* dst, int d
   return set_error(STMOE_ERR_UNSUPPORTED, "prepack: format pair %d -> %d has no packed order", src->format, dst->format);
 }
 
+// ---- raw ggml blocks -> planes (planar or streaming order) ---------------------------------------------
+// One thread per 32-element block.  Q8_0 block: {f16 d; i8 qs[32]} (34 bytes); Q4_1 block: {f16 d; f16 m; u8 qs[16]}
+// (20 bytes) with element i in the low nibble of byte i and element i + 16 in the high nibble.  The raw buffer is only
+// 2-byte aligned, so it is read as half-words.  PACKED writes the streaming order described at the top of this file.
+template <int Q4, int PACKED>
+__global__ void __launch_bounds__(256)
+gguf_ingest_kernel(const uint16_t* __restrict__ raw, uint8_t* __restrict__ qs, uint16_t* __restrict__ d, uint16_t* __restrict__ m,
+                   int64_t n_blocks, int64_t cols) {
+  const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;  // block index in row-major [rows_total][cols / 32]
+  if (b >= n_blocks) return;
+  constexpr int HW = Q4 ? 10 : 17;  // half-words per raw block
+  const uint16_t* src = raw + b * HW;
+  const int64_t bpr = cols >> 5, r = b / bpr, kb32 = b - r * bpr;  // global row, block inside the row
+  const int64_t rt = r >> 4;
+  const int n = (int)(r & 15);
+  // position of the block's scale: planar [r][kb32]; packed [rt][K/256][16 rows][8]
+  const int64_t dpos = PACKED ? ((rt * (cols >> 8) + (kb32 >> 3)) * 16 + n) * 8 + (kb32 & 7) : b;
+  d[dpos] = src[0];
+  if (Q4) {
+    m[dpos] = src[1];
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)src[2 + 2 * i] | ((uint32_t)src[3 + 2 * i] << 16);
+    // linear order: element e at nibble e; elements 0..15 are the low nibbles of the 16 raw bytes, 16..31 the high ones
+    uint32_t lin[4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      uint32_t lo = 0, hi = 0;  // 8 consecutive low (high) nibbles of raw bytes 8 i .. 8 i + 7
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t byte = (w[2 * i + (j >> 2)] >> (8 * (j & 3))) & 0xffu;
+        lo |= (byte & 0xfu) << (4 * j);
+        hi |= (byte >> 4) << (4 * j);
+      }
+      lin[i] = lo;
+      lin[2 + i] = hi;
+    }
+    uint4 v = make_uint4(lin[0], lin[1], lin[2], lin[3]);
+    int64_t piece = b;  // 16-byte piece index, planar [r][kb32]
+    if (PACKED) {
+      v = make_uint4(q4_dword_to_packed(v.x), q4_dword_to_packed(v.y), q4_dword_to_packed(v.z), q4_dword_to_packed(v.w));
+      piece = (rt * (cols >> 7) + (kb32 >> 2)) * 64 + 16 * (kb32 & 3) + n;
+    }
+    reinterpret_cast<uint4*>(qs)[piece] = v;
+  } else {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint32_t w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[i] = (uint32_t)src[1 + 8 * h + 2 * i] | ((uint32_t)src[2 + 8 * h + 2 * i] << 16);
+      int64_t piece = 2 * b + h;  // planar [r][cols / 16]
+      if (PACKED) {
+        const int64_t k16 = 2 * kb32 + h;  // 16-element group inside the row
+        piece = (rt * (cols >> 6) + (k16 >> 2)) * 64 + 16 * (k16 & 3) + n;
+      }
+      reinterpret_cast<uint4*>(qs)[piece] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+}
+
+static int gguf_ingest(const void* raw, int gguf_type, const stmoe_weight* out, stmoe_stream_t stream) {
+  STMOE_REQUIRE(raw && out, STMOE_ERR_NULL, "gguf_ingest: NULL argument");
+  STMOE_REQUIRE((reinterpret_cast<uintptr_t>(raw) & 1) == 0, STMOE_ERR_ALIGN, "gguf_ingest: raw blocks must be 2-byte aligned");
+  STMOE_REQUIRE(out->experts >= 0 && out->rows >= 0 && out->cols >= 0 && out->cols % 32 == 0, STMOE_ERR_SHAPE,
+                "gguf_ingest: cols must be a multiple of the block size 32 (got %lld)", (long long)out->cols);
+  const bool q4 = gguf_type == STMOE_GGUF_Q4_1;
+  STMOE_REQUIRE(q4 || gguf_type == STMOE_GGUF_Q8_0, STMOE_ERR_UNSUPPORTED, "gguf_ingest: unknown block type %d", gguf_type);
+  const int planar_fmt = q4 ? STMOE_W_Q4_1 : STMOE_W_Q8_0, packed_fmt = q4 ? STMOE_W_Q4_1_PACKED : STMOE_W_Q8_0_PACKED;
+  STMOE_REQUIRE(out->format == planar_fmt || out->format == packed_fmt, STMOE_ERR_UNSUPPORTED,
+                "gguf_ingest: block type %d cannot become weight format %d", gguf_type, out->format);
+  const bool packed = out->format == packed_fmt;
+  if (packed)
+    STMOE_REQUIRE(out->rows % 16 == 0 && out->cols % 256 == 0, STMOE_ERR_SHAPE,
+                  "gguf_ingest: the streaming order needs rows %% 16 == 0 and cols %% 256 == 0 (got %lld x %lld)",
+                  (long long)out->rows, (long long)out->cols);
+  const int64_t n_blocks = out->experts * out->rows * (out->cols / 32);
+  if (n_blocks == 0) return STMOE_OK;
+  STMOE_REQUIRE(out->qs && out->d && (!q4 || out->m), STMOE_ERR_NULL, "gguf_ingest: output plane is NULL");
+  STMOE_REQUIRE(aligned16(out->qs), STMOE_ERR_ALIGN, "gguf_ingest: qs plane must be 16-byte aligned");
+  STMOE_REQUIRE((n_blocks + 255) / 256 < ((int64_t)1 << 31), STMOE_ERR_SHAPE, "gguf_ingest: too many blocks");
+  hipStream_t st = as_stream(stream);
+  dim3 grid((unsigned)((n_blocks + 255) / 256));
+  auto* qs = static_cast<uint8_t*>(const_cast<void*>(out->qs));
+  auto* d = static_cast<uint16_t*>(const_cast<void*>(out->d));
+  auto* m = static_cast<uint16_t*>(const_cast<void*>(out->m));
+  const auto* r = static_cast<const uint16_t*>(raw);
+  if (q4) {
+    if (packed) gguf_ingest_kernel<1, 1><<<grid, 256, 0, st>>>(r, qs, d, m, n_blocks, out->cols);
+    else gguf_ingest_kernel<1, 0><<<grid, 256, 0, st>>>(r, qs, d, m, n_blocks, out->cols);
+  } else {
+    if (packed) gguf_ingest_kernel<0, 1><<<grid, 256, 0, st>>>(r, qs, d, nullptr, n_blocks, out->cols);
+    else gguf_ingest_kernel<0, 0><<<grid, 256, 0, st>>>(r, qs, d, nullptr, n_blocks, out->cols);
+  }
+  return check_launch("gguf_ingest");
+}
+
 }  // namespace stmoe
+
+extern "C" int stmoe_gguf_ingest(const void* raw_blocks, int gguf_type, const stmoe_weight* out, stmoe_stream_t stream) {
+  return stmoe::gguf_ingest(raw_blocks, gguf_type, out, stream);
+}
 
 extern "C" int stmoe_prepack(const stmoe_weight* planar, const stmoe_weight* packed_out, stmoe_stream_t stream) {
   return stmoe::repack_weight(planar, packed_out, 0, stream);

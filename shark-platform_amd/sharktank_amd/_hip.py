@@ -26,6 +26,7 @@ W_Q8_0_PACKED, W_Q4_1_PACKED, W_FP8_PACKED = 4, 5, 6
 _PACKED_OF = {W_Q8_0: W_Q8_0_PACKED, W_Q4_1: W_Q4_1_PACKED, W_FP8: W_FP8_PACKED}
 # grouped_ffn variants
 VARIANT_AUTO, VARIANT_GENERIC, VARIANT_MFMA_TILE, VARIANT_SKINNY, VARIANT_MFMA_BIG, VARIANT_FP8_MFMA, VARIANT_MFMA_WS = 0, 1, 2, 3, 4, 5, 6
+VARIANT_FP8_TILE = 7
 
 _DTYPE_ENUM = {
     torch.float32: F32,
@@ -72,6 +73,7 @@ SIGNATURES = {
     "stmoe_dequant_tensor_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p]),
     "stmoe_prepack": (c_int, [POINTER(StmoeWeight), POINTER(StmoeWeight), c_void_p]),
     "stmoe_unpack": (c_int, [POINTER(StmoeWeight), POINTER(StmoeWeight), c_void_p]),
+    "stmoe_gguf_ingest": (c_int, [c_void_p, c_int, POINTER(StmoeWeight), c_void_p]),
     "stmoe_quantize_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
     "stmoe_fake_quant_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
     "stmoe_rms_norm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_float, c_void_p, c_void_p]),
@@ -373,6 +375,32 @@ class DeviceWeight:
         with torch.cuda.device(self.device):
             _check(lib.stmoe_unpack(self.ref, out.ref, _stream(self.device)))
         return out
+
+
+GGUF_Q8_0, GGUF_Q4_1 = 0, 1
+
+
+def gguf_ingest(raw: torch.Tensor, gguf_type: int, experts: int, rows: int, cols: int, *, packed: bool) -> DeviceWeight:
+    """Raw ggml blocks (uint8, on the device) -> a DeviceWeight with freshly allocated planes, planar (the reference's
+    planes bit for bit) or in the streaming order of stmoe_prepack."""
+    dev = _dev(raw)
+    lib = load_library()
+    raw_c = _contig(raw)
+    if raw_c.dtype != torch.uint8:
+        raise TypeError(f"raw blocks must be uint8, got {raw_c.dtype}")
+    nb = experts * rows * (cols // 32)
+    block_bytes = {GGUF_Q8_0: 34, GGUF_Q4_1: 20}[gguf_type]
+    if cols % 32 != 0 or raw_c.numel() != nb * block_bytes:
+        raise ValueError(f"raw buffer of {raw_c.numel()} bytes does not hold [{experts},{rows},{cols}] in {block_bytes}-byte blocks")
+    q4 = gguf_type == GGUF_Q4_1
+    qs = torch.empty((experts, rows, cols // 32, 16 if q4 else 32), dtype=torch.uint8 if q4 else torch.int8, device=dev)
+    d = torch.empty((experts, rows, cols // 32, 1), dtype=torch.float16, device=dev)
+    m = torch.empty_like(d) if q4 else None
+    fmt = W_Q4_1 if q4 else W_Q8_0
+    out = DeviceWeight(_PACKED_OF[fmt] if packed else fmt, experts, rows, cols, qs, d, m)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_gguf_ingest(_ptr(raw_c), gguf_type, out.ref, _stream(dev)))
+    return out
 
 
 def grouped_ffn_workspace_bytes(T: int, k: int, K: int, N: int, dtype: torch.dtype) -> int:

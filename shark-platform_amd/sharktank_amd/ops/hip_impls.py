@@ -11,6 +11,7 @@ import torch
 from torch import Tensor
 
 from .. import _hip
+from ..types.gguf_interop import Q4_1, Q8_0
 from ..types.layouts import BlockScaledI4Layout, BlockScaledLayout, TensorScaledLayout
 from ..types.tensors import GatheredExpertsTensor, InferenceTensor, PrimitiveTensor, QuantizedTensor, unbox_tensor
 from ._registry import AllOfType
@@ -25,6 +26,12 @@ def device_weight(w, *, stacked: bool, prepack: bool = False) -> _hip.DeviceWeig
     """C-ABI descriptor of a weight tensor.  `stacked`: [E, rows, cols]; otherwise a single [rows, cols] matrix.
     Planes are made contiguous once here (GGUF-derived planes are strided views of the raw blocks).  With
     `prepack`, quantized planes whose shape allows it are re-ordered once into the kernels' streaming order."""
+    if isinstance(w, (Q8_0, Q4_1)) and w.raw.is_cuda:
+        # raw ggml blocks go to planes (planar or streaming order) in one kernel pass
+        shape = list(w.shape)
+        experts, rows, cols = shape if stacked else [1] + shape
+        packed = prepack and rows % 16 == 0 and cols % 256 == 0
+        return _hip.gguf_ingest(w.raw, _hip.GGUF_Q8_0 if isinstance(w, Q8_0) else _hip.GGUF_Q4_1, experts, rows, cols, packed=packed)
     dw = _device_weight_planar(w, stacked=stacked)
     if prepack and dw.can_prepack():
         dw = dw.prepack()

@@ -55,6 +55,17 @@ def test_argument_validation_without_a_gpu():
     rc = lib.stmoe_grouped_ffn(None, _hip.F16, 4, 48, 64, 8, 2, ctypes.byref(w), ctypes.byref(w), ctypes.byref(w), 0,
                                None, None, None, None, None, None, 0, 0, None)
     assert rc == 2 and b"32" in lib.stmoe_last_error()  # Q8_0 needs cols % 32 == 0
+    # raw GGUF blocks: shape, format pairing and streaming-order constraints are checked before any launch
+    assert lib.stmoe_gguf_ingest(16, _hip.GGUF_Q8_0, ctypes.byref(w), None) == 2
+    w2 = _hip.StmoeWeight(format=_hip.W_Q4_1, dtype=0, experts=1, rows=16, cols=64, qs=16, d=16, m=16, d_count=1)
+    assert lib.stmoe_gguf_ingest(16, _hip.GGUF_Q8_0, ctypes.byref(w2), None) == 5  # Q8_0 blocks cannot become Q4_1 planes
+    assert lib.stmoe_gguf_ingest(17, _hip.GGUF_Q4_1, ctypes.byref(w2), None) == 4  # odd address
+    w2.format = _hip.W_Q4_1_PACKED
+    assert lib.stmoe_gguf_ingest(16, _hip.GGUF_Q4_1, ctypes.byref(w2), None) == 2 and b"256" in lib.stmoe_last_error()
+    w2.rows = 0
+    assert lib.stmoe_gguf_ingest(16, _hip.GGUF_Q4_1, ctypes.byref(w2), None) == 2  # still not whole 256-column pieces
+    w2.format, w2.cols = _hip.W_Q4_1, 64
+    assert lib.stmoe_gguf_ingest(16, _hip.GGUF_Q4_1, ctypes.byref(w2), None) == 0  # nothing to do
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

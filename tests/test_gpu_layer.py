@@ -88,7 +88,8 @@ def test_fp8_matrix_core_layer(device, dtype, T):
     assert err < (2e-2 if dtype == torch.float16 else 6e-2), f"MoE contribution rel-L2 {err:.3e}"
 
 
-def test_fp8_matrix_core_path_is_exact_up_to_dequant_rounding(device):
+@pytest.mark.parametrize("variant_name,down_packed", [("VARIANT_FP8_MFMA", False), ("VARIANT_FP8_MFMA", True), ("VARIANT_FP8_TILE", True)])
+def test_fp8_matrix_core_path_is_exact_up_to_dequant_rounding(device, variant_name, down_packed):
     """With activations that are exactly representable after quantisation (integers times the scale) and power-of-two
     scales, scaling the fp32 dot product once equals dequantise-then-multiply: the fp8 path must then agree with the
     16-bit path to the rounding of the result only."""
@@ -108,11 +109,11 @@ def test_fp8_matrix_core_path_is_exact_up_to_dequant_rounding(device):
     dw = [device_weight(ST.PlanarQuantizedTensor(name=n, shape=list(q.shape),
                                                  layout=ST.TensorScaledLayout(shape=list(q.shape), d=d.to(device), qs=q.to(device))),
                         stacked=True, prepack=pp)
-          for (n, q), pp in zip(planes.items(), (True, True, False))]
+          for (n, q), pp in zip(planes.items(), (True, True, down_packed))]
     _, offsets, perm, inv = _hip.dispatch_build(experts.to(device), E)
     xs = torch.tensor(0.25)
     zs = torch.tensor(2.0 ** -4)
-    got = _hip.grouped_ffn(x.to(device), *dw, _hip.ACT_SILU, offsets, perm, k, variant=_hip.VARIANT_FP8_MFMA,
+    got = _hip.grouped_ffn(x.to(device), *dw, _hip.ACT_SILU, offsets, perm, k, variant=getattr(_hip, variant_name),
                            x_scale=xs.to(device), z_scale=zs.to(device)).cpu()
     dense = [O.dequant_tensor_scaled(d, q).to(torch.float16) for q in planes.values()]
     want_pairs = torch.zeros(T * k, K, dtype=torch.float16)

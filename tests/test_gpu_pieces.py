@@ -358,3 +358,83 @@ def test_ffn_mfma_ws_kernel_formats(device, dtype, fmt):
         outs[variant] = hip.combine(y, gate.to(device), inv, T, case.k).cpu()
         assert O.rel_l2(outs[variant], want) < tol
     assert O.rel_l2(outs[hip.VARIANT_MFMA_WS], outs[hip.VARIANT_MFMA_TILE]) < tol
+
+
+def _raw_blocks(fmt: str, shape, seed: int):
+    """Random bit patterns in ggml block structs: the scales are arbitrary fp16 bits (NaNs included), so a conversion
+    anywhere on the way would show."""
+    g = torch.Generator().manual_seed(seed)
+    nb = shape[0] * shape[1] * shape[2] // 32
+    return torch.randint(0, 256, (nb * (34 if fmt == "q8_0" else 20),), dtype=torch.uint8, generator=g)
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1"])
+@pytest.mark.parametrize("shape", [(3, 64, 512), (1, 16, 256), (2, 40, 96)])
+def test_gguf_raw_blocks_to_planes(device, fmt, shape):
+    """stmoe_gguf_ingest: raw ggml blocks -> the reference's planar planes, bit for bit, and -> the streaming order
+    directly, identical to stmoe_prepack of the planar planes."""
+    H = _hip()
+    raw = _raw_blocks(fmt, shape, 90 + shape[1])
+    E, rows, cols = shape
+    gt = H.GGUF_Q8_0 if fmt == "q8_0" else H.GGUF_Q4_1
+    planar = H.gguf_ingest(raw.to(device), gt, E, rows, cols, packed=False)
+    qs, d, m = planar.keep
+    if fmt == "q8_0":
+        want_d, want_qs = O.q8_0_unpack(raw, list(shape))
+        assert m is None
+    else:
+        want_d, want_m, want_qs = O.q4_1_unpack(raw, list(shape))
+        assert torch.equal(m.cpu().view(torch.int16), want_m.contiguous().view(torch.int16))
+    assert torch.equal(d.cpu().view(torch.int16), want_d.contiguous().view(torch.int16))
+    assert torch.equal(qs.cpu().view(torch.uint8), want_qs.contiguous().view(torch.uint8))
+    if rows % 16 == 0 and cols % 256 == 0:
+        direct = H.gguf_ingest(raw.to(device), gt, E, rows, cols, packed=True)
+        via = planar.prepack()
+        for a, b in zip(direct.keep, via.keep):
+            assert (a is None) == (b is None)
+            if a is not None:
+                assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+        back = direct.unpack()
+        for a, b in zip(back.keep, planar.keep):
+            if a is not None:
+                assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    else:
+        with pytest.raises(RuntimeError, match="rows % 16 == 0"):
+            H.gguf_ingest(raw.to(device), gt, E, rows, cols, packed=True)
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1"])
+def test_layer_from_gguf_raw_blocks(device, fmt):
+    """A MoeBlock whose expert weights are raw ggml blocks on the device gives the same output, bit for bit, as the
+    block built from the planar planes of the same blocks."""
+    import moe_cases as MC
+    from sharktank_amd import types as ST
+    from sharktank_amd.layers import MoeBlock
+
+    case = MC.build(MC.Case(T=24, K=256, N=512, fmt=fmt, dtype=torch.float16, seed=95))
+    theta = MC.make_theta(case, device)
+    ref_block = MoeBlock(theta, expert_count=case.E, expert_used_count=case.k, rms_epsilon=case.eps)
+    tree = dict(theta.flatten())
+    for name, key in (("ffn_gate_exps", "gate"), ("ffn_up_exps", "up"), ("ffn_down_exps", "down")):
+        p = case.planes[key]
+        shape = list(tree[f"{name}.weight"].shape)
+        if fmt == "q8_0":
+            raw = torch.cat([p["d"].view(torch.uint8).reshape(-1, 2), p["qs"].view(torch.uint8).reshape(-1, 32)], dim=1).reshape(-1)
+            tree[f"{name}.weight"] = ST.Q8_0(raw=raw.to(device), shape=shape, name=f"{name}.weight")
+        else:
+            ggml = O.interleave_linear_i4_block(p["qs"]).reshape(-1, 16)
+            raw = torch.cat([p["d"].view(torch.uint8).reshape(-1, 2), p["m"].view(torch.uint8).reshape(-1, 2), ggml], dim=1).reshape(-1)
+            tree[f"{name}.weight"] = ST.Q4_1(raw=raw.to(device), shape=shape, name=f"{name}.weight")
+    raw_block = MoeBlock(ST.Theta(tree), expert_count=case.E, expert_used_count=case.k, rms_epsilon=case.eps)
+    h = case.planes["h"].to(device).reshape(1, case.T, case.K)
+    assert torch.equal(raw_block(h), ref_block(h))
+    assert raw_block.experts.device_weights()[0].is_packed
+    # to_planar() of device-resident raw blocks equals the view-based unpack of the same blocks on the host
+    t = tree["ffn_gate_exps.weight"]
+    planar = t.to_planar().unpack()
+    host = type(t)(raw=t.raw.cpu(), shape=t.shape).unpack()
+    assert torch.equal(planar.d.cpu(), host.d)
+    if fmt == "q8_0":
+        assert torch.equal(planar.qs.cpu(), host.qs)
+    else:
+        assert torch.equal(planar.m.cpu(), host.m) and torch.equal(planar.qs_bit_packed.cpu(), host.qs_bit_packed)
