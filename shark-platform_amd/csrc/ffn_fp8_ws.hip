@@ -85,7 +85,7 @@ grouped_fp8_ws_kernel(GemmParams p, int n_tiles) {
   const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)lds8);
   const uint32_t w_lds = lds0 + 2 * wave * 1024, x_lds = lds0 + WSTAGE + 32 * wave * KS;
   const uint32_t lane16 = lane * 16;
-  auto issue = [&](int st) {  // stage st of the reduction into LDS slot st % D
+  auto issue = [&](int st) __attribute__((always_inline)) {  // stage st of the reduction into LDS slot st % D
     const uint32_t slot = (uint32_t)(st % D) * STAGE;
     vm_load16_to_lds(wq[0], lane16 + (uint32_t)st * 1024, w_lds + slot);
     vm_load16_to_lds(wq[1], lane16 + (uint32_t)st * 1024, w_lds + slot + 1024);
@@ -104,7 +104,7 @@ grouped_fp8_ws_kernel(GemmParams p, int n_tiles) {
   floatx16_t acc[4][2];
   const int my_rows = min(rpg, rows_here - wm * rpg);
 
-  auto compute = [&](auto both_tag, int slot) {
+  auto compute = [&](auto both_tag, int slot) __attribute__((always_inline)) {
     constexpr bool BOTH = decltype(both_tag)::value;  // rows in both 32-row token blocks
     const uint8_t* bp = b_rd + slot * STAGE;
     intx8_t bf[2];
@@ -122,7 +122,7 @@ grouped_fp8_ws_kernel(GemmParams p, int n_tiles) {
         acc[ti][q] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af, bf[q], acc[ti][q], 0, 0, 0, 127, 0, 127);
     }
   };
-  auto k_loop = [&](auto both_tag) {
+  auto k_loop = [&](auto both_tag) __attribute__((always_inline)) {
     constexpr bool BOTH = decltype(both_tag)::value;
 #pragma unroll
     for (int a = 0; a < 4; ++a)
@@ -153,8 +153,12 @@ grouped_fp8_ws_kernel(GemmParams p, int n_tiles) {
   const float s0 = xsc * reinterpret_cast<const float*>(p.w0.d)[p.w0.d_count > 1 ? e : 0];
   const float s1 = MODE == MODE_GATEUP ? xsc * reinterpret_cast<const float*>(p.w1.d)[p.w1.d_count > 1 ? e : 0] : 0.0f;
   const float out_rs = p.out_scale ? p.out_scale[0] : 0.0f;
-  auto epilogue = [&](auto tj_tag) {
+  // 1 / out_rs once; per element q = v * inv refined by one residual step (fma(-q, rs, v) * inv + q), which is the
+  // correctly rounded quotient except in rare last-bit cases that the following rounding to T absorbs
+  const float out_inv = p.out_scale ? __builtin_amdgcn_rcpf(out_rs) : 0.0f;
+  auto epilogue = [&](auto tj_tag, auto act_tag) __attribute__((always_inline)) {
     constexpr int tj = decltype(tj_tag)::value;
+    constexpr int ACT = decltype(act_tag)::value;
     if (tj * 32 + r32 < my_rows) {
       const int64_t orow = out_row(p, row_begin + wm * rpg + tj * 32 + r32) * p.ldo;
       if (MODE == MODE_GATEUP) {
@@ -163,25 +167,27 @@ grouped_fp8_ws_kernel(GemmParams p, int n_tiles) {
 #pragma unroll
           for (int b = 0; b < 4; ++b) {  // four consecutive features per 8-row band of the 32 x 32 result
             const int64_t col = (int64_t)ntile * (BN / 2) + wn * 64 + ti * 32 + 8 * b + 4 * h32;
-            float v[4];
+            float gq[4], uq[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-              const float gr = round_to<T>(acc[ti][tj][4 * b + q] * s0);
-              const float a = round_to<T>(act_rt(p.act, gr));
-              const float ur = round_to<T>(acc[ti + 2][tj][4 * b + q] * s1);
-              v[q] = round_to<T>(__fmul_rn(a, ur));
+              gq[q] = acc[ti][tj][4 * b + q] * s0;
+              uq[q] = acc[ti + 2][tj][4 * b + q] * s1;
             }
             if (p.out_scale) {  // e4m3fn(clamp(T(v / rscale))) for the next fp8 projection
-              uint32_t qv = 0;
+              float t[4];
 #pragma unroll
               for (int q = 0; q < 4; ++q) {
-                float t = round_to<T>(__fdiv_rn(v[q], out_rs));
-                t = fminf(fmaxf(t, -448.0f), 448.0f);
-                qv |= (uint32_t)f32_to_fp8_e4m3fn(t) << (8 * q);
+                const float a = round_to<T>(act_fast<ACT>(round_to<T>(gq[q])));
+                const float v = round_to<T>(__fmul_rn(a, round_to<T>(uq[q])));
+                const float q0 = v * out_inv;
+                const float q1 = __builtin_fmaf(__builtin_fmaf(-q0, out_rs, v), out_inv, q0);
+                t[q] = fminf(fmaxf(round_to<T>(q1), -448.0f), 448.0f);
               }
-              *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(p.out) + orow + col) = qv;
+              int qv = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);  // hardware OCP e4m3fn, round to nearest even
+              qv = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], qv, true);
+              *reinterpret_cast<int*>(reinterpret_cast<uint8_t*>(p.out) + orow + col) = qv;
             } else {
-              *reinterpret_cast<uint2*>(reinterpret_cast<T*>(p.out) + orow + col) = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
+              *reinterpret_cast<uint2*>(reinterpret_cast<T*>(p.out) + orow + col) = gateup_quad<T, ACT>(gq, uq);
             }
           }
       } else {
@@ -195,6 +201,16 @@ grouped_fp8_ws_kernel(GemmParams p, int n_tiles) {
                 make_uint2(pack2<T>(c[4 * b] * s0, c[4 * b + 1] * s0), pack2<T>(c[4 * b + 2] * s0, c[4 * b + 3] * s0));
           }
       }
+    }
+  };
+  auto epilogues = [&](auto both_tag) __attribute__((always_inline)) {
+    constexpr bool BOTH = decltype(both_tag)::value;
+    if (MODE == MODE_DOWN || p.act == STMOE_ACT_SILU) {
+      epilogue(F8Int<0>{}, EpiAct<STMOE_ACT_SILU>{});
+      if constexpr (BOTH) epilogue(F8Int<1>{}, EpiAct<STMOE_ACT_SILU>{});
+    } else {
+      epilogue(F8Int<0>{}, EpiAct<STMOE_ACT_GELU_ERF>{});
+      if constexpr (BOTH) epilogue(F8Int<1>{}, EpiAct<STMOE_ACT_GELU_ERF>{});
     }
   };
 
@@ -214,11 +230,10 @@ grouped_fp8_ws_kernel(GemmParams p, int n_tiles) {
     }
   } else if (my_rows <= 32) {
     k_loop(F8Int<0>{});
-    epilogue(F8Int<0>{});
+    epilogues(F8Int<0>{});
   } else {
     k_loop(F8Int<1>{});
-    epilogue(F8Int<0>{});
-    epilogue(F8Int<1>{});
+    epilogues(F8Int<1>{});
   }
 }
 

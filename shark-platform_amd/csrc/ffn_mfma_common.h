@@ -34,8 +34,7 @@ template <int A> struct EpiAct { static constexpr int value = A; };
 // tile times one feature tile.  Workgroup ids are dealt round-robin to the 8 XCDs; XCD i takes the i-th eighth of
 // the full units and then the i-th eighth of the partial units, so every XCD gets the same amount of work (within
 // one unit) and the short partial units run last, where they fill the end of the launch instead of delaying full
-// units.  Inside each class the token tile index runs fastest, so the token tiles of one expert work on the same
-// weight slab at the same time and share it in the XCD's L2.
+// units.  The order inside each class (big_unit) keeps workgroups that share operands together on an XCD.
 struct BigTile {
   int e, row_begin, row_end, ntile;
   int chunk, nchunks;  // this workgroup's part of the reduction (0 of 1 unless the unit is split)
@@ -91,41 +90,67 @@ __device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int lane_off, i
   }
   return pl;
 }
-// Unit number `unit` of the XCD's list (full units, then partial ones; token tile index fastest inside each class).
+// Unit number `unit` of the XCD's list: full units, then partial ones.
+// Full units are listed expert by expert, and inside an expert in blocks of about 32 units (one round over an XCD's
+// CUs) made of all of the expert's full token tiles x as many neighbouring feature tiles as fit: the workgroups that run
+// together on an XCD then share a few token tiles and a few weight tiles through its L2 instead of each fetching its own
+// (with 4 token tiles per expert: 4 + 8 operand streams for 32 workgroups).  Partial units: feature tile by feature
+// tile, one unit per expert that has a partial token tile.
+__device__ __forceinline__ void big_full_unit(int u, int c, int n_tiles, int& token_tile, int& ntile) {
+  const int bn0 = c >= kBigCusPerXcd ? 1 : kBigCusPerXcd / c;  // feature tiles per block
+  const int per = c * bn0;
+  const int b = u / per, v = u - b * per;
+  const int bn = min(bn0, n_tiles - b * bn0);
+  token_tile = v / bn;
+  ntile = b * bn0 + v - token_tile * bn;
+}
 __device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int BM, int n_tiles, const BigPlan& pl, int unit, BigTile& t) {
-  int u, cnt;
+  int u;
   bool partial;
   if (unit < pl.f1 - pl.f0) {
     u = pl.f0 + unit;
-    cnt = pl.F;
     partial = false;
   } else if (unit - (pl.f1 - pl.f0) < pl.r1 - pl.r0) {
     u = pl.r0 + unit - (pl.f1 - pl.f0);
-    cnt = pl.R;
     partial = true;
   } else {
     return false;
   }
-  t.ntile = u / cnt;
-  int s = u - t.ntile * cnt;
   if (!p.offsets) {
     t.e = 0;
-    t.row_begin = partial ? pl.F * BM : s * BM;
-    t.row_end = partial ? (int)p.fixed_rows : t.row_begin + BM;
+    if (partial) {
+      t.ntile = u;
+      t.row_begin = pl.F * BM;
+      t.row_end = (int)p.fixed_rows;
+    } else {
+      int s;
+      big_full_unit(u, pl.F, n_tiles, s, t.ntile);
+      t.row_begin = s * BM;
+      t.row_end = t.row_begin + BM;
+    }
     return true;
   }
-  for (int e = 0; e < p.E; ++e) {
-    const int b = __builtin_amdgcn_readlane(lane_off, e), rows = __builtin_amdgcn_readlane(lane_off, e + 1) - b;
-    if (!partial) {
-      const int c = rows / BM;
-      if (s < c) {
+  if (!partial) {
+    for (int e = 0; e < p.E; ++e) {
+      const int b = __builtin_amdgcn_readlane(lane_off, e), rows = __builtin_amdgcn_readlane(lane_off, e + 1) - b;
+      const int c = rows / BM, units = c * n_tiles;
+      if (u < units) {
+        int s;
+        big_full_unit(u, c, n_tiles, s, t.ntile);
         t.e = e;
         t.row_begin = b + s * BM;
         t.row_end = t.row_begin + BM;
         return true;
       }
-      s -= c;
-    } else if (rows % BM) {
+      u -= units;
+    }
+    return false;
+  }
+  t.ntile = u / pl.R;
+  int s = u - t.ntile * pl.R;
+  for (int e = 0; e < p.E; ++e) {
+    const int b = __builtin_amdgcn_readlane(lane_off, e), rows = __builtin_amdgcn_readlane(lane_off, e + 1) - b;
+    if (rows % BM) {
       if (s == 0) {
         t.e = e;
         t.row_begin = b + rows / BM * BM;
@@ -273,11 +298,9 @@ template <> struct BigPiece<WF_Q4_1_P> {
     m = a.m[s];
   }
   template <typename T> __device__ __forceinline__ void convert(const BigAddr<WF_Q4_1_P>&, uint32_t out[8]) const {
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      out[b] = q4_pair_dequant(q4_pair_packed(q.x, b), d, m);
-      out[4 + b] = q4_pair_dequant(q4_pair_packed(q.y, b), d, m);
-    }
+    const Q4Scale sc = q4_scale(d, m);
+    q4_dword_dequant_packed(q.x, sc, out);
+    q4_dword_dequant_packed(q.y, sc, out + 4);
     f16x16_to_T<T>(out);
   }
 };

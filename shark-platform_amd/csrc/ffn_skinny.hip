@@ -61,6 +61,7 @@ template <int WF> __device__ __forceinline__ int x_offset(int s, int g) {
 template <> struct SkinnyW<WF_Q8_0> {
   u32x4_t q[4];
   u32x4_t d;  // the chunk's 8 block scales
+  __device__ __forceinline__ void init(const WeightView&, int64_t) {}
   __device__ __forceinline__ void touch() { asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]), "+v"(d)); }
   __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
     const uint8_t* base = w.qs + row * w.cols + c * 256 + 16 * g;
@@ -90,6 +91,7 @@ template <> struct SkinnyW<WF_Q8_0> {
 template <> struct SkinnyW<WF_Q4_1> {
   u32x4_t q[2];
   uint16_t d[2], m[2];  // scale / offset of the lane's own two blocks (4*i + g, i = 0, 1)
+  __device__ __forceinline__ void init(const WeightView&, int64_t) {}
   __device__ __forceinline__ void touch() { asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(d[0]), "+v"(d[1]), "+v"(m[0]), "+v"(m[1])); }
   __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
     const uint8_t* base = w.qs + ((row * w.cols + c * 256) >> 1) + 16 * g;
@@ -109,9 +111,15 @@ template <> struct SkinnyW<WF_Q4_1> {
     const int i = s >> 2, j = s & 3;
     const uint32_t w4 = q[i][j];  // 8 nibbles of block 4*i + g
     u32x4_t out;
+    if constexpr (PACKED) {
+      uint32_t h[4];
+      q4_dword_dequant_packed(w4, q4_scale(d[i], m[i]), h);
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
-      out[b] = h2_to_T<T>(q4_pair_dequant(PACKED ? q4_pair_packed(w4, b) : q4_pair_linear(w4, b), d[i], m[i]));
+      for (int b = 0; b < 4; ++b) out[b] = h2_to_T<T>(h[b]);
+    } else {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) out[b] = h2_to_T<T>(q4_pair_dequant(q4_pair_linear(w4, b), d[i], m[i]));
+    }
     return out;
   }
 };
@@ -124,6 +132,9 @@ template <> struct SkinnyW<WF_FP8_F32D> {
     const uint8_t* base = w.qs + row * w.cols + c * 256 + 16 * g;
 #pragma unroll
     for (int i = 0; i < 4; ++i) q[i] = ld_stream16(base + 64 * i);
+  }
+  // the scale depends on the item only (one per tensor or per expert): fetched once, not with every chunk
+  __device__ __forceinline__ void init(const WeightView& w, int64_t row) {
     dv = reinterpret_cast<const float*>(w.d)[w.d_count > 1 ? row / w.rows : 0];
   }
   template <typename T> __device__ __forceinline__ u32x4_t frag(int s, int g) const {
@@ -134,10 +145,8 @@ template <> struct SkinnyW<WF_FP8_F32D> {
       const uint32_t u = q[i][2 * h + j];
       float f[4];
       fp8x4_to_f32(u, f);
-#pragma unroll
-      for (int b = 0; b < 4; ++b) f[b] = __fmul_rn(f[b], dv);
-      out[2 * j] = pack2<T>(f[0], f[1]);
-      out[2 * j + 1] = pack2<T>(f[2], f[3]);
+      out[2 * j] = scale2_pack<T>(f[0], f[1], dv);
+      out[2 * j + 1] = scale2_pack<T>(f[2], f[3], dv);
     }
     return out;
   }
@@ -174,13 +183,13 @@ template <> struct SkinnyW<WF_FP8_F32D_P> : SkinnyW<WF_FP8_F32D> {
     const uint8_t* base = w.qs + (rt * (w.cols >> 6) + c * 4) * 1024 + (g * 16 + (int)(row & 15)) * 16;
 #pragma unroll
     for (int i = 0; i < 4; ++i) q[i] = ld_stream16(base + 1024 * i);
-    dv = reinterpret_cast<const float*>(w.d)[w.d_count > 1 ? row / w.rows : 0];
   }
 };
 
 template <bool BF> struct SkinnyWDense16 {
   u32x4_t q[8];
   __device__ __forceinline__ void touch() {}
+  __device__ __forceinline__ void init(const WeightView&, int64_t) {}
   __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
     const uint8_t* base = w.qs + (row * w.cols + c * 256 + 16 * g) * 2;
 #pragma unroll
@@ -240,6 +249,10 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
   // before the next weight chunk so that weight requests stay in flight while they arrive.
   constexpr bool XDB = MT == 1;
   SkinnyW<WF> w0[NT], w1[NT];
+  w0[0].init(p.w0, wrow[0]);
+  w1[0].init(p.w0, wrow[0]);
+  w0[1].init(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1]);
+  w1[1].init(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1]);
   SkinnyX<WF> x0[MT], x1[XDB ? MT : 1];
   auto load_w = [&](SkinnyW<WF>* w, int64_t c) {
     w[0].load(p.w0, wrow[0], c, g);
@@ -424,6 +437,13 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[mt][t] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
   SkinnyW<WF> w0[G][NT], w1[G][NT];
+#pragma unroll
+  for (int q = 0; q < G; ++q) {
+    w0[q][0].init(p.w0, wrow[0]);
+    w1[q][0].init(p.w0, wrow[0]);
+    w0[q][1].init(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1]);
+    w1[q][1].init(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1]);
+  }
   auto load_w = [&](SkinnyW<WF> (*w)[NT], int64_t c) {
 #pragma unroll
     for (int q = 0; q < G; ++q) {
@@ -567,7 +587,7 @@ static int launch_skinny_t(int mode, const GemmParams& p, int64_t max_rows, hipS
   // a workgroup shares each item and splits its reduction
   const int64_t active_bound = max_rows < p.E ? max_rows : p.E;
   const int64_t items_bound = active_bound * tiles;
-  if (items_bound * 4 <= 1024 * SkinnyOcc<WF>::value && (p.kred >> 8) >= 4) {
+  if (items_bound * 4 <= 2 * 1024 * SkinnyOcc<WF>::value && (p.kred >> 8) >= 4) {
     dim3 grid((unsigned)items_bound);
     if (mode == MODE_GATEUP) grouped_skinny_kernel<T, WF, MODE_GATEUP, 4><<<grid, 256, 0, st>>>(p, tiles, (int)items_bound);
     else grouped_skinny_kernel<T, WF, MODE_DOWN, 4><<<grid, 256, 0, st>>>(p, tiles, (int)items_bound);

@@ -45,10 +45,9 @@ template <int WF> struct IsQ4 { static constexpr bool value = WF == WF_Q4_1 || W
 // pack two fp32 values, already rounded to T, into one dword of T bits
 template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
 template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi) {
-  union { f16_t h[2]; uint32_t u; } c;
-  c.h[0] = (f16_t)lo;
-  c.h[1] = (f16_t)hi;
-  return c.u;
+  typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+  const f16x2_t v = {(f16_t)lo, (f16_t)hi};  // a vector, so that both halves are written in place (no shift-and-or packing)
+  return __builtin_bit_cast(uint32_t, v);
 }
 template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) {
   typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -57,6 +56,20 @@ template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi
 }
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+// pack2<T>(a0 * d, a1 * d) with each product rounded to fp32 and then to T.  For fp16 the mixed-precision fused
+// multiply-add writes each half of the result in place (fp32 arithmetic, then the conversion): two instructions
+// instead of two multiplies and a packed conversion.
+template <typename T> __device__ __forceinline__ uint32_t scale2_pack(float a0, float a1, float d) {
+  if constexpr (__is_same(T, f16_t)) {
+    uint32_t r;
+    asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(r) : "v"(a0), "v"(d));
+    asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(r) : "v"(a1), "v"(d));
+    return r;
+  } else {
+    return pack2<T>(__fmul_rn(a0, d), __fmul_rn(a1, d));
+  }
+}
 
 __device__ __forceinline__ half2_t as_half2(uint32_t u) {
   union { uint32_t u; half2_t h; } c;
@@ -91,6 +104,40 @@ __device__ __forceinline__ uint32_t q4_pair_linear(uint32_t w, int p) {
   return 0x64006400u | (byte & 0xfu) | ((byte & 0xf0u) << 12);
 }
 __device__ __forceinline__ uint32_t q4_pair_packed(uint32_t w, int p) { return ((w >> (4 * p)) & 0x000f000fu) | 0x64006400u; }
+// The four pairs of a packed dword, dequantised, with fewer operations than four q4_pair_dequant calls.  The nibbles at
+// bits 0-3 and 4-7 of each half-word become the fp16 numbers 1024 + q and 64 + q by one and-or each (the nibble lands
+// in the mantissa of 0x6400 / 0x5400); the other two pairs come the same way from the dword shifted right by 8.  One
+// fused multiply-add per pair removes the bias and applies the scale: (bias + q) * d - bias * d is the exact product
+// q * d rounded once, like the reference's multiply (bias * d is exact; it stays finite for |d| < 64, far beyond any
+// block scale of fp16-range weights), and one add applies m: the reference's two roundings.
+struct Q4Scale {
+  half2_t dd, mm, c1024, c64;
+};
+__device__ __forceinline__ Q4Scale q4_scale(uint32_t dbits, uint32_t mbits) {
+  Q4Scale s;
+  s.dd = as_half2(dbits | (dbits << 16));
+  s.mm = as_half2(mbits | (mbits << 16));
+  const half2_t n1024 = {(f16_t)-1024.0f, (f16_t)-1024.0f}, n64 = {(f16_t)-64.0f, (f16_t)-64.0f};
+  s.c1024 = s.dd * n1024;
+  s.c64 = s.dd * n64;
+  return s;
+}
+// (a & mask) | magic in one instruction; written out because the compiler splits it into an and and an or when both
+// constants are literals (a VOP3 instruction of this ISA cannot take two of them; here they sit in registers)
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(mask), "v"(magic));
+  return r;
+}
+__device__ __forceinline__ void q4_dword_dequant_packed(uint32_t w, const Q4Scale& s, uint32_t out[4]) {
+  const uint32_t w8 = w >> 8;
+  const uint32_t p0 = and_or(w, 0x000f000fu, 0x64006400u), p1 = and_or(w, 0x00f000f0u, 0x54005400u);
+  const uint32_t p2 = and_or(w8, 0x000f000fu, 0x64006400u), p3 = and_or(w8, 0x00f000f0u, 0x54005400u);
+  out[0] = as_u32(__builtin_elementwise_fma(as_half2(p0), s.dd, s.c1024) + s.mm);
+  out[1] = as_u32(__builtin_elementwise_fma(as_half2(p1), s.dd, s.c64) + s.mm);
+  out[2] = as_u32(__builtin_elementwise_fma(as_half2(p2), s.dd, s.c1024) + s.mm);
+  out[3] = as_u32(__builtin_elementwise_fma(as_half2(p3), s.dd, s.c64) + s.mm);
+}
 __device__ __forceinline__ uint32_t q4_dword_to_packed(uint32_t w) {
   uint32_t out = 0;
 #pragma unroll
