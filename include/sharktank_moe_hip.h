@@ -59,6 +59,7 @@ typedef enum {
   STMOE_W_DENSE = 0, /* DefaultPrimitiveTensor: qs = elements of `dtype` */
   STMOE_W_Q8_0 = 1,  /* BlockScaledLayout, block 32: d fp16 [.,K/32], qs int8 [.,K/32,32] */
   STMOE_W_Q4_1 = 2,  /* BlockScaledI4Layout, block 32, unsigned: d,m fp16 [.,K/32], qs u8 [.,K/32,16] */
+                     /* (the matrix-multiply kernels on the packed form assume block scales |d| < 64) */
   STMOE_W_FP8 = 3,   /* TensorScaledLayout: qs e4m3fn [.,K], d = d_count scales of `dtype` (f32 or f16) */
   /* The same bytes re-ordered by stmoe_prepack() into the order the matrix-core kernels stream (every wavefront
    * load is one contiguous kilobyte; see stmoe_prepack).  Plane sizes are unchanged. */

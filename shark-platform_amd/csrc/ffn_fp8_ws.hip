@@ -18,6 +18,10 @@
 //            registers, so every operand byte is read from LDS once per wavefront.
 //   epilogue: the fp32 dot products of the quantised samples are scaled once by scale_x * d_w; the gate/up epilogue can
 //            quantise the gated intermediate to e4m3fn for the down projection.
+//   What bounds it: at 256 flop per operand byte the tile needs 32 KB per stage from L2 / HBM; with the operand loads
+//   alone (no MFMA) the launch takes two thirds of its full time and with the MFMAs alone 60 %, i.e. the two overlap only
+//   partly: the bytes in flight are capped by the LDS (4 stages of 32 KB), which covers the load latency under load only
+//   just.  Reading the next stage's operands from LDS ahead of the barrier (software pipelining) changed nothing.
 #include "ffn_mfma_common.h"
 
 namespace stmoe {
@@ -241,13 +245,9 @@ template <typename T, int MODE>
 static int launch_fp8_ws_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   constexpr int BN = 256, BM = 256;
   constexpr size_t lds_bytes = (size_t)5 * (BN + BM) * 64;
-  static bool attr_set = false;
+  static std::atomic<uint64_t> lds_ready{0};
   auto kern = grouped_fp8_ws_kernel<T, MODE>;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-      return set_error(STMOE_ERR_LAUNCH, "fp8 ws kernel: cannot reserve %zu bytes of LDS", lds_bytes);
-    attr_set = true;
-  }
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ready, "fp8 ws kernel")) return rc;
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;

@@ -280,13 +280,9 @@ template <typename T, int WF, int MODE, int WN, int WM, int STAGES>
 static int launch_big_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
   constexpr int BN = 128 * WN, BM = 64 * WM;
   constexpr size_t lds_bytes = (size_t)(2 * BN + 3 * BM) * BIG_LS * 2;
-  static bool attr_set = false;
+  static std::atomic<uint64_t> lds_ready{0};
   auto kern = grouped_mfma_big_kernel<T, WF, MODE, WN, WM, STAGES>;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-      return set_error(STMOE_ERR_LAUNCH, "mfma big kernel: cannot reserve %zu bytes of LDS", lds_bytes);
-    attr_set = true;
-  }
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ready, "mfma big kernel")) return rc;
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;

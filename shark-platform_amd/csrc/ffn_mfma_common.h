@@ -1,6 +1,7 @@
 // Pieces shared by the prefill kernels: MFMA wrappers, the swizzled LDS row layout, the hand-issued direct
 // global->LDS load and the register form of one packed weight piece.
 #pragma once
+#include <atomic>
 #include "ffn_kernels.h"
 
 namespace stmoe {
@@ -187,6 +188,20 @@ static inline int big_grid(int n_tiles, int slots_bound, bool allow_split) {
   return 8 * ((n_tiles * slots_bound + 7) / 8 + 2 + (allow_split ? 24 : 0));
 }
 static inline size_t big_partial_bytes(int BN, int BM) { return (size_t)8 * kBigChunkSlotsPerXcd * BN * BM * sizeof(float); }
+
+// ---- LDS reservation --------------------------------------------------------------------------------------
+// Kernels that use more than 64 KB of dynamic LDS must be told so once per device.  `done` is a per-kernel bit mask of
+// the devices already set up (a process that uses several GPUs launches the same kernel on each of them).
+static inline int reserve_lds(const void* kernel, size_t bytes, std::atomic<uint64_t>& done, const char* what) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return set_error(STMOE_ERR_LAUNCH, "%s: no current device", what);
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return STMOE_OK;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+    return set_error(STMOE_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", what, bytes);
+  done.fetch_or(bit, std::memory_order_release);
+  return STMOE_OK;
+}
 
 // ---- hand-issued vector-memory operations ------------------------------------------------------------
 // Lane l's 16 bytes at base + byte_off land at LDS byte address lds_addr + 16*l (base and lds_addr wave-uniform).
