@@ -53,6 +53,7 @@ rms_norm_kernel(const T* __restrict__ x, const W* __restrict__ w, int64_t K, flo
 template <typename T> struct Vec8;
 template <> struct Vec8<float> {
   float v[8];
+  __device__ __forceinline__ void from_raw(const uint4&) {}  // (16-bit rows only)
   __device__ __forceinline__ void load(const float* p) {
     const float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
@@ -60,8 +61,8 @@ template <> struct Vec8<float> {
 };
 template <> struct Vec8<f16_t> {
   float v[8];
-  __device__ __forceinline__ void load(const f16_t* p) {
-    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+  __device__ __forceinline__ void load(const f16_t* p) { from_raw(*reinterpret_cast<const uint4*>(p)); }
+  __device__ __forceinline__ void from_raw(const uint4& raw) {
     const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -75,8 +76,8 @@ template <> struct Vec8<f16_t> {
 };
 template <> struct Vec8<bf16_t> {
   float v[8];
-  __device__ __forceinline__ void load(const bf16_t* p) {
-    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+  __device__ __forceinline__ void load(const bf16_t* p) { from_raw(*reinterpret_cast<const uint4*>(p)); }
+  __device__ __forceinline__ void from_raw(const uint4& raw) {
     const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -192,15 +193,53 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
   const int64_t t = blockIdx.x;
   const T* xr = x + t * K;
 
+  // The first expert's router-weight row chunks of this wavefront are requested before anything else, so that their
+  // latency runs in parallel with the norm (they do not depend on it).  PRE chunks of 512 elements are kept in registers.
+  constexpr int PRE = 4;
+  uint4 wpre[PRE];
+  if (sizeof(T) == 2 && wave < E) {  // 16-bit rows (a chunk of 8 elements is one 16-byte load)
+    const T* wrow = wr + (int64_t)wave * K;
+#pragma unroll
+    for (int j = 0; j < PRE; ++j) {
+      const int64_t k0 = (int64_t)lane * 8 + (int64_t)j * 512;
+      if (k0 < K) wpre[j] = *reinterpret_cast<const uint4*>(wrow + k0);
+    }
+  }
   if constexpr (FUSE_NORM) {
+    // the row's elements tid + 512 j are read once and kept (NC of them) for the second pass; the norm weights are
+    // requested before the reduction
+    constexpr int NC = 8;
+    float xv[NC], nw[NC];
     float ss = 0.0f;
-    for (int64_t i = tid; i < K; i += 512) {
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+      const int64_t i = tid + (int64_t)j * 512;
+      if (i < K) {
+        xv[j] = Cvt<T>::to_f32(xr[i]);
+        nw[j] = Cvt<W>::to_f32(norm_w[i]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NC; ++j)
+      if (tid + (int64_t)j * 512 < K) ss = __fadd_rn(ss, __fmul_rn(xv[j], xv[j]));
+    for (int64_t i = tid + (int64_t)NC * 512; i < K; i += 512) {
       const float v = Cvt<T>::to_f32(xr[i]);
       ss = __fadd_rn(ss, __fmul_rn(v, v));
     }
     const float total = block512_sum_sq_finish(ss, part);
     const float rs = rms_scale(total, K, eps);
-    for (int64_t i = tid; i < K; i += 512) {
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+      const int64_t i = tid + (int64_t)j * 512;
+      if (i < K) {
+        float o = round_to<W>(keep_f32(__fmul_rn(xv[j], rs)));
+        o = round_to<W>(keep_f32(__fmul_rn(nw[j], o)));
+        const T r = Cvt<T>::from_f32(o);
+        xs[i] = r;
+        xn[t * K + i] = r;
+      }
+    }
+    for (int64_t i = tid + (int64_t)NC * 512; i < K; i += 512) {
       float o = round_to<W>(keep_f32(__fmul_rn(Cvt<T>::to_f32(xr[i]), rs)));
       o = round_to<W>(keep_f32(__fmul_rn(Cvt<W>::to_f32(norm_w[i]), o)));
       const T r = Cvt<T>::from_f32(o);
@@ -220,13 +259,24 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
   for (int e = wave; e < E; e += 8) {
     float acc = 0.0f;
     const T* wrow = wr + (int64_t)e * K;
-    for (int64_t k0 = (int64_t)lane * 8; k0 < K; k0 += 512) {
+    auto chunk = [&](int64_t k0, const uint4* pre) {
       Vec8<T> xv, wv;
       xv.load(xs + k0);
-      wv.load(wrow + k0);
+      if (pre) wv.from_raw(*pre);  // the prefetched chunk (16-bit rows, the wavefront's first expert)
+      else wv.load(wrow + k0);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc = __fadd_rn(acc, __fmul_rn(xv.v[j], wv.v[j]));
+      for (int jj = 0; jj < 8; ++jj) acc = __fadd_rn(acc, __fmul_rn(xv.v[jj], wv.v[jj]));
+    };
+    const bool pre_ok = sizeof(T) == 2 && e == wave;
+#pragma unroll
+    for (int j = 0; j < PRE; ++j) {  // chunks in increasing order, as the summation order requires
+      const int64_t k0 = (int64_t)lane * 8 + (int64_t)j * 512;
+      if (k0 < K) {
+        if (pre_ok) chunk(k0, &wpre[j]);
+        else chunk(k0, nullptr);
+      }
     }
+    for (int64_t k0 = (int64_t)lane * 8 + (int64_t)PRE * 512; k0 < K; k0 += 512) chunk(k0, nullptr);
     const float l = round_to<T>(wave_xor_sum(acc));
     if (lane == 0) {
       lg_s[e] = l;
