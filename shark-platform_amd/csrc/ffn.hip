@@ -53,7 +53,7 @@ static constexpr int64_t kSkinnyMaxAvgRows = 40;
 // fp8 activations x fp8 weights on the fp8 matrix cores: the 256 x 256 kernel for packed weights and launches with
 // enough rows to fill its tiles (variant 5), the 128 x 128 kernel otherwise (and always with variant 7).
 static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
-  const bool ws_ok = variant == 5 && wtag == WF_FP8_F32D_P && max_rows >= 512 && p.kred % 256 == 0 && p.lda % 16 == 0 &&
+  const bool ws_ok = variant == 5 && wtag == WF_FP8_F32D_P && max_rows >= 320 && p.kred % 256 == 0 && p.lda % 16 == 0 &&
                      p.ldo % 4 == 0 && p.n_out % (mode == MODE_GATEUP ? 128 : 256) == 0 && (!p.offsets || p.E < 64) &&
                      max_rows * p.lda < ((int64_t)1 << 32);
   if (ws_ok) return launch_fp8_ws(dtype, wtag, mode, p, max_rows, st);
@@ -65,7 +65,7 @@ static int run_projection(int variant, int dtype, int wtag, int mode, const Gemm
     if (dtype == STMOE_F32) variant = 1;
     else if (p.offsets && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
                            max_rows <= kSkinnyMaxAvgRows * p.E)) variant = 3;
-    else variant = max_rows >= 512 ? 6 : 2;
+    else variant = max_rows >= 256 ? 6 : 2;  // (grouped launches that are not streamed have more than 40 rows per expert)
   }
   if (variant == 6) {
     int rc = launch_mfma_ws(dtype, wtag, mode, p, max_rows, p.split_scratch, st);
@@ -108,7 +108,7 @@ static FfnWs carve_ffn(int64_t T, int k, int64_t K, int64_t N, int dtype) {
   w.zq = w.xa + align_up((size_t)T * K * es, 256);
   w.split = w.zq + align_up((size_t)T * k * N, 256);
   // fp32 partial tiles of split reductions (prefill kernels only)
-  w.total = w.split + (T * k >= 512 ? align_up(mfma_ws_partial_bytes(), 256) : 0);
+  w.total = w.split + (T * k >= 256 ? align_up(mfma_ws_partial_bytes(), 256) : 0);
   return w;
 }
 
