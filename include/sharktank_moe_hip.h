@@ -181,6 +181,9 @@ size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int64_t K, int
  * weights feeds both operands to the fp8 matrix cores as bytes and scales the fp32 dot product once by scale_x * d_w
  * (variant 7: the same arithmetic on the general 128x128 tile kernel only).
  * x itself is always given unquantised in `dtype`.
+ * `perm` may be NULL when k == 1 and the rows of x are already grouped by expert (sorted row i is row i of x): with
+ * E == 1 and offsets {0, T} this is the plain feed-forward network of one expert (FFNMOE,
+ * sharktank/sharktank/layers/ffn_moe_block.py:77-127).
  * `variant` 0 picks the kernel by shape; other values force one (see the kernel list in ffn.hip). */
 int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                       const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,

@@ -138,7 +138,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   STMOE_REQUIRE(weight_tag(w_gate) == weight_tag(w_up), STMOE_ERR_UNSUPPORTED,
                 "grouped_ffn: gate and up weights must share one format");
   if (T == 0) return STMOE_OK;
-  STMOE_REQUIRE(x && offsets && perm && y_sorted, STMOE_ERR_NULL, "grouped_ffn: NULL pointer");
+  STMOE_REQUIRE(x && offsets && (perm || k == 1) && y_sorted, STMOE_ERR_NULL, "grouped_ffn: NULL pointer");
   STMOE_REQUIRE(aligned16(x) && aligned16(y_sorted) && aligned16(workspace), STMOE_ERR_ALIGN,
                 "grouped_ffn: x, y_sorted and workspace must be 16-byte aligned");
   STMOE_REQUIRE((K * dtype_size(dtype)) % 16 == 0 && (N * dtype_size(dtype)) % 16 == 0, STMOE_ERR_SHAPE,

@@ -1,5 +1,5 @@
 from .base import BaseLayer, ThetaLayer
 from .linear import LinearLayer
 from .norm import RMSNormLayer
-from .ffn_moe_block import PreGatherFFNMOE
+from .ffn_moe_block import FFNMOE, PreGatherFFNMOE, extract_ffn_layer
 from .mixture_of_experts_block import MoeBlock

@@ -14,10 +14,11 @@ import torch.nn.functional as F
 from .. import _hip
 from .. import ops
 from ..ops import device_weight, gather_experts
-from ..types import StaticScaledQuantizer, Theta
+from ..types import DefaultPrimitiveTensor, PlanarQuantizedTensor, QuantizedTensor, StaticScaledQuantizer, Theta
 from .base import ThetaLayer
+from .linear import LinearLayer
 
-__all__ = ["PreGatherFFNMOE", "activation_enum"]
+__all__ = ["FFNMOE", "PreGatherFFNMOE", "activation_enum", "extract_ffn_layer"]
 
 
 def activation_enum(activation) -> int:
@@ -97,3 +98,52 @@ class PreGatherFFNMOE(ThetaLayer):
         xs, zs = self.activation_scales()
         y = _hip.grouped_ffn(h, wg, wu, wd, self._act, offsets, perm, k, variant=self.kernel_variant, x_scale=xs, z_scale=zs)
         return _hip.combine(y, expert_gate.to(h.dtype), inv, T, k)
+
+
+def extract_ffn_layer(merged_tensor, layer_name: str, expert_idx: int):
+    """One expert's matrix out of an expert-stacked weight, named as the reference names it
+    (sharktank/sharktank/layers/ffn_moe_block.py:130-140: `blk.<block>.<layer_name>.<expert>.weight`).  The reference
+    slices plain tensors only; planar quantized tensors are sliced plane by plane here (a view, no copy)."""
+    parts = merged_tensor.name.split(".")
+    block = parts[1] if len(parts) > 1 else "0"
+    name = f"blk.{block}.{layer_name}.{expert_idx}.weight"
+    if isinstance(merged_tensor, QuantizedTensor):
+        planar = merged_tensor.to_planar()
+        layout = planar.unpack()
+        planes = {k: (v[expert_idx] if v.dim() > 0 and v.shape[0] == merged_tensor.shape[0] else v) for k, v in layout.planes.items()}
+        shape = list(merged_tensor.shape[1:])
+        return PlanarQuantizedTensor(name=name, shape=shape, layout=type(layout).create(shape, getattr(layout, "metadata", None), planes))
+    return DefaultPrimitiveTensor(name=name, data=merged_tensor.as_torch()[expert_idx])
+
+
+class FFNMOE(ThetaLayer):
+    """One expert's feed-forward network, `ffn_down(silu(ffn_gate(h)) * ffn_up(h))`: the mirror of the reference's
+    FFNMOE (sharktank/sharktank/layers/ffn_moe_block.py:77-127), built from expert-stacked weights
+    (`ffn_{gate,up,down}_exps.weight[expert_idx]`) or from per-expert thetas (`ffn_gate.<expert_idx>` ...).  The three
+    projections are LinearLayers, as in the reference; `forward` runs them as one fused gate/up kernel and one down
+    kernel (the grouped kernels with a single expert), with every intermediate rounded where the reference's three
+    linears and two element-wise ops round."""
+
+    def __init__(self, theta: Theta, expert_idx=None):
+        super().__init__(theta)
+        if theta.optional_tensor("ffn_gate_exps") is not None or "ffn_gate_exps" in theta.keys:
+            for layer_name in ("ffn_gate", "ffn_up", "ffn_down"):
+                merged = theta.tensor(f"{layer_name}_exps", "weight")
+                expert = extract_ffn_layer(merged_tensor=merged, layer_name=layer_name, expert_idx=expert_idx)
+                self.add_module(layer_name, LinearLayer(Theta({"weight": expert})))
+        else:
+            self.add_module("ffn_gate", LinearLayer(theta("ffn_gate", expert_idx)))
+            self.add_module("ffn_up", LinearLayer(theta("ffn_up", expert_idx)))
+            self.add_module("ffn_down", LinearLayer(theta("ffn_down", expert_idx)))
+        self._dw = None
+
+    def forward(self, h: torch.Tensor):
+        if self._dw is None:
+            self._dw = tuple(device_weight(layer.weight, stacked=False, prepack=True)
+                             for layer in (self.ffn_gate, self.ffn_up, self.ffn_down))
+        wg, wu, wd = self._dw
+        x = h.reshape(-1, h.shape[-1])
+        T = x.shape[0]
+        offsets = torch.tensor([0, T], dtype=torch.int32, device=x.device)
+        y = _hip.grouped_ffn(x, wg, wu, wd, _hip.ACT_SILU, offsets, None, 1)
+        return y.reshape(*h.shape[:-1], y.shape[-1])

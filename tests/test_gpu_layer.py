@@ -206,3 +206,37 @@ def test_forward_under_hip_graph_capture(device, fmt, T):
             scratch = torch.randn(256, 256, device=device) @ torch.randn(256, 256, device=device)  # unrelated eager work
             assert torch.equal(got, want), f"replay {rep} differs from the eager result"
             del scratch
+
+
+@pytest.mark.parametrize("fmt", ["dense", "q8_0", "q4_1"])
+def test_ffnmoe_single_expert_and_cross_check(device, fmt):
+    """FFNMOE (one expert as three linears, sharktank/sharktank/layers/ffn_moe_block.py:77-127) against the oracle's
+    dense arithmetic, against its own three LinearLayers composed with torch's element-wise ops, and as the second
+    formulation of the MoE sum: sum_j gate[t, j] * FFNMOE_{e(t, j)}(x_t) equals PreGatherFFNMOE's output."""
+    from sharktank_amd.layers import FFNMOE, PreGatherFFNMOE
+
+    case = MC.build(MC.Case(T=40, K=256, N=512, fmt=fmt, dtype=torch.float16, seed=77))
+    theta = MC.make_theta(case, device)
+    wg, wu, wd = MC.dense_weights(case)
+    x = case.planes["h"].to(torch.float16)
+    xd = x.to(device)
+    outs = []
+    for e in range(case.E):
+        layer = FFNMOE(theta, expert_idx=e)
+        got = layer(xd)
+        want = O._mm_rt(F.silu(O._mm_rt(x, wg[e])) * O._mm_rt(x, wu[e]), wd[e])
+        assert got.shape == (case.T, case.K) and O.rel_l2(got.cpu(), want) < 1e-3
+        composed = layer.ffn_down(F.silu(layer.ffn_gate(xd)) * layer.ffn_up(xd))  # the reference's forward, op by op
+        assert O.rel_l2(got.cpu(), composed.cpu()) < 1e-3
+        assert layer.ffn_gate.weight.name == f"blk.0.ffn_gate.{e}.weight" or ".ffn_gate." in layer.ffn_gate.weight.name
+        outs.append(got)
+    g = torch.Generator().manual_seed(78)
+    experts = torch.stack([torch.randperm(case.E, generator=g)[: case.k] for _ in range(case.T)]).to(device)
+    gate = torch.rand(case.T, case.k, generator=g).to(torch.float16).to(device)
+    fused = PreGatherFFNMOE(theta)(xd, experts, gate)
+    stacked = torch.stack(outs)  # [E, T, K]
+    second = torch.zeros(case.T, case.K, dtype=torch.float32, device=device)
+    for j in range(case.k):
+        picked = stacked[experts[:, j], torch.arange(case.T, device=device)]
+        second += (gate[:, j:j + 1] * picked).float()
+    assert O.rel_l2(fused.float().cpu(), second.cpu()) < 2e-3
