@@ -114,6 +114,15 @@ int stmoe_dequant_tensor_scaled(const void* qs, int qs_dtype, const void* d, con
 int stmoe_quantize_fp8(const void* x, int x_dtype, const float* rscale, int64_t n, void* out_fp8,
                        stmoe_stream_t stream);
 
+/* DynamicScaledQuantizer._quantize_raw_tensor for float8_e4m3fn (sharktank/sharktank/types/quantizers.py:368-389):
+ * amax = max|x|; scale = T(448 / max(amax, eps)), eps = finfo(float8_e4m3fn).eps = 0.125; rscale = T(1 / scale);
+ * out = e4m3fn(clamp(T(x * scale))), every step in x's dtype T as eager torch computes it.  scale_rscale_out receives
+ * {scale, rscale} (the T values, widened to fp32); `scratch` is device memory of at least
+ * stmoe_dynamic_quantize_fp8_scratch_bytes() bytes.  Two launches, no synchronisation. */
+size_t stmoe_dynamic_quantize_fp8_scratch_bytes(void);
+int stmoe_dynamic_quantize_fp8(const void* x, int dtype, int64_t n, void* out_fp8, float* scale_rscale_out, void* scratch,
+                               size_t scratch_bytes, stmoe_stream_t stream);
+
 /* quantize(x).unpack().dequant() of the same quantizer in one pass (the fake-quantised activations of
  * sharktank/sharktank/layers/linear.py:72-78): out = T(f32(e4m3fn(clamp(T(x / rscale)))) * rscale), T = `dtype`. */
 int stmoe_fake_quant_fp8(const void* x, int dtype, const float* rscale, int64_t n, void* out, stmoe_stream_t stream);

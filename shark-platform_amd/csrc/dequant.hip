@@ -92,6 +92,68 @@ quantize_fp8_kernel(const T* __restrict__ x, const float* __restrict__ rscale, i
   out[i] = f32_to_fp8_e4m3fn(q);
 }
 
+// ---- dynamic per-tensor quantisation -------------------------------------------------------------------------
+// Pass 1: every workgroup writes the maximum of |x| over its grid-stride share (NaN if it saw one, as torch.max does).
+template <typename T>
+__global__ void __launch_bounds__(256)
+absmax_partial_kernel(const T* __restrict__ x, int64_t n, float* __restrict__ partial) {
+  __shared__ float red[4];
+  float m = 0.0f;
+  bool nan = false;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const float v = fabsf(Cvt<T>::to_f32(x[i]));
+    nan |= v != v;
+    m = fmaxf(m, v);
+  }
+  if (nan) m = __uint_as_float(0x7fc00000u);
+  // max is exact and order-independent, so any reduction tree gives the same bits; NaN is carried by hand
+  for (int off = 32; off; off >>= 1) {
+    const float o = __shfl_xor(m, off);
+    m = (m != m || o != o) ? __uint_as_float(0x7fc00000u) : fmaxf(m, o);
+  }
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float r = red[0];
+    for (int w = 1; w < 4; ++w) r = (r != r || red[w] != red[w]) ? __uint_as_float(0x7fc00000u) : fmaxf(r, red[w]);
+    partial[blockIdx.x] = r;
+  }
+}
+// Pass 2: every workgroup folds the partial maxima itself (a few KB from L2), derives the scale as eager torch does in
+// x's dtype T -- scale = T(448 / max(amax, eps)), rscale = T(1 / scale), eps = finfo(float8_e4m3fn).eps = 0.125 -- and
+// quantises its elements: e4m3fn(clamp(T(x * scale))).
+template <typename T>
+__global__ void __launch_bounds__(256)
+dynamic_quantize_fp8_kernel(const T* __restrict__ x, int64_t n, const float* __restrict__ partial, int n_partial,
+                            uint8_t* __restrict__ out, float* __restrict__ scale_rscale) {
+  __shared__ float red[4];
+  float m = 0.0f;
+  for (int i = threadIdx.x; i < n_partial; i += 256) {
+    const float o = partial[i];
+    m = (m != m || o != o) ? __uint_as_float(0x7fc00000u) : fmaxf(m, o);
+  }
+  for (int off = 32; off; off >>= 1) {
+    const float o = __shfl_xor(m, off);
+    m = (m != m || o != o) ? __uint_as_float(0x7fc00000u) : fmaxf(m, o);
+  }
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  float amax = red[0];
+  for (int w = 1; w < 4; ++w) amax = (amax != amax || red[w] != red[w]) ? __uint_as_float(0x7fc00000u) : fmaxf(amax, red[w]);
+  const float clamped = amax != amax ? amax : fmaxf(amax, 0.125f);
+  const float scale = round_to<T>(__fdiv_rn(448.0f, clamped));
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    scale_rscale[0] = scale;
+    scale_rscale[1] = round_to<T>(__fdiv_rn(1.0f, scale));
+  }
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float q = round_to<T>(__fmul_rn(Cvt<T>::to_f32(x[i]), scale));
+  q = fminf(fmaxf(q, -448.0f), 448.0f);
+  if (q != q) q = __uint_as_float(0x7fc00000u);
+  out[i] = f32_to_fp8_e4m3fn(q);
+}
+
 // Quantise and dequantise again in one pass: the values a fake-quantised activation tensor holds.
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -230,6 +292,34 @@ extern "C" int stmoe_quantize_fp8(const void* x, int x_dtype, const float* rscal
     default: return set_error(STMOE_ERR_DTYPE, "quantize_fp8: x dtype %d is not f32/f16/bf16", x_dtype);
   }
   return check_launch("quantize_fp8");
+}
+
+extern "C" size_t stmoe_dynamic_quantize_fp8_scratch_bytes(void) { return 1024 * sizeof(float); }
+
+extern "C" int stmoe_dynamic_quantize_fp8(const void* x, int dtype, int64_t n, void* out_fp8, float* scale_rscale_out,
+                                          void* scratch, size_t scratch_bytes, stmoe_stream_t stream) {
+  STMOE_REQUIRE(n >= 0, STMOE_ERR_SHAPE, "dynamic_quantize_fp8: n %lld < 0", (long long)n);
+  STMOE_REQUIRE(scale_rscale_out && scratch, STMOE_ERR_NULL, "dynamic_quantize_fp8: NULL pointer");
+  STMOE_REQUIRE(scratch_bytes >= stmoe_dynamic_quantize_fp8_scratch_bytes(), STMOE_ERR_WORKSPACE,
+                "dynamic_quantize_fp8: scratch %zu < %zu bytes", scratch_bytes, stmoe_dynamic_quantize_fp8_scratch_bytes());
+  STMOE_REQUIRE(n == 0 || (x && out_fp8), STMOE_ERR_NULL, "dynamic_quantize_fp8: NULL pointer");
+  STMOE_REQUIRE((n + 255) / 256 < ((int64_t)1 << 31), STMOE_ERR_SHAPE, "dynamic_quantize_fp8: n too large");
+  hipStream_t st = as_stream(stream);
+  float* partial = static_cast<float*>(scratch);
+  // an empty tensor has no maximum (torch raises); the scale of amax = 0 is reported and nothing is written
+  const int n_partial = (int)(n == 0 ? 1 : ((n + 2047) / 2048 < 1024 ? (n + 2047) / 2048 : 1024));
+  const dim3 g2((unsigned)(n == 0 ? 1 : (n + 255) / 256));
+#define STMOE_DQ(TT)                                                                                          \
+  absmax_partial_kernel<TT><<<dim3((unsigned)n_partial), 256, 0, st>>>((const TT*)x, n, partial);             \
+  dynamic_quantize_fp8_kernel<TT><<<g2, 256, 0, st>>>((const TT*)x, n, partial, n_partial, (uint8_t*)out_fp8, scale_rscale_out)
+  switch (dtype) {
+    case STMOE_F32: STMOE_DQ(float); break;
+    case STMOE_F16: STMOE_DQ(f16_t); break;
+    case STMOE_BF16: STMOE_DQ(bf16_t); break;
+    default: return set_error(STMOE_ERR_DTYPE, "dynamic_quantize_fp8: dtype %d is not f32/f16/bf16", dtype);
+  }
+#undef STMOE_DQ
+  return check_launch("dynamic_quantize_fp8");
 }
 
 extern "C" int stmoe_fake_quant_fp8(const void* x, int dtype, const float* rscale, int64_t n, void* out,

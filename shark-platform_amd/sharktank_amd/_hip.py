@@ -75,6 +75,8 @@ SIGNATURES = {
     "stmoe_unpack": (c_int, [POINTER(StmoeWeight), POINTER(StmoeWeight), c_void_p]),
     "stmoe_gguf_ingest": (c_int, [c_void_p, c_int, POINTER(StmoeWeight), c_void_p]),
     "stmoe_quantize_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
+    "stmoe_dynamic_quantize_fp8_scratch_bytes": (c_size_t, []),
+    "stmoe_dynamic_quantize_fp8": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "stmoe_fake_quant_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
     "stmoe_rms_norm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_float, c_void_p, c_void_p]),
     "stmoe_router_topk": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -252,6 +254,22 @@ def quantize_fp8(x: torch.Tensor, rscale: torch.Tensor) -> torch.Tensor:
     with torch.cuda.device(dev):
         _check(lib.stmoe_quantize_fp8(_ptr(x_c), dtype_enum(x_c.dtype), _ptr(rs), x_c.numel(), _ptr(out), _stream(dev)))
     return out
+
+
+def dynamic_quantize_fp8(x: torch.Tensor):
+    """DynamicScaledQuantizer for float8_e4m3fn: (qs e4m3fn like x, scale, rscale), the two scales as 0-dim tensors of
+    x's dtype holding the values eager torch computes."""
+    dev = _dev(x)
+    lib = load_library()
+    x_c = _contig(x)
+    out = torch.empty(x_c.shape, dtype=torch.float8_e4m3fn, device=dev)
+    sr = torch.empty(2, dtype=torch.float32, device=dev)
+    scratch = torch.empty(int(lib.stmoe_dynamic_quantize_fp8_scratch_bytes()), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_dynamic_quantize_fp8(_ptr(x_c), dtype_enum(x_c.dtype), x_c.numel(), _ptr(out), _ptr(sr), _ptr(scratch),
+                                              scratch.numel(), _stream(dev)))
+    sr_t = sr.to(x_c.dtype)  # exact: both values were rounded to x's dtype on the device
+    return out, sr_t[0], sr_t[1]
 
 
 def fake_quant_fp8(x: torch.Tensor, rscale: torch.Tensor) -> torch.Tensor:

@@ -11,7 +11,7 @@ import torch
 from .layouts import TensorScaledLayout
 from .tensors import InferenceTensor, PlanarQuantizedTensor, QuantizedTensor, UnnamedTensorName, unbox_tensor
 
-__all__ = ["QuantizerTensor", "StaticScaledQuantizer"]
+__all__ = ["DynamicScaledQuantizer", "QuantizerTensor", "StaticScaledQuantizer"]
 
 
 class QuantizerTensor(InferenceTensor):
@@ -72,4 +72,37 @@ class StaticScaledQuantizer(QuantizerTensor):
         return PlanarQuantizedTensor(
             shape=shape, name=name,
             layout=TensorScaledLayout(shape=shape, d=self._reciprocal_scale, qs=qs, m=None, dtype=t.dtype),
+        )
+
+
+class DynamicScaledQuantizer(QuantizerTensor):
+    """Per-tensor quantizer whose scale comes from the tensor itself: `scale = finfo.max / amax.clamp(finfo.eps)`
+    (mirror of sharktank/sharktank/types/quantizers.py:338-389 for float8_e4m3fn, the fp8 format gfx950's matrix cores
+    consume).  Produces a `TensorScaledLayout` with `d = 1 / scale` and `dtype` = the source dtype, like the reference."""
+
+    def __init__(self, *, dtype: torch.dtype, name: str = UnnamedTensorName):
+        super().__init__(name=name, shape=())
+        if dtype != torch.float8_e4m3fn:
+            raise NotImplementedError(f"DynamicScaledQuantizer: target dtype {dtype} has no kernel (have float8_e4m3fn)")
+        self._dtype = dtype
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self._dtype
+
+    @property
+    def globals(self):
+        return {}
+
+    def _clone_with_globals(self, new_globals):
+        return DynamicScaledQuantizer(dtype=self._dtype, name=self.name)
+
+    def _quantize_raw_tensor(self, t: torch.Tensor, *, name: str) -> QuantizedTensor:
+        from .. import _hip
+
+        qs, _, rscale = _hip.dynamic_quantize_fp8(t)
+        shape = list(t.shape)
+        return PlanarQuantizedTensor(
+            shape=shape, name=name,
+            layout=TensorScaledLayout(shape=shape, d=rscale, qs=qs, m=None, dtype=t.dtype),
         )

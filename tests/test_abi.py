@@ -55,6 +55,9 @@ def test_argument_validation_without_a_gpu():
     rc = lib.stmoe_grouped_ffn(None, _hip.F16, 4, 48, 64, 8, 2, ctypes.byref(w), ctypes.byref(w), ctypes.byref(w), 0,
                                None, None, None, None, None, None, 0, 0, None)
     assert rc == 2 and b"32" in lib.stmoe_last_error()  # Q8_0 needs cols % 32 == 0
+    assert lib.stmoe_dynamic_quantize_fp8_scratch_bytes() == 4096
+    assert lib.stmoe_dynamic_quantize_fp8(None, _hip.F16, 8, None, 16, 16, 16, None) == 6  # scratch too small
+    assert lib.stmoe_dynamic_quantize_fp8(None, _hip.F16, 8, None, 16, 16, 4096, None) == 1  # NULL x
     # raw GGUF blocks: shape, format pairing and streaming-order constraints are checked before any launch
     assert lib.stmoe_gguf_ingest(16, _hip.GGUF_Q8_0, ctypes.byref(w), None) == 2
     w2 = _hip.StmoeWeight(format=_hip.W_Q4_1, dtype=0, experts=1, rows=16, cols=64, qs=16, d=16, m=16, d_count=1)

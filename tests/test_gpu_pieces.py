@@ -438,3 +438,29 @@ def test_layer_from_gguf_raw_blocks(device, fmt):
         assert torch.equal(planar.qs.cpu(), host.qs)
     else:
         assert torch.equal(planar.m.cpu(), host.m) and torch.equal(planar.qs_bit_packed.cpu(), host.qs_bit_packed)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("n,kind", [(1, "normal"), (1000, "normal"), (70001, "normal"), (4096, "zeros"), (4096, "large"), (3000, "tiny")])
+def test_dynamic_quantizer_bit_exact(device, dtype, n, kind):
+    """DynamicScaledQuantizer for float8_e4m3fn (sharktank/sharktank/types/quantizers.py:368-389): samples and the
+    reciprocal scale equal the oracle's, which follows eager torch step by step, bit for bit."""
+    from sharktank_amd import types as ST
+
+    g = torch.Generator().manual_seed(123 + n)
+    x = torch.randn(n, generator=g)
+    if kind == "zeros":
+        x = torch.zeros(n)
+    elif kind == "large":
+        x = x * 3000.0
+    elif kind == "tiny":
+        x = x * 1e-3
+    x = x.to(dtype)
+    want_qs, want_rscale = O.dynamic_quantize(x, torch.float8_e4m3fn)
+    qt = ST.DynamicScaledQuantizer(dtype=torch.float8_e4m3fn).quantize(x.to(device).reshape(-1, 1) if n > 1 else x.to(device))
+    lay = qt.unpack()
+    assert lay.d.dtype == dtype and lay.dtype == dtype
+    assert torch.equal(lay.d.cpu().reshape(()), want_rscale.reshape(()))
+    assert torch.equal(lay.qs.cpu().reshape(-1).view(torch.uint8), want_qs.reshape(-1).view(torch.uint8))
+    # and the layout dequantises as the reference's TensorScaledLayout does
+    assert torch.equal(lay.dequant().cpu().reshape(-1), O.dequant_tensor_scaled(want_rscale, want_qs, layout_dtype=dtype).reshape(-1))
