@@ -145,3 +145,73 @@ def test_forward_unfused_equals_fused(device):
     wg, wu, wd = MC.dense_weights(case)
     want = O.pre_gather_ffn_moe(case.planes["h"], experts.cpu(), gate.cpu(), wg, wu, wd, torch.nn.functional.gelu)
     assert O.rel_l2(b.cpu(), want) < 1e-3
+
+
+# ---- the reference's custom-op layer: same operand sets and argument checks ---------------------------------------
+# Generators as in sharktank/tests/kernels/mmt_block_scaled_q8_test.py:31-41, mmt_block_scaled_offset_q4_test.py:32-44
+# and einsum_q4_test.py:32-89 (fp16 scales); expected values from the layouts' dequantisation (in the scales' dtype,
+# as the eager reference path dequantises) followed by an fp32 product.
+@pytest.mark.parametrize("a_dtype", [torch.float32, torch.float16])
+def test_kernels_mmt_block_scaled_q8(device, a_dtype):
+    from sharktank_amd import kernels
+
+    torch.manual_seed(42)
+    # (the reference's factors of 64 overflow an fp16 result to inf on both sides; fp16 runs use 1/16 instead)
+    amp = 64.0 if a_dtype == torch.float32 else 1.0 / 16
+    a = torch.rand([4, 16, 3200], dtype=a_dtype) * amp
+    d = torch.rand([3200, 100, 1], dtype=torch.float16) * amp
+    qs = (torch.rand([3200, 100, 32], dtype=torch.float32) * 32.0).to(torch.int8)
+    got = kernels.mmt_block_scaled_q8(a.to(device), d.to(device), qs.to(device))
+    b = O.dequant_block_scaled(d, qs).reshape(3200, 3200).to(a_dtype)
+    want = torch.matmul(a.float(), b.float().T)
+    assert got.shape == (4, 16, 3200) and got.dtype == a_dtype
+    assert O.rel_l2(got.float().cpu(), want) < (1e-5 if a_dtype == torch.float32 else 1e-3)
+    with pytest.raises(RuntimeError, match="Expected 3d tensor"):
+        kernels.mmt_block_scaled_q8(a[0].to(device), d.to(device), qs.to(device))
+    with pytest.raises(RuntimeError, match="arg 'qs': Incorrect shape"):
+        kernels.mmt_block_scaled_q8(a.to(device), d.to(device), qs[:, :50].to(device))
+
+
+@pytest.mark.parametrize("a_dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("batched", [False, True])
+def test_kernels_mmt_block_scaled_offset_q4_unsigned(device, a_dtype, batched):
+    from sharktank_amd import kernels
+
+    torch.manual_seed(42)
+    n = 320 if batched else 3200
+    lead = [4] if batched else []
+    a = torch.rand([4, 16, 3200], dtype=a_dtype) / 256.0
+    d = torch.rand(lead + [n, 100, 1], dtype=torch.float16) / 256.0
+    qs = (torch.rand(lead + [n, 100, 16], dtype=torch.float32) * 255.0).to(torch.uint8)
+    m = torch.rand(lead + [n, 100, 1], dtype=torch.float16) + 16.0
+    got = kernels.mmt_block_scaled_offset_q4_unsigned(a.to(device), d.to(device), qs.to(device), m.to(device))
+    b = O.dequant_block_scaled_i4(d, qs, m).reshape(lead + [n, 3200]).to(a_dtype)
+    want = torch.matmul(a.float(), b.float().transpose(-1, -2))
+    assert got.shape == (4, 16, n) and got.dtype == a_dtype
+    assert O.rel_l2(got.float().cpu(), want) < (1e-5 if a_dtype == torch.float32 else 1e-3)
+    with pytest.raises(RuntimeError, match="arg 'm': Incorrect shape"):
+        kernels.mmt_block_scaled_offset_q4_unsigned(a.to(device), d.to(device), qs.to(device), m[..., :50, :].to(device))
+
+
+@pytest.mark.parametrize("a_dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("es", ["mk,menk->men", "mek,menk->men", "me,men->men"])
+def test_kernels_einsum_2args_q4(device, a_dtype, es):
+    from sharktank_amd import kernels
+
+    torch.manual_seed(42)
+    if es == "me,men->men":
+        a = torch.rand([2, 4], dtype=a_dtype) / 256.0
+        planes = [2, 4, 10]
+    else:
+        a = torch.rand([2, 320] if es.startswith("mk") else [2, 4, 320], dtype=a_dtype) / 256.0
+        planes = [2, 4, 8, 10]
+    d = torch.rand(planes + [1], dtype=torch.float16) / 256.0
+    qs = (torch.rand(planes + [16], dtype=torch.float32) * 255.0).to(torch.uint8)
+    m = torch.rand(planes + [1], dtype=torch.float16) + 16.0
+    got = kernels.einsum_2args_q4(a.to(device), d.to(device), qs.to(device), m.to(device), es)
+    b = O.dequant_block_scaled_i4(d, qs, m).flatten(len(planes) - 1).to(a_dtype)
+    want = torch.einsum(es, a.float(), b.float())
+    assert got.shape == want.shape and got.dtype == a_dtype
+    assert O.rel_l2(got.float().cpu(), want) < (1e-5 if a_dtype == torch.float32 else 1e-3)
+    with pytest.raises(NotImplementedError):
+        kernels.einsum_2args_q4(a.to(device), d.to(device), qs.to(device), m.to(device), "ij,jk->ik")
