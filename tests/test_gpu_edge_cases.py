@@ -126,3 +126,42 @@ def test_three_experts_top3_router(device):
     want, want_idx, want_gate = MC.oracle_block(case)
     assert torch.equal(idx.cpu().long(), want_idx)
     assert O.rel_l2(y.reshape(33, case.K).cpu(), want) < 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("E,k,T,K,N,routing", [
+    (8, 2, 400, 256, 128, "random"),      # smallest tile counts the 256 x 256 fp8 kernel takes; every token tile partial
+    (3, 1, 900, 1024, 384, "random"),     # three experts, one slot, full and partial token tiles
+    (8, 2, 600, 512, 768, "two"),         # six experts without rows
+    (1, 1, 513, 256, 256, "random"),      # one expert: two full tiles and a one-row tile
+])
+def test_fp8_matrix_core_kernels_agree(device, dtype, E, k, T, K, N, routing):
+    """fp8 activations x fp8 weights: the 256 x 256 kernel with direct global -> LDS loads (variant 5) against the
+    128 x 128 kernel (variant 7) -- the same arithmetic, up to the order of the fp32 sums -- and both against the
+    oracle's quantise-dequantise arithmetic at the fp8 tolerance."""
+    from sharktank_amd import _hip as hip
+    from sharktank_amd.ops import device_weight
+
+    case = MC.build(MC.Case(T=T, K=K, N=N, E=E, k=k, fmt="fp8", dtype=dtype, act_quant=True, seed=90 + E + T))
+    g = torch.Generator().manual_seed(case.seed)
+    if routing == "two":
+        idx = torch.tensor([[1, 6]]).repeat(T, 1)
+    else:
+        idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    x = case.planes["h"]
+    gate = torch.rand(T, k, generator=g)
+    gate = (gate / gate.sum(-1, keepdim=True)).to(dtype)
+    wg, wu, wd = MC.dense_weights(case)
+    xs, zs = case.planes["x_rscale"], case.planes["z_rscale"]
+    want = O.grouped_ffn_moe(x, idx, gate, wg, wu, wd, case.activation, x_rscale=xs, z_rscale=zs)
+    dws = [device_weight(MC.to_inference_tensor("fp8", case.planes[n], shp, n, device), stacked=True, prepack=True)
+           for n, shp in (("gate", [E, N, K]), ("up", [E, N, K]), ("down", [E, K, N]))]
+    _, offsets, perm, inv = hip.dispatch_build(idx.to(torch.int32).to(device), E)
+    outs = {}
+    for variant in (hip.VARIANT_FP8_MFMA, hip.VARIANT_FP8_TILE):
+        y = hip.grouped_ffn(x.to(device), dws[0], dws[1], dws[2], hip.ACT_SILU, offsets, perm, k, variant=variant,
+                            x_scale=xs.to(device), z_scale=zs.to(device))
+        outs[variant] = hip.combine(y, gate.to(device), inv, T, k).cpu()
+    a, b = outs[hip.VARIANT_FP8_MFMA], outs[hip.VARIANT_FP8_TILE]
+    assert O.rel_l2(a, b) < (2e-3 if dtype == torch.float16 else 1.5e-2), "the two fp8 kernels disagree"
+    assert O.rel_l2(a, want) < 6e-2 and O.rel_l2(b, want) < 6e-2
