@@ -11,8 +11,8 @@
 //            MFMA lane (r, h) supplies row r, samples 32 h .. 32 h + 31: pieces' units 2 h and 2 h + 1 of row r % 16,
 //            16 consecutive lanes read 256 consecutive bytes.
 //   tokens:  quantised rows, 64 bytes per stage; lane l of a load fetches the 16 bytes that belong at LDS position l
-//            (row l / 4 of its 16 rows, unit (l % 4) ^ ((row / 4) % 4 ... see x_unit), so that the gather and the bank swizzle
-//            cost nothing; rows of a partial token tile are spread over the four token-row groups.
+//            (row l / 4 of the load's 16 rows, the unit that x_unit maps to position l % 4), so that the gather and the
+//            bank swizzle cost nothing; rows of a partial token tile are spread over the four token-row groups.
 //   results: D[8 (i / 4) + 4 h + i % 4][r] (probed on the hardware: rows are the weight rows, columns the token rows);
 //            both token blocks' operands (16 registers) stay resident while the four weight blocks stream through 8
 //            registers, so every operand byte is read from LDS once per wavefront.
