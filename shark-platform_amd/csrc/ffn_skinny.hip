@@ -139,16 +139,15 @@ template <> struct SkinnyW<WF_FP8_F32D> {
   }
   template <typename T> __device__ __forceinline__ u32x4_t frag(int s, int g) const {
     const int i = s >> 1, h = s & 1;
-    u32x4_t out;
+    float f[8];
+    fp8x4_to_f32(q[i][2 * h], f);
+    float f2[4];
+    fp8x4_to_f32(q[i][2 * h + 1], f2);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const uint32_t u = q[i][2 * h + j];
-      float f[4];
-      fp8x4_to_f32(u, f);
-      out[2 * j] = scale2_pack<T>(f[0], f[1], dv);
-      out[2 * j + 1] = scale2_pack<T>(f[2], f[3], dv);
-    }
-    return out;
+    for (int b = 0; b < 4; ++b) f[4 + b] = f2[b];
+    uint32_t o[4];
+    scale8_pack<T>(f, dv, o);
+    return (u32x4_t){o[0], o[1], o[2], o[3]};
   }
 };
 

@@ -57,17 +57,29 @@ template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
-// pack2<T>(a0 * d, a1 * d) with each product rounded to fp32 and then to T.  For fp16 the mixed-precision fused
-// multiply-add writes each half of the result in place (fp32 arithmetic, then the conversion): two instructions
-// instead of two multiplies and a packed conversion.
-template <typename T> __device__ __forceinline__ uint32_t scale2_pack(float a0, float a1, float d) {
+// Eight products a[i] * d, each rounded to fp32 and then to T, packed into four dwords.  For fp16 the mixed-precision
+// fused multiply-add writes each half of a result dword in place (fp32 arithmetic, then the conversion): one instruction
+// per element instead of a multiply per element and a packed conversion per pair.  These instructions write half a
+// register, and on this ISA a read of such a register needs one wait state after the write; the compiler's hazard
+// handling cannot see into inline assembly, so the sequence is ordered to keep every dependent pair at least three
+// instructions apart and ends with an s_nop of two wait states, which covers the half-register read hazard and the
+// wait a matrix-core instruction needs after a vector write of one of its operands.
+template <typename T> __device__ __forceinline__ void scale8_pack(const float (&a)[8], float d, uint32_t (&out)[4]) {
   if constexpr (__is_same(T, f16_t)) {
-    uint32_t r;
-    asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(r) : "v"(a0), "v"(d));
-    asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(r) : "v"(a1), "v"(d));
-    return r;
+    asm("v_fma_mixlo_f16 %0, %4, %12, 0\n\t"
+        "v_fma_mixlo_f16 %1, %6, %12, 0\n\t"
+        "v_fma_mixlo_f16 %2, %8, %12, 0\n\t"
+        "v_fma_mixlo_f16 %3, %10, %12, 0\n\t"
+        "v_fma_mixhi_f16 %0, %5, %12, 0\n\t"
+        "v_fma_mixhi_f16 %1, %7, %12, 0\n\t"
+        "v_fma_mixhi_f16 %2, %9, %12, 0\n\t"
+        "v_fma_mixhi_f16 %3, %11, %12, 0\n\t"
+        "s_nop 1"
+        : "=&v"(out[0]), "=&v"(out[1]), "=&v"(out[2]), "=&v"(out[3])
+        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7]), "v"(d));
   } else {
-    return pack2<T>(__fmul_rn(a0, d), __fmul_rn(a1, d));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = pack2<T>(__fmul_rn(a[2 * i], d), __fmul_rn(a[2 * i + 1], d));
   }
 }
 

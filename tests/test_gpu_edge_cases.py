@@ -165,3 +165,57 @@ def test_fp8_matrix_core_kernels_agree(device, dtype, E, k, T, K, N, routing):
     a, b = outs[hip.VARIANT_FP8_MFMA], outs[hip.VARIANT_FP8_TILE]
     assert O.rel_l2(a, b) < (2e-3 if dtype == torch.float16 else 1.5e-2), "the two fp8 kernels disagree"
     assert O.rel_l2(a, want) < 6e-2 and O.rel_l2(b, want) < 6e-2
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_streaming_kernel_two_row_tiles_in_one_pass(device, fmt, dtype):
+    """33 tokens over 16 experts with one expert taking 30 rows: the streaming kernel multiplies two 16-row tiles of
+    that expert with one weight fragment.  (The first tile once read fp8 fragments whose fp16 halves had been written by
+    half-register instructions one cycle earlier, without the wait state that such a read needs.)"""
+    case = MC.build(MC.Case(T=33, K=1024, N=1024, E=16, k=2, fmt=fmt, dtype=dtype, seed=1006))
+    idx = torch.zeros(33, 2, dtype=torch.long)
+    idx[:, 1] = 1 + torch.arange(33) % 15
+    idx[30:, 0] = torch.tensor([2, 3, 4])
+    idx[30:, 1] = torch.tensor([5, 6, 7])
+    got, want = _run(device, case, idx)
+    assert O.rel_l2(got, want) < (1e-3 if dtype == torch.float16 else 8e-3)
+
+
+def test_random_shapes_automatic_choice_against_vector_alu_kernel(device):
+    """Seeded random shapes, formats, routings and activations: the automatically chosen kernels against the vector-ALU
+    kernel (an independent implementation of the same arithmetic)."""
+    import random
+    from sharktank_amd import _hip as hip
+    from sharktank_amd.ops import device_weight
+
+    rng = random.Random(2024)
+    for it in range(40):
+        fmt = rng.choice(["q8_0", "q4_1", "fp8", "dense"])
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        E = rng.choice([1, 2, 3, 5, 8, 16])
+        k = rng.randint(1, min(E, 3))
+        K = rng.choice([256, 512, 768, 1024])
+        N = rng.choice([128, 256, 384, 512, 1024])
+        T = rng.choice([1, 3, 17, 33, 64, 100, 200, 330, 600, 1100])
+        mode = rng.choice(["uniform", "skew", "few"])
+        case = MC.build(MC.Case(T=T, K=K, N=N, E=E, k=k, fmt=fmt, dtype=dtype, seed=3000 + it))
+        g = torch.Generator().manual_seed(it)
+        if mode == "uniform":
+            idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+        elif mode == "skew":
+            w = torch.tensor([1.0 / (e + 1) ** 2 for e in range(E)])
+            idx = torch.stack([torch.multinomial(w, k, replacement=False, generator=g) for _ in range(T)])
+        else:
+            idx = torch.randperm(E, generator=g)[:k].repeat(T, 1)
+        what = f"case {it}: {fmt} {dtype} E={E} k={k} K={K} N={N} T={T} {mode}"
+        print(what, flush=True)
+        dws = [device_weight(MC.to_inference_tensor(fmt, case.planes[n], shp, n, device), stacked=True, prepack=True)
+               for n, shp in (("gate", [E, N, K]), ("up", [E, N, K]), ("down", [E, K, N]))]
+        _, offsets, perm, _ = hip.dispatch_build(idx.to(torch.int32).to(device), E)
+        x = case.planes["h"].to(device)
+        act = rng.choice([hip.ACT_SILU, hip.ACT_GELU_ERF])
+        auto = hip.grouped_ffn(x, *dws, act, offsets, perm, k, variant=hip.VARIANT_AUTO)
+        alu = hip.grouped_ffn(x, *dws, act, offsets, perm, k, variant=hip.VARIANT_GENERIC)
+        err = O.rel_l2(auto.float().cpu(), alu.float().cpu())
+        assert torch.isfinite(auto.float()).all() and err < (2e-3 if dtype == torch.float16 else 1.2e-2), f"{what}: rel-L2 {err:.3e}"
