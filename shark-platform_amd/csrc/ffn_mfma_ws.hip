@@ -130,8 +130,14 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     }
     if (nkt > 2) load_w(WsInt<2>{}, 2);
     store_w(WsInt<0>{}, WsInt<0>{});
-    if (nkt > 3) load_w(WsInt<0>{}, 3);
-    vm_wait<0>();
+    if (nkt > 3) {
+      load_w(WsInt<0>{}, 3);
+      // step 0 needs the weights (stored above) and the token rows of step 0 only: issued after those token loads are
+      // the weight loads of steps 1, 2, 3 and the token loads of step 1, which may stay in flight
+      vm_wait<3 * WLOADS + XLOADS>();
+    } else {
+      vm_wait<0>();
+    }
     __syncthreads();
     int64_t kt = 0;
     for (; kt + 9 < nkt; kt += 6) {
