@@ -63,8 +63,8 @@ static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const 
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
-    else if (p.offsets && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
-                           max_rows <= kSkinnyMaxAvgRows * p.E)) variant = 3;
+    else if ((p.offsets || p.E == 1) && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
+                                         max_rows <= kSkinnyMaxAvgRows * p.E)) variant = 3;
     else variant = max_rows >= 256 ? 6 : 2;  // (grouped launches that are not streamed have more than 40 rows per expert)
   }
   if (variant == 6) {

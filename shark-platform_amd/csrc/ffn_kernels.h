@@ -33,6 +33,17 @@ struct GemmParams {
   float* split_scratch;       // optional fp32 scratch for split reductions (mfma_ws_partial_bytes() bytes)
 };
 
+// Row range of expert e; without offsets there is one expert with `fixed_rows` rows.
+__device__ __forceinline__ void expert_range(const GemmParams& p, int e, int& row_begin, int& row_end) {
+  if (p.offsets) {
+    row_begin = p.offsets[e];
+    row_end = p.offsets[e + 1];
+  } else {
+    row_begin = 0;
+    row_end = (int)p.fixed_rows;
+  }
+}
+
 // (expert, first row, end row) of m-tile `slot` when every expert's rows are cut into tiles of BM.
 __device__ __forceinline__ bool find_tile(const GemmParams& p, int slot, int BM, int& e, int& row_begin, int& row_end) {
   if (!p.offsets) {

@@ -359,11 +359,14 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
   // experts that received rows, in increasing id
   int n_active = 0;
   uint64_t active_mask = 0;
-  for (int e = 0; e < p.E; ++e)
-    if (p.offsets[e + 1] > p.offsets[e]) {
+  for (int e = 0; e < p.E; ++e) {
+    int b, en;
+    expert_range(p, e, b, en);
+    if (en > b) {
       active_mask |= 1ull << e;
       ++n_active;
     }
+  }
   const int n_items = n_active * tiles_per_expert;
 
   for (int item = wave_global; item < n_items; item += total_waves) {
@@ -377,7 +380,8 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves) {
           ++seen;
         }
     }
-    const int rb = p.offsets[e], re = p.offsets[e + 1];
+    int rb, re;
+    expert_range(p, e, rb, re);
 
     // the two weight tiles of this item
     int64_t wrow[2];
@@ -535,11 +539,14 @@ grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
       (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)xs));
   int n_active = 0;
   uint64_t active_mask = 0;
-  for (int e = 0; e < p.E; ++e)
-    if (p.offsets[e + 1] > p.offsets[e]) {
+  for (int e = 0; e < p.E; ++e) {
+    int b, en;
+    expert_range(p, e, b, en);
+    if (en > b) {
       active_mask |= 1ull << e;
       ++n_active;
     }
+  }
   const int groups_per_expert = tiles_per_expert >> 2;
   const int n_groups = n_active * groups_per_expert;
   for (int grp = blockIdx.x; grp < n_groups; grp += gridDim.x) {
@@ -553,7 +560,8 @@ grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
           ++seen;
         }
     }
-    const int rb = p.offsets[e], re = p.offsets[e + 1];
+    int rb, re;
+    expert_range(p, e, rb, re);
     int64_t wrow[2];
     if (MODE == MODE_GATEUP) {
       wrow[0] = (int64_t)e * p.w0.rows + tile * 16 + n_in;
@@ -615,8 +623,8 @@ static int launch_skinny_t(int mode, const GemmParams& p, int64_t max_rows, hipS
 }
 
 int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
-  if (!p.offsets || p.E > 64)
-    return set_error(STMOE_ERR_UNSUPPORTED, "skinny kernel: needs per-expert offsets and at most 64 experts");
+  if ((!p.offsets && p.E != 1) || p.E > 64 || (!p.offsets && p.fixed_rows >= ((int64_t)1 << 31)))
+    return set_error(STMOE_ERR_UNSUPPORTED, "skinny kernel: needs per-expert offsets (or a single matrix) and at most 64 experts");
   if (p.kred % 256 != 0 || p.n_out % 32 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0)
     return set_error(STMOE_ERR_UNSUPPORTED, "skinny kernel: needs K %% 256 == 0 and N %% 32 == 0");
   if (max_rows == 0) return STMOE_OK;

@@ -62,6 +62,33 @@ def test_linear_and_dense_matmul(device):
         ops.matmul(x.to(device), w.to(device), transpose_rhs=False)
 
 
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 32, 33, 40])
+def test_quantized_linear_few_rows(device, fmt, dtype, M):
+    """One quantized matrix times a handful of rows (a Llama-style projection at decode): the streaming kernel runs
+    without an expert offsets array, from planar and from packed planes, with the same bits from both."""
+    import moe_cases as MC
+    from sharktank_amd import _hip
+    from sharktank_amd.ops import device_weight
+
+    N, K = 96, 1024
+    case = MC.build(MC.Case(T=4, K=K, N=N, E=1, k=1, fmt=fmt, dtype=dtype, seed=90 + M))
+    it = MC.to_inference_tensor(fmt, case.planes["gate"], [1, N, K], "w", device)
+    x = (torch.randn(M, K, generator=torch.Generator().manual_seed(M)) * 0.5).to(dtype)
+    w_ref = MC.dense_weights(case)[0][0].to(dtype)
+    ref = O.mmt(x, w_ref)
+    outs = []
+    for prepack in (False, True):
+        dw = device_weight(it, stacked=True, prepack=prepack)
+        auto = _hip.mmt(x.to(device), dw)
+        assert O.rel_l2(auto.cpu(), ref) < (1e-3 if dtype == torch.float16 else 8e-3)
+        # the automatic choice for so few rows is the streaming kernel
+        assert torch.equal(auto.view(torch.int16), _hip.mmt(x.to(device), dw, variant=_hip.VARIANT_SKINNY).view(torch.int16))
+        outs.append(auto.cpu())
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+
+
 def test_layout_classes_dequant_on_device(device):
     from sharktank_amd import types as ST
 
