@@ -15,6 +15,7 @@ import torch.nn.functional as F
 
 from .. import _hip
 from ..types import Theta, unbox_tensor
+from ..utils import debugging
 from .base import ThetaLayer
 from .ffn_moe_block import PreGatherFFNMOE
 from .linear import LinearLayer
@@ -62,13 +63,25 @@ class MoeBlock(ThetaLayer):
         if self._workspace is None or self._workspace.numel() < need or self._workspace.device != h.device:
             self._workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=h.device)
         xs, zs = self.experts.activation_scales()
+        # With tracing or golden dumps switched on, the routing is fetched as well and recorded beside the output (the
+        # kernels and the results are the same either way).
+        tracing = debugging.flags.enable_tensor_trace or debugging.flags.save_goldens_path is not None
         res = _hip.moe_forward(
             x, unbox_tensor(self.ffn_norm.weight), out_norm_w, self.rms_epsilon, self._router_weight(h.dtype),
             wg, wu, wd, self.experts._act, self.expert_used_count,
-            variant=self.experts.kernel_variant, workspace=self._workspace, want_routing=return_routing,
+            variant=self.experts.kernel_variant, workspace=self._workspace, want_routing=return_routing or tracing,
             x_scale=xs, z_scale=zs,
         )
-        if return_routing:
+        if return_routing or tracing:
             out, idx, gate = res
-            return out.reshape(batch_size, sequence_length, feature_dim), idx, gate
-        return res.reshape(batch_size, sequence_length, feature_dim)
+        else:
+            out, idx, gate = res, None, None
+        out = out.reshape(batch_size, sequence_length, feature_dim)
+        if tracing:
+            record = {"top_k_experts": idx, "expert_gate": gate, "output": out}
+            self.trace_tensors("moe_block", record)
+            self.trace_goldens("moe_block", record)
+        self.assert_not_nan(out)
+        if return_routing:
+            return out, idx, gate
+        return out

@@ -240,3 +240,35 @@ def test_ffnmoe_single_expert_and_cross_check(device, fmt):
         picked = stacked[experts[:, j], torch.arange(case.T, device=device)]
         second += (gate[:, j:j + 1] * picked).float()
     assert O.rel_l2(fused.float().cpu(), second.cpu()) < 2e-3
+
+
+def test_trace_hooks_dump_routing_and_output(device, tmp_path, capsys):
+    """With golden dumps switched on (the reference's TURBINE_LLM_DEBUG=save_goldens_path=...), a forward of the block
+    leaves one file holding its routing and its output, equal to what the call returns and to a forward without
+    dumps; a model's own `trace_tensor` calls go through the same switchboard."""
+    from safetensors.torch import load_file
+    from sharktank_amd.layers import MoeBlock
+    from sharktank_amd.utils import debugging
+
+    case = MC.build(MC.Case(T=24, K=256, N=512, fmt="q4_1", dtype=torch.float16, seed=63))
+    theta = MC.make_theta(case, device)
+    block = MoeBlock(theta, expert_count=case.E, expert_used_count=case.k, rms_epsilon=case.eps)
+    h = case.planes["h"].reshape(2, 12, case.K).to(device)
+    plain = block(h)
+    saved = debugging.DebugFlags(**vars(debugging.flags))
+    try:
+        debugging.flags.save_goldens_path = tmp_path
+        debugging.flags.golden_sequence_value = 0
+        debugging.flags.enable_nan_checks = True
+        out, idx, gate = block(h, return_routing=True)
+        block.trace_golden("mixtral.moe_block.0.output", out)
+    finally:
+        for k, v in vars(saved).items():
+            setattr(debugging.flags, k, v)
+    assert torch.equal(out, plain)
+    files = sorted(p.name for p in tmp_path.iterdir())
+    assert files == ["0000_moe_block.safetensors", "0001_mixtral.moe_block.0.output.safetensors"]
+    dump = load_file(tmp_path / files[0])
+    assert torch.equal(dump["output"], out.cpu())
+    assert torch.equal(dump["top_k_experts"], idx.cpu()) and torch.equal(dump["expert_gate"], gate.cpu())
+    assert torch.equal(load_file(tmp_path / files[1])["default"], out.cpu())
