@@ -90,7 +90,10 @@ template <> struct SkinnyW<WF_Q8_0> {
 
 template <> struct SkinnyW<WF_Q4_1> {
   u32x4_t q[2];
-  uint16_t d[2], m[2];  // scale / offset of the lane's own two blocks (4*i + g, i = 0, 1)
+  // fp16 bits of the scale / offset of the lane's own two blocks (4*i + g, i = 0, 1).  Kept as 32-bit values: a 16-bit
+  // field is zero-extended again where a register of it is named, and the compiler placed that instruction, with a
+  // wait for the prefetch just issued, in the middle of the running chunk, which serialised load and compute.
+  uint32_t d[2], m[2];
   __device__ __forceinline__ void init(const WeightView&, int64_t) {}
   __device__ __forceinline__ void touch() { asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(d[0]), "+v"(d[1]), "+v"(m[0]), "+v"(m[1])); }
   __device__ __forceinline__ void load(const WeightView& w, int64_t row, int64_t c, int g) {
@@ -523,7 +526,7 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
   }
 }
 
-// Workgroups per CU (three for the 4-bit format, which needs fewer registers, measured no faster).
+// Workgroups per CU (three for the 4-bit format, which then has to fit 168 registers, measured 4-10 % slower).
 template <int WF> struct SkinnyLdsOcc { static constexpr int value = 2; };
 
 // A workgroup takes groups of four neighbouring items (tiles 4q .. 4q+3 of one expert), strided by the grid size.
