@@ -195,28 +195,50 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
 
   // The first expert's router-weight row chunks of this wavefront are requested before anything else, so that their
   // latency runs in parallel with the norm (they do not depend on it).  PRE chunks of 512 elements are kept in registers.
+  // Rows of at least NC * 512 elements (the usual case) take their first loads without a bounds test per load: loads
+  // under separate conditions are waited for one by one, those of a straight line are all in flight together.
   constexpr int PRE = 4;
+  constexpr int NC = 8;
+  const bool long_row = K >= (int64_t)NC * 512;
   uint4 wpre[PRE];
   if (sizeof(T) == 2 && wave < E) {  // 16-bit rows (a chunk of 8 elements is one 16-byte load)
     const T* wrow = wr + (int64_t)wave * K;
+    if (long_row) {
 #pragma unroll
-    for (int j = 0; j < PRE; ++j) {
-      const int64_t k0 = (int64_t)lane * 8 + (int64_t)j * 512;
-      if (k0 < K) wpre[j] = *reinterpret_cast<const uint4*>(wrow + k0);
+      for (int j = 0; j < PRE; ++j) wpre[j] = *reinterpret_cast<const uint4*>(wrow + lane * 8 + j * 512);
+    } else {
+#pragma unroll
+      for (int j = 0; j < PRE; ++j) {
+        const int64_t k0 = (int64_t)lane * 8 + (int64_t)j * 512;
+        if (k0 < K) wpre[j] = *reinterpret_cast<const uint4*>(wrow + k0);
+      }
     }
   }
   if constexpr (FUSE_NORM) {
     // the row's elements tid + 512 j are read once and kept (NC of them) for the second pass; the norm weights are
     // requested before the reduction
-    constexpr int NC = 8;
     float xv[NC], nw[NC];
     float ss = 0.0f;
+    if (long_row) {
+      T xraw[NC];
+      W wraw[NC];
 #pragma unroll
-    for (int j = 0; j < NC; ++j) {
-      const int64_t i = tid + (int64_t)j * 512;
-      if (i < K) {
-        xv[j] = Cvt<T>::to_f32(xr[i]);
-        nw[j] = Cvt<W>::to_f32(norm_w[i]);
+      for (int j = 0; j < NC; ++j) xraw[j] = xr[tid + j * 512];
+#pragma unroll
+      for (int j = 0; j < NC; ++j) wraw[j] = norm_w[tid + j * 512];
+#pragma unroll
+      for (int j = 0; j < NC; ++j) {
+        xv[j] = Cvt<T>::to_f32(xraw[j]);
+        nw[j] = Cvt<W>::to_f32(wraw[j]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NC; ++j) {
+        const int64_t i = tid + (int64_t)j * 512;
+        if (i < K) {
+          xv[j] = Cvt<T>::to_f32(xr[i]);
+          nw[j] = Cvt<W>::to_f32(norm_w[i]);
+        }
       }
     }
 #pragma unroll
