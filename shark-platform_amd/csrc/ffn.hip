@@ -328,12 +328,15 @@ static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int6
   if (!fused_front && (rc = stmoe_rms_norm(h, dtype, ffn_norm_w, w_dtype, T, K, eps, xn, stream))) return rc;
   mark(events, 1, st);
   mark(events, 2, st);
-  if (fused_front) rc = norm_router(h, dtype, ffn_norm_w, w_dtype, eps, xn, w_router, T, K, E, k, idx, gate, st);
+  // a single token's dispatch is written by the router launch itself
+  const bool router_dispatches = fused_front && T == 1;
+  if (fused_front) rc = norm_router(h, dtype, ffn_norm_w, w_dtype, eps, xn, w_router, T, K, E, k, idx, gate, st,
+                                    router_dispatches ? counts : nullptr, offsets, perm, inv);
   else rc = stmoe_router_topk(xn, w_router, dtype, T, K, E, k, nullptr, idx, nullptr, gate, stream);
   if (rc) return rc;
   mark(events, 3, st);
   mark(events, 4, st);
-  if ((rc = stmoe_dispatch_build(idx, T * k, E, counts, offsets, perm, inv, stream))) return rc;
+  if (!router_dispatches && (rc = stmoe_dispatch_build(idx, T * k, E, counts, offsets, perm, inv, stream))) return rc;
   mark(events, 5, st);
   if ((rc = grouped_ffn_impl(xn, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, z_scale, y,
                              base + ws.ffn, workspace_bytes - ws.ffn, variant, stream, events ? events + 6 : nullptr)))

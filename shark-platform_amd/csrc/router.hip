@@ -180,11 +180,17 @@ router_topk_kernel(const T* __restrict__ x, const T* __restrict__ wr, int64_t T_
 // all loads of a logit be in flight at once, which is what a 32-token decode batch needs.
 // FUSE_NORM: the workgroup first normalises the token row (rms_norm_kernel's arithmetic), writes it to `xn`
 // (the expert projections read it) and routes the normalised row kept in LDS.
+// Dispatch arrays of a one-token launch (all NULL otherwise): counts [E], offsets [E+1], perm [k], inv [k].
+struct SingleTokenDispatch {
+  int32_t *counts, *offsets, *perm, *inv;
+};
+
 template <typename T, typename W, bool FUSE_NORM>
 __global__ void __launch_bounds__(512)
 router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float eps, T* __restrict__ xn,
                  const T* __restrict__ wr, int64_t K, int E, int k, T* __restrict__ logits_out,
-                 int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out, T* __restrict__ gate_out) {
+                 int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out, T* __restrict__ gate_out,
+                 SingleTokenDispatch disp) {
   extern __shared__ __align__(16) unsigned char smem[];
   T* xs = reinterpret_cast<T*>(smem);                                  // [K] the (normalised) token row
   float* lg_s = reinterpret_cast<float*>(smem + ((K * sizeof(T) + 15) / 16) * 16);  // [E] logits, then 8 partials
@@ -334,22 +340,44 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
     vsum += p;
   }
   for (int j = 0; j < k; ++j) gate_out[t * k + j] = Cvt<T>::from_f32(part[8 + j] / vsum);
+
+  // A launch of one token can also write that token's dispatch (what dispatch_build_kernel would compute from idx):
+  // every chosen expert has one row, the rows are ordered by expert id, pair j sits at the number of chosen experts
+  // with a smaller id.  Saves a kernel launch where a forward is a handful of short launches.
+  if (disp.counts) {
+    for (int e = 0; e < E; ++e) {
+      disp.counts[e] = (int32_t)((taken >> e) & 1ull);
+      disp.offsets[e] = (int32_t)__popcll(taken & ((1ull << e) - 1ull));
+    }
+    disp.offsets[E] = k;
+    for (int j = 0; j < k; ++j) {
+      const int e = idx_out[j];
+      const int pos = (int)__popcll(taken & ((1ull << e) - 1ull));
+      disp.perm[pos] = j;
+      disp.inv[j] = pos;
+    }
+  }
 }
 
 template <typename T, typename W, bool FUSE_NORM>
 static int launch_router_wg(const void* x, const void* norm_w, float eps, void* xn, const void* wr, int64_t T_tokens,
-                            int64_t K, int E, int k, void* logits, int32_t* idx, int64_t* idx64, void* gate, hipStream_t st) {
+                            int64_t K, int E, int k, void* logits, int32_t* idx, int64_t* idx64, void* gate, hipStream_t st,
+                            SingleTokenDispatch disp = SingleTokenDispatch{nullptr, nullptr, nullptr, nullptr}) {
   const size_t lds = ((K * sizeof(T) + 15) / 16) * 16 + (64 + 8 + 64) * sizeof(float);
   if (lds > 64 * 1024) return set_error(STMOE_ERR_UNSUPPORTED, "router: K=%lld does not fit the per-token LDS row", (long long)K);
   router_wg_kernel<T, W, FUSE_NORM><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
-      (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate);
+      (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
   return check_launch("router_wg");
 }
 
 // ffn_norm + router in one launch (used by the fused layer forward).  norm weight dtype: f32, or the activation dtype.
+// With all four dispatch pointers given and T_tokens == 1 the launch also writes the token's dispatch arrays.
 int norm_router(const void* h, int dtype, const void* norm_w, int w_dtype, float eps, void* xn, const void* wr,
-                int64_t T_tokens, int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st) {
-#define STMOE_NR(TT, WW) return launch_router_wg<TT, WW, true>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, nullptr, idx, nullptr, gate, st)
+                int64_t T_tokens, int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st,
+                int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv) {
+  SingleTokenDispatch disp{nullptr, nullptr, nullptr, nullptr};
+  if (T_tokens == 1 && counts && offsets && perm && inv) disp = SingleTokenDispatch{counts, offsets, perm, inv};
+#define STMOE_NR(TT, WW) return launch_router_wg<TT, WW, true>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, nullptr, idx, nullptr, gate, st, disp)
   if (dtype == STMOE_F32 && w_dtype == STMOE_F32) STMOE_NR(float, float);
   if (dtype == STMOE_F16 && w_dtype == STMOE_F32) STMOE_NR(f16_t, float);
   if (dtype == STMOE_BF16 && w_dtype == STMOE_F32) STMOE_NR(bf16_t, float);

@@ -15,7 +15,8 @@ namespace stmoe {
 int set_error(int code, const char* fmt, ...);
 int check_launch(const char* what);
 int norm_router(const void* h, int dtype, const void* norm_w, int w_dtype, float eps, void* xn, const void* wr,
-                int64_t T_tokens, int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st);
+                int64_t T_tokens, int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st,
+                int32_t* counts = nullptr, int32_t* offsets = nullptr, int32_t* perm = nullptr, int32_t* inv = nullptr);
 
 #define STMOE_REQUIRE(cond, code, ...)            \
   do {                                            \

@@ -272,3 +272,29 @@ def test_trace_hooks_dump_routing_and_output(device, tmp_path, capsys):
     assert torch.equal(dump["output"], out.cpu())
     assert torch.equal(dump["top_k_experts"], idx.cpu()) and torch.equal(dump["expert_gate"], gate.cpu())
     assert torch.equal(load_file(tmp_path / files[1])["default"], out.cpu())
+
+
+@pytest.mark.parametrize("E,k", [(8, 2), (3, 3), (16, 4), (4, 1), (64, 6)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_single_token_forward_equals_staged_calls(device, E, k, dtype):
+    """A forward of one token lets the router launch write the dispatch arrays itself; the result must be the same bits
+    as router, dispatch_build, grouped_ffn and combine called one after the other."""
+    from sharktank_amd import _hip
+    from sharktank_amd.layers import MoeBlock
+    from sharktank_amd.types import unbox_tensor
+
+    case = MC.build(MC.Case(T=1, K=512, N=256, E=E, k=k, fmt="q8_0", dtype=dtype, seed=700 + E))
+    theta = MC.make_theta(case, device)
+    block = MoeBlock(theta, expert_count=E, expert_used_count=k, rms_epsilon=case.eps)
+    wg, wu, wd = block.experts.device_weights()
+    h = case.planes["h"].to(device)
+    fused, idx_f, gate_f = block(h.reshape(1, 1, case.K), return_routing=True)
+
+    xn = _hip.rms_norm(h, unbox_tensor(block.ffn_norm.weight), case.eps)
+    idx, gate, _ = _hip.router_topk(xn, block._router_weight(dtype), k)
+    assert torch.equal(idx.cpu().to(torch.int64), idx_f.cpu().to(torch.int64)) and torch.equal(gate, gate_f)
+    counts, offsets, perm, inv = _hip.dispatch_build(idx, E)
+    assert counts.sum().item() == k and offsets[-1].item() == k
+    y = _hip.grouped_ffn(xn, wg, wu, wd, block.experts._act, offsets, perm, k)
+    staged = _hip.combine(y, gate, inv, 1, k, residual=h)
+    assert torch.equal(staged.view(torch.int16), fused.reshape(1, case.K).view(torch.int16))
