@@ -196,6 +196,16 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
 #pragma unroll
       for (int tj = 0; tj < NTJ; ++tj) acc[ti][tj] = mfma16b<T>(af, bf[tj], acc[ti][tj]);
     }
+    // Issue order of the block above: the token fragments and two weight fragments first, then one weight fragment
+    // read after every fragment's MFMAs, so that each read has the next fragment's MFMAs to land in.  Left alone the
+    // compiler reads the fragments in pairs and waits for each pair right away (same registers either way).
+    __builtin_amdgcn_sched_group_barrier(0x100, NTJ + 2, 0);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, NTJ, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 2 * NTJ, 0);
   };
   __syncthreads();  // first stage filled
   auto k_loop = [&](auto ntj_tag) {
