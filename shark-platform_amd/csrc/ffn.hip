@@ -50,6 +50,10 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 // average (it then walks an expert's rows in passes of 32, re-reading the expert's weights for every pass).
 static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
 static constexpr int64_t kSkinnyMaxAvgRows = 40;
+// A single matrix (no grouping): the streaming kernel re-reads the weights once per 32 rows and still wins up to 80 rows
+// (38 / 45 / 66 us at 48 / 64 / 96 rows of a [14336, 4096] Q8_0 matrix, against 60 / 64 / 64 us for the 256 x 256 kernel
+// and 77 us for the 128 x 128 one); beyond that the 256 x 256 kernel is the fastest at every size.
+static constexpr int64_t kSkinnyMaxRowsSingle = 80;
 // fp8 activations x fp8 weights on the fp8 matrix cores: the 256 x 256 kernel for packed weights and launches with
 // enough rows to fill its tiles (variant 5), the 128 x 128 kernel otherwise (and always with variant 7).
 static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
@@ -63,8 +67,9 @@ static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const 
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
-    else if ((p.offsets || p.E == 1) && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
-                                         max_rows <= kSkinnyMaxAvgRows * p.E)) variant = 3;
+    else if (!p.offsets && p.E == 1) variant = max_rows <= kSkinnyMaxRowsSingle ? 3 : 6;
+    else if (p.offsets && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
+                           max_rows <= kSkinnyMaxAvgRows * p.E)) variant = 3;
     else variant = max_rows >= 256 ? 6 : 2;  // (grouped launches that are not streamed have more than 40 rows per expert)
   }
   if (variant == 6) {
