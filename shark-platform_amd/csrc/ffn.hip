@@ -69,8 +69,13 @@ static int run_projection(int variant, int dtype, int wtag, int mode, const Gemm
     if (dtype == STMOE_F32) variant = 1;
     else if (!p.offsets && p.E == 1) variant = max_rows <= kSkinnyMaxRowsSingle ? 3 : 6;
     else if (p.offsets && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
-                           max_rows <= kSkinnyMaxAvgRows * p.E)) variant = 3;
-    else variant = max_rows >= 256 ? 6 : 2;  // (grouped launches that are not streamed have more than 40 rows per expert)
+                           max_rows <= kSkinnyMaxAvgRows * p.E || (p.E <= 2 && max_rows <= 64 * p.E) ||
+                           (p.E <= 4 && max_rows <= 56 * p.E))) variant = 3;
+    // Everything else goes to the 256 x 256 kernel (which hands shapes it does not take down to the 128 x 128 one).
+    // With few experts a launch can have more than 40 rows per expert and still fewer than 256 rows in all: measured
+    // there (2 / 4 / 6 experts, 100-254 rows, Q8_0 Mixtral shapes) the 128 x 128 kernel took 405-780 us per layer, the
+    // 256 x 256 one 295-440 us, and streaming 185-336 us up to 64 rows per expert with 2 experts or 56 with 4.
+    else variant = 6;
   }
   if (variant == 6) {
     int rc = launch_mfma_ws(dtype, wtag, mode, p, max_rows, p.split_scratch, st);
