@@ -243,6 +243,21 @@ int stmoe_moe_forward_timed(const void* h, int dtype, int64_t T, int64_t K, int6
                             void* workspace, size_t workspace_bytes, int variant, stmoe_stream_t stream,
                             void** events);
 
+/* stmoe_moe_forward without a workspace argument, for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The workspace is a
+ * fixed array of STMOE_STATIC_SCRATCH_BYTES in device memory that belongs to the library (one copy on every GPU the
+ * library runs on, held until the process ends); the call itself allocates nothing.  Shapes whose
+ * stmoe_moe_forward_workspace_bytes() exceeds that size (prefill-sized batches) are refused with STMOE_ERR_WORKSPACE.
+ * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race; serialise them.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress): make it outside graph capture. */
+#define STMOE_STATIC_SCRATCH_BYTES (16u << 20)
+int stmoe_moe_forward_static(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                             const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
+                             const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
+                             const stmoe_weight* w_down, int act, const float* x_scale /*nullable*/,
+                             const float* z_scale /*nullable*/, void* out, int32_t* idx_out, void* gate_out,
+                             int variant, stmoe_stream_t stream);
+
 /* x @ W^T for one quantised (or dense) matrix W [rows, cols]: the operand set of the reference's
  * `mmt_block_scaled_q8(a,d,qs)` (sharktank/sharktank/kernels/mmt_block_scaled_q8.py:30) and
  * `mmt_block_scaled_offset_q4_unsigned(a,d,qs,m)` (mmt_block_scaled_offset_q4.py:31), reached from

@@ -1,4 +1,5 @@
 // C-ABI entry points of the grouped expert FFN, the fused layer forward and the single-matrix mmt.
+#include <atomic>
 #include "ffn_kernels.h"
 
 namespace stmoe {
@@ -375,4 +376,51 @@ extern "C" int stmoe_moe_forward_timed(const void* h, int dtype, int64_t T, int6
                                        size_t workspace_bytes, int variant, stmoe_stream_t stream, void** events) {
   return moe_forward_impl(h, dtype, T, K, N, E, k, ffn_norm_w, out_norm_w, w_dtype, eps, w_router, w_gate, w_up, w_down,
                           act, x_scale, z_scale, out, idx_out, gate_out, workspace, workspace_bytes, variant, stream, events);
+}
+
+// ---- whole layer, workspace inside the library ---------------------------------------------------------
+// For callers that cannot allocate (code under HIP graph capture, tight serving loops): the same forward with its
+// workspace in a fixed array in device memory that belongs to the library, so the call needs no allocation by anyone.
+// Every GPU the library runs on holds its own copy of the array until the process ends.  `scratch` below is the
+// host-side handle of that array, not a device address: the address on the current device comes from
+// hipGetSymbolAddress, is looked up once per device and is what the kernels receive.
+static __device__ __align__(256) unsigned char scratch[STMOE_STATIC_SCRATCH_BYTES];
+
+static constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+static int static_scratch(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return set_error(STMOE_ERR_LAUNCH, "moe_forward_static: no current device");
+  STMOE_REQUIRE(dev >= 0 && dev < kMaxDevices, STMOE_ERR_UNSUPPORTED, "moe_forward_static: device ordinal %d is beyond %d", dev, kMaxDevices - 1);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return set_error(STMOE_ERR_LAUNCH, "moe_forward_static: hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // two threads racing here store the same address
+  }
+  *out = ptr;
+  return STMOE_OK;
+}
+
+extern "C" int stmoe_moe_forward_static(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                                        const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
+                                        const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,
+                                        const stmoe_weight* w_down, int act, const float* x_scale, const float* z_scale,
+                                        void* out, int32_t* idx_out, void* gate_out, int variant, stmoe_stream_t stream) {
+  STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1 && k <= E, STMOE_ERR_SHAPE,
+                "moe_forward_static: T=%lld K=%lld N=%lld E=%d k=%d", (long long)T, (long long)K, (long long)N, E, k);
+  if (T == 0) return STMOE_OK;
+  const size_t need = carve(T, k, E, K, N, dtype).total;
+  STMOE_REQUIRE(need <= (size_t)STMOE_STATIC_SCRATCH_BYTES, STMOE_ERR_WORKSPACE,
+                "moe_forward_static: this shape needs a workspace of %zu bytes, the built-in one holds %zu (use stmoe_moe_forward "
+                "with a caller-owned workspace)", need, (size_t)STMOE_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // Nothing in the workspace has to start at zero: every piece (normalised rows, routing, dispatch arrays, the two
+  // intermediates) is written by one kernel of the forward before another one reads it.
+  return moe_forward_impl(h, dtype, T, K, N, E, k, ffn_norm_w, out_norm_w, w_dtype, eps, w_router, w_gate, w_up, w_down,
+                          act, x_scale, z_scale, out, idx_out, gate_out, ws, (size_t)STMOE_STATIC_SCRATCH_BYTES, variant, stream,
+                          nullptr);
 }

@@ -95,8 +95,12 @@ SIGNATURES = {
     "stmoe_moe_forward_timed": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
                                         POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p, POINTER(c_void_p)]),
+    "stmoe_moe_forward_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
+                                         POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_void_p, c_int, c_void_p]),
     "stmoe_mmt": (c_int, [c_void_p, c_int, c_int64, POINTER(StmoeWeight), c_void_p, c_int, c_void_p]),
 }
+STATIC_SCRATCH_BYTES = 16 << 20  # STMOE_STATIC_SCRATCH_BYTES
 
 _lib = None
 
@@ -520,6 +524,26 @@ def moe_forward(h, ffn_norm_w, out_norm_w, eps: float, w_router, w_gate: DeviceW
             _check(lib.stmoe_moe_forward_timed(*args, events))
     if want_routing:
         return out, idx, gate
+    return out
+
+
+def moe_forward_static(h, ffn_norm_w, out_norm_w, eps: float, w_router, w_gate: DeviceWeight, w_up: DeviceWeight,
+                       w_down: DeviceWeight, act: int, k: int, out: torch.Tensor, *, variant: int = VARIANT_AUTO,
+                       idx: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                       x_scale: Optional[torch.Tensor] = None, z_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """moe_forward on the library's built-in workspace (stmoe_moe_forward_static): every buffer is the caller's (`h` contiguous
+    [T,K], `out` like it, optional `idx` int32 / `gate` [T,k], scales as single fp32 device values), so the call allocates
+    nothing.  Shapes beyond the built-in workspace raise StmoeError (status 6)."""
+    dev = _dev(h, ffn_norm_w, out_norm_w, w_router, out, idx, gate, x_scale, z_scale)
+    lib = load_library()
+    if not h.is_contiguous() or not out.is_contiguous():
+        raise ValueError("moe_forward_static: h and out must be contiguous")
+    T, K = h.shape
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_moe_forward_static(_ptr(h), dtype_enum(h.dtype), T, K, w_gate.rows, w_gate.experts, k, _ptr(ffn_norm_w),
+                                            _ptr(out_norm_w), dtype_enum(ffn_norm_w.dtype), float(eps), _ptr(w_router), w_gate.ref,
+                                            w_up.ref, w_down.ref, act, _ptr(x_scale), _ptr(z_scale), _ptr(out), _ptr(idx), _ptr(gate),
+                                            variant, _stream(dev)))
     return out
 
 
