@@ -381,10 +381,9 @@ def pre_gather_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation
     return out
 
 
-def grouped_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation: Callable = F.silu, x_rscale=None,
-                    z_rscale=None):
-    """Same function, independent formulation: per expert, dense FFN on the rows routed to it (the shape of
-    FFNMOE.forward, ST/layers/ffn_moe_block.py:120-127), then the weighted slot sum."""
+def grouped_ffn_pairs(h, experts, w_gate, w_up, w_down, activation: Callable = F.silu, x_rscale=None, z_rscale=None):
+    """Per (token, slot) pair the expert FFN output before the gate weighting, [T, k, K]: per expert, dense FFN on the
+    rows routed to it (the shape of FFNMOE.forward, ST/layers/ffn_moe_block.py:120-127)."""
     T, K = h.shape
     k = experts.shape[1]
     E = w_gate.shape[0]
@@ -402,6 +401,14 @@ def grouped_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation: C
         if z_rscale is not None:
             z = fake_quant_per_tensor(z, z_rscale)
         down[t_idx, j_idx] = _mm_rt(z, w_down[e])
+    return down
+
+
+def grouped_ffn_moe(h, experts, expert_gate, w_gate, w_up, w_down, activation: Callable = F.silu, x_rscale=None,
+                    z_rscale=None):
+    """PreGatherFFNMOE.forward, independent formulation: per-expert grouped FFN (grouped_ffn_pairs), then the gate
+    weighting and the slot sum (ST/layers/ffn_moe_block.py:73-74)."""
+    down = grouped_ffn_pairs(h, experts, w_gate, w_up, w_down, activation, x_rscale=x_rscale, z_rscale=z_rscale)
     down = expert_gate.unsqueeze(-1) * down
     return torch.sum(down, dim=1)
 

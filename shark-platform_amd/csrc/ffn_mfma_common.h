@@ -40,7 +40,17 @@ struct BigTile {
   int e, row_begin, row_end, ntile;
   int chunk, nchunks;  // this workgroup's part of the reduction (0 of 1 unless the unit is split)
   int chunk_slot;      // index of the fp32 partial tile of a split unit's chunk
+  int tail_begin, tail_rows;  // rows of the expert's absorbed tail that ride along with this full tile (tail_rows 0: none)
 };
+// Absorbed tails.  An expert whose row count is a few rows above a multiple of BM would need a whole partial token tile
+// (its own pass over the weight slab of every feature tile) for those few rows.  A kernel that asks for it (`absorb`)
+// instead lets every full token tile of such an expert take up to kBigTailRows of the tail rows along: full tile s of
+// the expert's c full tiles takes tail rows [16 s, 16 s + 16).  A tail is absorbed when it fits: 0 < tail <= 16 c.
+static constexpr int kBigTailRows = 16;
+__device__ __forceinline__ bool big_tail_absorbed(int rows, int BM, bool absorb) {
+  const int c = rows / BM, t = rows - c * BM;
+  return absorb && t > 0 && t <= kBigTailRows * c;
+}
 // A launch whose units do not fill a whole number of rounds over the 32 CUs of an XCD leaves most CUs idle while the
 // last few units run.  With `allow_split` those last units (the partial token tiles come last) are cut along the
 // reduction into up to 4 chunks (as many as keep units x chunks within the 32 CUs) that run on separate CUs and write
@@ -57,7 +67,8 @@ __device__ __forceinline__ int big_lane_offsets(const GemmParams& p) {
   const int lane = threadIdx.x & 63;
   return (p.offsets && lane <= p.E) ? p.offsets[lane] : 0;
 }
-__device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int lane_off, int BM, int n_tiles, int xcd, bool allow_split) {
+__device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int lane_off, int BM, int n_tiles, int xcd, bool allow_split,
+                                            bool absorb = false) {
   BigPlan pl;
   pl.F = 0;
   pl.R = 0;
@@ -65,11 +76,11 @@ __device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int lane_off, i
     for (int e = 0; e < p.E; ++e) {
       const int rows = __builtin_amdgcn_readlane(lane_off, e + 1) - __builtin_amdgcn_readlane(lane_off, e);
       pl.F += rows / BM;
-      pl.R += (rows % BM) != 0;
+      pl.R += (rows % BM) != 0 && !big_tail_absorbed(rows, BM, absorb);
     }
   } else {
     pl.F = (int)(p.fixed_rows / BM);
-    pl.R = (p.fixed_rows % BM) != 0;
+    pl.R = (p.fixed_rows % BM) != 0 && !big_tail_absorbed((int)p.fixed_rows, BM, absorb);
   }
   const int UF = pl.F * n_tiles, UR = pl.R * n_tiles;
   pl.f0 = (int)((int64_t)UF * xcd / 8);
@@ -105,9 +116,22 @@ __device__ __forceinline__ void big_full_unit(int u, int c, int n_tiles, int& to
   token_tile = v / bn;
   ntile = b * bn0 + v - token_tile * bn;
 }
-__device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int BM, int n_tiles, const BigPlan& pl, int unit, BigTile& t) {
+// Tail rows that full token tile s of an expert (first row b, `rows` rows) takes along.
+__device__ __forceinline__ void big_set_tail(int b, int rows, int BM, int s, bool absorb, BigTile& t) {
+  t.tail_begin = 0;
+  t.tail_rows = 0;
+  if (!big_tail_absorbed(rows, BM, absorb)) return;
+  const int c = rows / BM, first = c * BM + kBigTailRows * s;
+  if (first >= rows) return;
+  t.tail_begin = b + first;
+  t.tail_rows = min(kBigTailRows, rows - first);
+}
+__device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int BM, int n_tiles, const BigPlan& pl, int unit, BigTile& t,
+                                         bool absorb = false) {
   int u;
   bool partial;
+  t.tail_begin = 0;
+  t.tail_rows = 0;
   if (unit < pl.f1 - pl.f0) {
     u = pl.f0 + unit;
     partial = false;
@@ -128,6 +152,7 @@ __device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int 
       big_full_unit(u, pl.F, n_tiles, s, t.ntile);
       t.row_begin = s * BM;
       t.row_end = t.row_begin + BM;
+      big_set_tail(0, (int)p.fixed_rows, BM, s, absorb, t);
     }
     return true;
   }
@@ -141,6 +166,7 @@ __device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int 
         t.e = e;
         t.row_begin = b + s * BM;
         t.row_end = t.row_begin + BM;
+        big_set_tail(b, rows, BM, s, absorb, t);
         return true;
       }
       u -= units;
@@ -151,7 +177,7 @@ __device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int 
   int s = u - t.ntile * pl.R;
   for (int e = 0; e < p.E; ++e) {
     const int b = __builtin_amdgcn_readlane(lane_off, e), rows = __builtin_amdgcn_readlane(lane_off, e + 1) - b;
-    if (rows % BM) {
+    if (rows % BM && !big_tail_absorbed(rows, BM, absorb)) {
       if (s == 0) {
         t.e = e;
         t.row_begin = b + rows / BM * BM;
@@ -163,10 +189,10 @@ __device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int 
   }
   return false;
 }
-__device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_tiles, bool allow_split, BigTile& t) {
+__device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_tiles, bool allow_split, BigTile& t, bool absorb = false) {
   const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
   const int lane_off = big_lane_offsets(p);
-  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, allow_split);
+  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, allow_split, absorb);
   int unit;
   if (j < pl.whole) {
     unit = j;
@@ -181,13 +207,14 @@ __device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_t
     t.nchunks = pl.chunks;
     t.chunk_slot = xcd * kBigChunkSlotsPerXcd + c;
   }
-  return big_unit(p, lane_off, BM, n_tiles, pl, unit, t);
+  return big_unit(p, lane_off, BM, n_tiles, pl, unit, t, absorb);
 }
 // Grid size that covers every XCD's share for at most `slots_bound` token tiles (a split adds up to 24 workgroups).
 static inline int big_grid(int n_tiles, int slots_bound, bool allow_split) {
   return 8 * ((n_tiles * slots_bound + 7) / 8 + 2 + (allow_split ? 24 : 0));
 }
-static inline size_t big_partial_bytes(int BN, int BM) { return (size_t)8 * kBigChunkSlotsPerXcd * BN * BM * sizeof(float); }
+// fp32 partial tiles of the split units: BM rows plus the rows of an absorbed tail
+static inline size_t big_partial_bytes(int BN, int BM) { return (size_t)8 * kBigChunkSlotsPerXcd * BN * (BM + kBigTailRows) * sizeof(float); }
 
 // ---- LDS reservation --------------------------------------------------------------------------------------
 // Kernels that use more than 64 KB of dynamic LDS must be told so once per device.  `done` is a per-kernel bit mask of
@@ -211,6 +238,19 @@ __device__ __forceinline__ void vm_load16_to_lds(const void* base, uint32_t byte
                : "memory", "m0");
 }
 template <int N> __device__ __forceinline__ void vm_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// Loads into registers from a wave-uniform base (scalar registers) plus a 32-bit lane offset, issued by hand: the compiler
+// places no wait for the result, so nothing may read it before a vm_wait that covers the load, followed by vm_landed on
+// the same variable (an empty statement that makes every later use of the variable come after it in program order).
+__device__ __forceinline__ void vm_load16_to_regs(u32x4_t& dst, const void* base, uint32_t byte_off) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(dst) : "v"(byte_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void vm_load8_to_regs(uint2& dst, const void* base, uint32_t byte_off) {
+  asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(dst) : "v"(byte_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void vm_load_u16_to_reg(uint32_t& dst, const void* base, uint32_t byte_off) {
+  asm volatile("global_load_ushort %0, %1, %2" : "=&v"(dst) : "v"(byte_off), "s"(base) : "memory");
+}
+template <typename V> __device__ __forceinline__ void vm_landed(V& v) { asm volatile("" : "+v"(v)::"memory"); }
 
 // ---- packed weight pieces -----------------------------------------------------------------------------
 // Per K step (64 reduction elements) and row tile (16 rows), lane (n = lane % 16, g = lane / 16) fetches the samples
@@ -241,11 +281,14 @@ template <typename T> __device__ __forceinline__ void f16x16_to_T(uint32_t v[8])
 
 // Q8_0: 1 KB piece = 16 rows x 64 k; scales d_p[rt][K/256][16][8]
 template <> struct BigAddr<WF_Q8_0_P> {
-  const uint8_t* q;
-  const uint16_t* d;
+  const uint8_t* q;  // the row tile's pieces (the same for every lane, so it lives in scalar registers)
+  const uint8_t* d;
+  uint32_t lq, ld;   // the lane's byte offsets inside a piece / inside the scales of 256 reduction elements
   __device__ __forceinline__ void init(const WeightView& w, int64_t rt, int64_t, int lane, int64_t kred) {
-    q = w.qs + (rt * (kred >> 6) * 64 + lane) * 16;
-    d = reinterpret_cast<const uint16_t*>(w.d) + (rt * (kred >> 8) * 16 + (lane & 15)) * 8 + (lane >> 5);
+    q = w.qs + rt * (kred >> 6) * 1024;
+    d = w.d + rt * (kred >> 8) * 256;
+    lq = (uint32_t)lane * 16;
+    ld = (uint32_t)(((lane & 15) * 8 + (lane >> 5)) * 2);
   }
 };
 template <> struct BigPiece<WF_Q8_0_P> {
@@ -253,8 +296,16 @@ template <> struct BigPiece<WF_Q8_0_P> {
   u32x4_t q;
   uint32_t d;  // fp16 bits, zero-extended
   __device__ __forceinline__ void load(const BigAddr<WF_Q8_0_P>& a, int64_t kt) {
-    q = *reinterpret_cast<const u32x4_t*>(a.q + kt * 1024);
-    d = a.d[(kt >> 2) * 128 + (kt & 3) * 2];
+    q = *reinterpret_cast<const u32x4_t*>(a.q + kt * 1024 + a.lq);
+    d = *reinterpret_cast<const uint16_t*>(a.d + ((kt >> 2) * 256 + (kt & 3) * 4) + a.ld);
+  }
+  __device__ __forceinline__ void load_async(const BigAddr<WF_Q8_0_P>& a, int64_t kt) {
+    vm_load16_to_regs(q, a.q + kt * 1024, a.lq);
+    vm_load_u16_to_reg(d, a.d + ((kt >> 2) * 256 + (kt & 3) * 4), a.ld);
+  }
+  __device__ __forceinline__ void landed() {
+    vm_landed(q);
+    vm_landed(d);
   }
   template <typename T> __device__ __forceinline__ void convert(const BigAddr<WF_Q8_0_P>&, uint32_t out[8]) const {
     q8x16_to_f16(q, d, out);
@@ -265,9 +316,11 @@ template <> struct BigPiece<WF_Q8_0_P> {
 // fp8 e4m3fn with one fp32 scale per tensor or per expert: pieces as Q8_0, T(f32(q) * d)
 template <> struct BigAddr<WF_FP8_F32D_P> {
   const uint8_t* q;
+  uint32_t lq;
   float dv;
   __device__ __forceinline__ void init(const WeightView& w, int64_t rt, int64_t e, int lane, int64_t kred) {
-    q = w.qs + (rt * (kred >> 6) * 64 + lane) * 16;
+    q = w.qs + rt * (kred >> 6) * 1024;
+    lq = (uint32_t)lane * 16;
     dv = reinterpret_cast<const float*>(w.d)[w.d_count > 1 ? e : 0];
   }
 };
@@ -275,8 +328,10 @@ template <> struct BigPiece<WF_FP8_F32D_P> {
   static constexpr int LOADS = 1;
   u32x4_t q;
   __device__ __forceinline__ void load(const BigAddr<WF_FP8_F32D_P>& a, int64_t kt) {
-    q = *reinterpret_cast<const u32x4_t*>(a.q + kt * 1024);
+    q = *reinterpret_cast<const u32x4_t*>(a.q + kt * 1024 + a.lq);
   }
+  __device__ __forceinline__ void load_async(const BigAddr<WF_FP8_F32D_P>& a, int64_t kt) { vm_load16_to_regs(q, a.q + kt * 1024, a.lq); }
+  __device__ __forceinline__ void landed() { vm_landed(q); }
   template <typename T> __device__ __forceinline__ void convert(const BigAddr<WF_FP8_F32D_P>& a, uint32_t out[8]) const {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -292,14 +347,16 @@ template <> struct BigPiece<WF_FP8_F32D_P> {
 // takes half of it: the lane's 16 samples are 8 bytes of block 2*(kt % 2) + g/2, half g % 2
 template <> struct BigAddr<WF_Q4_1_P> {
   const uint8_t* q;
-  const uint16_t* d;
-  const uint16_t* m;
+  const uint8_t* d;
+  const uint8_t* m;
+  uint32_t lq, ld;
   __device__ __forceinline__ void init(const WeightView& w, int64_t rt, int64_t, int lane, int64_t kred) {
     const int n = lane & 15, g = lane >> 4;
-    q = w.qs + rt * (kred >> 7) * 1024 + (((g >> 1) * 16 + n) * 16 + (g & 1) * 8);
-    const int64_t s = (rt * (kred >> 8) * 16 + n) * 8 + (g >> 1);
-    d = reinterpret_cast<const uint16_t*>(w.d) + s;
-    m = reinterpret_cast<const uint16_t*>(w.m) + s;
+    q = w.qs + rt * (kred >> 7) * 1024;
+    lq = (uint32_t)((((g >> 1) * 16 + n) * 16 + (g & 1) * 8));
+    d = w.d + rt * (kred >> 8) * 256;
+    m = w.m + rt * (kred >> 8) * 256;
+    ld = (uint32_t)((n * 8 + (g >> 1)) * 2);
   }
 };
 template <> struct BigPiece<WF_Q4_1_P> {
@@ -307,10 +364,21 @@ template <> struct BigPiece<WF_Q4_1_P> {
   uint2 q;
   uint32_t d, m;
   __device__ __forceinline__ void load(const BigAddr<WF_Q4_1_P>& a, int64_t kt) {
-    q = *reinterpret_cast<const uint2*>(a.q + (kt >> 1) * 1024 + (kt & 1) * 512);
-    const int64_t s = (kt >> 2) * 128 + (kt & 3) * 2;
-    d = a.d[s];
-    m = a.m[s];
+    q = *reinterpret_cast<const uint2*>(a.q + ((kt >> 1) * 1024 + (kt & 1) * 512) + a.lq);
+    const int64_t s = (kt >> 2) * 256 + (kt & 3) * 4;
+    d = *reinterpret_cast<const uint16_t*>(a.d + s + a.ld);
+    m = *reinterpret_cast<const uint16_t*>(a.m + s + a.ld);
+  }
+  __device__ __forceinline__ void load_async(const BigAddr<WF_Q4_1_P>& a, int64_t kt) {
+    vm_load8_to_regs(q, a.q + ((kt >> 1) * 1024 + (kt & 1) * 512), a.lq);
+    const int64_t s = (kt >> 2) * 256 + (kt & 3) * 4;
+    vm_load_u16_to_reg(d, a.d + s, a.ld);
+    vm_load_u16_to_reg(m, a.m + s, a.ld);
+  }
+  __device__ __forceinline__ void landed() {
+    vm_landed(q);
+    vm_landed(d);
+    vm_landed(m);
   }
   template <typename T> __device__ __forceinline__ void convert(const BigAddr<WF_Q4_1_P>&, uint32_t out[8]) const {
     const Q4Scale sc = q4_scale(d, m);

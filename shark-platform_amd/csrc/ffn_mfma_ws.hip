@@ -10,8 +10,14 @@
 //             one barrier per K step
 //   registers: 12 wavefronts leave 168 per lane; the consumers hold 128 accumulators and 20 operand registers
 //
-// The direct loads are inline assembly and are awaited by hand (see ffn_mfma_common.h); per K step a producer
-// issues XLOADS token loads followed by WLOADS weight loads, always in this order.
+//   tails:    a full token tile may take up to 16 more rows of its expert along (an absorbed tail, see big_tail_absorbed):
+//             the four producers multiply those rows themselves, each against 64 of the tile's 256 weight rows, with the
+//             weight operands taken from the registers they have just converted and the token operands straight from
+//             global memory (two K steps ahead, two register sets); 8 MFMAs per producer and K step, no LDS traffic
+//
+// All loads of the producers are inline assembly with a wave-uniform base in scalar registers and are awaited by hand
+// (see ffn_mfma_common.h); per K step a producer issues the tail's token loads (if any), then XLOADS token loads, then
+// WLOADS weight loads, always in this order and always all of them.
 #include "ffn_mfma_common.h"
 
 namespace stmoe {
@@ -27,11 +33,12 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   constexpr int XLOADS = 8;    // direct token loads per producer per K step (32 blocks of 8 rows / 4 producers)
   constexpr int WLOADS = BigPiece<WF>::LOADS * WPIECES;
   extern __shared__ __align__(16) uint16_t lds[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for all lanes: everything derived from it can live in scalar registers
   const int g = lane >> 4, n_in = lane & 15;
 
   BigTile tile;
-  if (!big_tile_id(p, BM, n_tiles, partial != nullptr, tile)) return;
+  if (!big_tile_id(p, BM, n_tiles, partial != nullptr, tile, true)) return;
   const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
   // Rows per token-row group: the rows of a partial tile are spread evenly (in multiples of 16) over the four groups,
@@ -39,8 +46,8 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   // grp * rpg + i (i < rpg) lives in LDS row grp * 64 + i.  Full tiles: rpg = 64, the identity.
   const int rpg = min(64, ((rows_here + 3) / 4 + 15) / 16 * 16);
   // this workgroup's K steps: all of them, or one chunk of a split unit
-  const int64_t kt0 = (p.kred >> 6) * tile.chunk / tile.nchunks;
-  const int64_t nkt = (p.kred >> 6) * (tile.chunk + 1) / tile.nchunks - kt0;
+  const int kt0 = (int)((p.kred >> 6) * tile.chunk / tile.nchunks);
+  const int nkt = (int)((p.kred >> 6) * (tile.chunk + 1) / tile.nchunks) - kt0;
 
   uint16_t* const Wbase = lds;               // [2][BN][64]
   uint16_t* const Xbase = lds + 2 * WSTAGE;  // [3][BM][64]
@@ -49,19 +56,20 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   if (wave >= 8) {
     // =================================== producer ===================================
     const int pw = wave - 8;
+    // This producer's four 16-row weight blocks, as rows of the workgroup tile: GATEUP: gate blocks 2 pw, 2 pw + 1 and the up
+    // blocks of the same features (so that an absorbed tail's gate and up sums meet in one lane); DOWN: blocks 4 pw .. 4 pw + 3
+    auto piece_row = [&](int j) { return MODE == MODE_GATEUP ? (j < 2 ? 0 : BN / 2) + (2 * pw + (j & 1)) * 16 : (4 * pw + j) * 16; };
     BigAddr<WF> waddr[WPIECES];
 #pragma unroll
     for (int j = 0; j < WPIECES; ++j) {
-      const int rtl = pw * WPIECES + j;  // row tile (16 rows) inside the workgroup tile
       int64_t row0;
       const WeightView* wv;
       if (MODE == MODE_GATEUP) {
-        const bool up = rtl >= BN / 32;
-        wv = up ? &p.w1 : &p.w0;
-        row0 = (int64_t)e * wv->rows + (int64_t)ntile * (BN / 2) + (rtl % (BN / 32)) * 16;
+        wv = j >= 2 ? &p.w1 : &p.w0;
+        row0 = (int64_t)e * wv->rows + (int64_t)ntile * (BN / 2) + (2 * pw + (j & 1)) * 16;
       } else {
         wv = &p.w0;
-        row0 = (int64_t)e * wv->rows + (int64_t)ntile * BN + rtl * 16;
+        row0 = (int64_t)e * wv->rows + (int64_t)ntile * BN + piece_row(j);
       }
       waddr[j].init(*wv, row0 >> 4, e, lane, p.kred);
     }
@@ -78,84 +86,160 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     }
     const uint32_t lds_addr0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)lds);
     const uint32_t x_lds0 = __builtin_amdgcn_readfirstlane(lds_addr0 + (2 * WSTAGE + pw * 8 * BIG_LS) * 2);
-    uint16_t* const w_st = Wbase + (pw * WPIECES * 16 + n_in) * BIG_LS;
+    uint16_t* const w_st = Wbase + n_in * BIG_LS;
     const int st_swz0 = ((2 * g) ^ sw) << 3, st_swz1 = ((2 * g + 1) ^ sw) << 3;
 
+    // Absorbed tail.  A converted piece sits in the lane's registers as row n_in of the block, reduction elements
+    // 16 g .. 16 g + 15 of the K step: exactly a weight operand of two MFMAs whose K index is permuted (lane group g
+    // supplies elements 16 g .. 16 g + 7 to the first and 16 g + 8 .. 16 g + 15 to the second).  A dot product does not care
+    // about the order of its terms as long as both operands agree, so lane (n_in, g) fetches the same 16 elements of token row
+    // tail_begin + n_in (rows past the end re-read the last one; never stored) straight from global memory and the tail
+    // costs neither LDS traffic nor extra operand registers: 8 MFMAs per producer and K step.
+    uint32_t toff = 0;
+    if (tile.tail_rows > 0) {
+      const int i = tile.tail_begin + min(n_in, tile.tail_rows - 1);
+      const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
+      toff = (uint32_t)((src * p.lda + g * 16) * 2);
+    }
+    u32x4_t tx[2][2];  // [register set = K step % 2][half of the lane's 16 elements]
+    floatx4_t tacc[WPIECES];
+#pragma unroll
+    for (int j = 0; j < WPIECES; ++j) tacc[j] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+
     BigPiece<WF> wreg[3][WPIECES];  // three register sets: weights are loaded three K steps before their conversion
-    auto load_w = [&](auto set_tag, int64_t kt) {
+    auto load_w = [&](auto set_tag, int kt) {
       constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
-      for (int j = 0; j < WPIECES; ++j) {
-        wreg[SET][j].load(waddr[j], kt0 + kt);
-      }
+      for (int j = 0; j < WPIECES; ++j) wreg[SET][j].load_async(waddr[j], kt0 + kt);
     };
-    auto store_w = [&](auto set_tag, auto stage_tag) {
-      constexpr int SET = decltype(set_tag)::value, STAGE = decltype(stage_tag)::value;
+    // Converts register set SET (the weights of a K step s) into weight stage STAGE; with TAIL the tail's MFMAs of step s
+    // follow each piece's conversion (token operands: register set s % 2 = TXSET).
+    auto store_w = [&](auto set_tag, auto stage_tag, auto tail_tag, auto txset_tag) {
+      constexpr int SET = decltype(set_tag)::value, STAGE = decltype(stage_tag)::value, TXSET = decltype(txset_tag)::value;
+      constexpr bool TAIL = decltype(tail_tag)::value != 0;
+      if constexpr (TAIL) {
+        vm_landed(tx[TXSET][0]);
+        vm_landed(tx[TXSET][1]);
+      }
 #pragma unroll
       for (int j = 0; j < WPIECES; ++j) {
         uint32_t v[8];
+        wreg[SET][j].landed();  // awaited by the previous step's vm_wait (or the prologue's)
         wreg[SET][j].template convert<T>(waddr[j], v);
-        uint16_t* row = w_st + STAGE * WSTAGE + j * 16 * BIG_LS;
-        *reinterpret_cast<u32x4_t*>(row + st_swz0) = (u32x4_t){v[0], v[1], v[2], v[3]};
-        *reinterpret_cast<u32x4_t*>(row + st_swz1) = (u32x4_t){v[4], v[5], v[6], v[7]};
+        uint16_t* row = w_st + STAGE * WSTAGE + piece_row(j) * BIG_LS;
+        const u32x4_t lo = (u32x4_t){v[0], v[1], v[2], v[3]}, hi = (u32x4_t){v[4], v[5], v[6], v[7]};
+        *reinterpret_cast<u32x4_t*>(row + st_swz0) = lo;
+        *reinterpret_cast<u32x4_t*>(row + st_swz1) = hi;
+        if constexpr (TAIL) {
+          tacc[j] = mfma16b<T>(lo, tx[TXSET][0], tacc[j]);
+          tacc[j] = mfma16b<T>(hi, tx[TXSET][1], tacc[j]);
+        }
       }
     };
-    auto load_x = [&](auto xstage_tag, int64_t kt) {
+    auto load_x = [&](auto xstage_tag, int kt) {
       constexpr int XS = decltype(xstage_tag)::value;
+      const char* xsrc = reinterpret_cast<const char*>(p.a) + (kt0 + kt) * (BIG_BK * 2);  // the step's columns: a scalar add
 #pragma unroll
       for (int j = 0; j < XLOADS; ++j)
-        vm_load16_to_lds(p.a, xoff[j] + (uint32_t)(kt0 + kt) * (BIG_BK * 2), x_lds0 + (uint32_t)((XS * XSTAGE + 32 * j * BIG_LS) * 2));
+        vm_load16_to_lds(xsrc, xoff[j], x_lds0 + (uint32_t)((XS * XSTAGE + 32 * j * BIG_LS) * 2));
     };
-    // K step kt (R = kt % 6 fixes every stage and register set at compile time): store the weights of step kt + 1
-    // (register set (kt+1) % 3, loaded during step kt - 3) into weight stage (kt+1) % 2, issue the token loads of step
-    // kt + 2 into token stage (kt+2) % 3 and the weight loads of step kt + 4 into the register set just freed.  Before
-    // the barrier the token loads of step kt + 1 must have landed: they were issued during step kt - 1, followed by
-    // that step's weight loads and this step's token and weight loads.  STEADY steps (kt + 4 < nkt) have no branch.
-    auto k_step = [&](auto r_tag, auto steady_tag, int64_t kt) {
+    auto load_tx = [&](auto set_tag, int kt) {
+      constexpr int SET = decltype(set_tag)::value;
+      const char* src = reinterpret_cast<const char*>(p.a) + (kt0 + kt) * (BIG_BK * 2);
+      vm_load16_to_regs(tx[SET][0], src, toff);
+      vm_load16_to_regs(tx[SET][1], src + 16, toff);
+    };
+    // K step kt (R = kt % 6 fixes every stage and register set at compile time): convert the weights of step kt + 1
+    // (register set (kt+1) % 3, loaded during step kt - 3) into weight stage (kt+1) % 2 (TAIL: and multiply them with the
+    // tail's token operands of step kt + 1, then request those of step kt + 3 into the set just freed), issue the token
+    // loads of step kt + 2 into token stage (kt+2) % 3 and the weight loads of step kt + 4 into the register set just
+    // freed.  Before the barrier the token loads of step kt + 1 must have landed, and before the next step's conversion the
+    // weights of step kt + 2 and the tail operands of step kt + 2: all were issued before the 2 WLOADS + XLOADS (+ TLOADS)
+    // youngest loads (the weight loads of steps kt + 3 and kt + 4, the token loads of step kt + 2, the tail operands of
+    // step kt + 3).
+    // Every step issues every load: requests past the last step read the last step again (cache hits, results unused), so
+    // the number of loads in flight is the same at every wait and the steps of a unit are one straight sequence without
+    // joins.  That matters because the loads into registers are invisible to the compiler: a register copy or a spill that
+    // it placed where two paths with different register assignments meet would move a register whose load has not landed.
+    const int last = nkt - 1;
+    auto k_step = [&](auto r_tag, auto tail_tag, int kt) {
       constexpr int R = decltype(r_tag)::value;
-      constexpr bool STEADY = decltype(steady_tag)::value;
+      constexpr bool TAIL = decltype(tail_tag)::value != 0;
+      constexpr int TLOADS = TAIL ? 2 : 0;
       using Set = WsInt<(R + 1) % 3>;
-      if (STEADY || kt + 1 < nkt) store_w(Set{}, WsInt<(R + 1) % 2>{});
-      if (STEADY || kt + 2 < nkt) load_x(WsInt<(R + 2) % 3>{}, kt + 2);
-      if (STEADY || kt + 4 < nkt) load_w(Set{}, kt + 4);
-      if constexpr (STEADY) vm_wait<2 * WLOADS + XLOADS>();
-      else vm_wait<0>();
+      using TxSet = WsInt<(R + 1) % 2>;
+      if (kt < last) store_w(Set{}, WsInt<(R + 1) % 2>{}, tail_tag, TxSet{});
+      if constexpr (TAIL) load_tx(TxSet{}, min(kt + 3, last));
+      load_x(WsInt<(R + 2) % 3>{}, min(kt + 2, last));
+      load_w(Set{}, min(kt + 4, last));
+      vm_wait<2 * WLOADS + XLOADS + TLOADS>();
       __syncthreads();
     };
-    load_w(WsInt<0>{}, 0);
-    load_x(WsInt<0>{}, 0);
-    if (nkt > 1) {
-      load_w(WsInt<1>{}, 1);
-      load_x(WsInt<1>{}, 1);
+    auto run = [&](auto tail_tag) {
+      constexpr bool TAIL = decltype(tail_tag)::value != 0;
+      constexpr int TLOADS = TAIL ? 2 : 0;
+      if constexpr (TAIL) {
+        load_tx(WsInt<0>{}, 0);
+        load_tx(WsInt<1>{}, min(1, last));
+      }
+      load_w(WsInt<0>{}, 0);
+      load_w(WsInt<1>{}, min(1, last));
+      load_x(WsInt<0>{}, 0);
+      load_w(WsInt<2>{}, min(2, last));
+      load_x(WsInt<1>{}, min(1, last));
+      // the weights of step 0 (and the tail operands of steps 0, 1) are older than everything else issued so far
+      vm_wait<2 * WLOADS + 2 * XLOADS>();
+      store_w(WsInt<0>{}, WsInt<0>{}, tail_tag, WsInt<0>{});
+      if constexpr (TAIL) load_tx(WsInt<0>{}, min(2, last));
+      load_w(WsInt<0>{}, min(3, last));
+      // step 0 reads the weights stored above and the token rows of step 0, and converts the weights of step 1 (TAIL: with
+      // the tail operands of step 1): younger than all of these are the weight loads of steps 2 and 3, the token loads of
+      // step 1 and the tail operands of step 2
+      vm_wait<2 * WLOADS + XLOADS + TLOADS>();
+      __syncthreads();
+      for (int kt = 0;; kt += 6) {
+        k_step(WsInt<0>{}, tail_tag, kt);
+        if (kt + 1 >= nkt) break;
+        k_step(WsInt<1>{}, tail_tag, kt + 1);
+        if (kt + 2 >= nkt) break;
+        k_step(WsInt<2>{}, tail_tag, kt + 2);
+        if (kt + 3 >= nkt) break;
+        k_step(WsInt<3>{}, tail_tag, kt + 3);
+        if (kt + 4 >= nkt) break;
+        k_step(WsInt<4>{}, tail_tag, kt + 4);
+        if (kt + 5 >= nkt) break;
+        k_step(WsInt<5>{}, tail_tag, kt + 5);
+        if (kt + 6 >= nkt) break;
+      }
+      vm_wait<0>();  // the requests past the last step: nothing may land in registers or LDS after this wavefront is done
+    };
+    if (tile.tail_rows == 0) {
+      run(WsInt<0>{});
+      return;
     }
-    if (nkt > 2) load_w(WsInt<2>{}, 2);
-    store_w(WsInt<0>{}, WsInt<0>{});
-    if (nkt > 3) {
-      load_w(WsInt<0>{}, 3);
-      // step 0 needs the weights (stored above) and the token rows of step 0 only: issued after those token loads are
-      // the weight loads of steps 1, 2, 3 and the token loads of step 1, which may stay in flight
-      vm_wait<3 * WLOADS + XLOADS>();
-    } else {
-      vm_wait<0>();
-    }
-    __syncthreads();
-    int64_t kt = 0;
-    for (; kt + 9 < nkt; kt += 6) {
-      k_step(WsInt<0>{}, WsInt<1>{}, kt);
-      k_step(WsInt<1>{}, WsInt<1>{}, kt + 1);
-      k_step(WsInt<2>{}, WsInt<1>{}, kt + 2);
-      k_step(WsInt<3>{}, WsInt<1>{}, kt + 3);
-      k_step(WsInt<4>{}, WsInt<1>{}, kt + 4);
-      k_step(WsInt<5>{}, WsInt<1>{}, kt + 5);
-    }
-    for (int r = 0; kt < nkt; ++kt, ++r) {  // kt % 6 == r here: the steady loop advances in sixes
-      switch (r % 6) {
-        case 0: k_step(WsInt<0>{}, WsInt<0>{}, kt); break;
-        case 1: k_step(WsInt<1>{}, WsInt<0>{}, kt); break;
-        case 2: k_step(WsInt<2>{}, WsInt<0>{}, kt); break;
-        case 3: k_step(WsInt<3>{}, WsInt<0>{}, kt); break;
-        case 4: k_step(WsInt<4>{}, WsInt<0>{}, kt); break;
-        default: k_step(WsInt<5>{}, WsInt<0>{}, kt); break;
+    run(WsInt<1>{});
+    // ---- the tail's results: lane (n_in, g) holds, for token row tail_begin + n_in, features 4 g .. 4 g + 3 of each block
+    if (n_in < tile.tail_rows) {
+      if (tile.nchunks > 1) {
+        float* pt = partial + (size_t)tile.chunk_slot * (BN * (BM + kBigTailRows)) + (BM + n_in) * BN;
+#pragma unroll
+        for (int bi = 0; bi < 4; ++bi) *reinterpret_cast<floatx4_t*>(pt + piece_row(bi) + 4 * g) = tacc[bi];
+      } else if (MODE == MODE_GATEUP) {
+        T* orow = reinterpret_cast<T*>(p.out) + out_row(p, tile.tail_begin + n_in) * p.ldo + (int64_t)ntile * (BN / 2) + 4 * g;
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi) {
+          const float gq[4] = {tacc[bi][0], tacc[bi][1], tacc[bi][2], tacc[bi][3]};
+          const float uq[4] = {tacc[bi + 2][0], tacc[bi + 2][1], tacc[bi + 2][2], tacc[bi + 2][3]};
+          uint2* dst = reinterpret_cast<uint2*>(orow + (2 * pw + bi) * 16);
+          if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq);
+          else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq);
+        }
+      } else {
+        T* orow = reinterpret_cast<T*>(p.out) + out_row(p, tile.tail_begin + n_in) * p.ldo + (int64_t)ntile * BN + 4 * g;
+#pragma unroll
+        for (int bi = 0; bi < 4; ++bi)
+          *reinterpret_cast<uint2*>(orow + (4 * pw + bi) * 16) =
+              make_uint2(pack2<T>(tacc[bi][0], tacc[bi][1]), pack2<T>(tacc[bi][2], tacc[bi][3]));
       }
     }
     return;
@@ -210,7 +294,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   __syncthreads();  // first stage filled
   auto k_loop = [&](auto ntj_tag) {
     int xs = 0;
-    for (int64_t kt = 0; kt < nkt; kt += 2) {
+    for (int kt = 0; kt < nkt; kt += 2) {
       compute(WsInt<0>{}, ntj_tag, xs, 0);
       compute(WsInt<0>{}, ntj_tag, xs, 1);
       __syncthreads();
@@ -224,7 +308,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     }
   };
   if (!active) {
-    for (int64_t kt = 0; kt < nkt; ++kt) __syncthreads();
+    for (int kt = 0; kt < nkt; ++kt) __syncthreads();
   } else if (ntj == 1) {
     k_loop(WsInt<1>{});
   } else if (ntj == 2) {
@@ -252,7 +336,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
   };
   if (tile.nchunks > 1) {
     // chunk of a split unit: fp32 partial tile [BM][BN], added to the other chunks by big_reduce_kernel
-    float* pt = partial + (size_t)tile.chunk_slot * (BN * BM);
+    float* pt = partial + (size_t)tile.chunk_slot * (BN * (BM + kBigTailRows));
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
       const int r = wm * rpg + tj * 16 + n_in;
@@ -290,20 +374,24 @@ __global__ void __launch_bounds__(256) big_reduce_kernel(GemmParams p, int n_til
   constexpr int BN = 256, BM = 256;
   const int xcd = blockIdx.x >> 4, su = blockIdx.x & 15;
   const int lane_off = big_lane_offsets(p);
-  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, true);
+  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, true, true);
   if (su >= pl.rest) return;
   BigTile t;
-  if (!big_unit(p, lane_off, BM, n_tiles, pl, pl.whole + su, t)) return;
+  if (!big_unit(p, lane_off, BM, n_tiles, pl, pl.whole + su, t, true)) return;
   const int rows_here = t.row_end - t.row_begin;
-  const int r = blockIdx.y * 32 + (threadIdx.x >> 3);
-  if (r >= rows_here) return;
-  const float* base = partial + (size_t)(xcd * kBigChunkSlotsPerXcd + su * pl.chunks) * (BN * BM) + r * BN;
+  const int r = blockIdx.y * 32 + (threadIdx.x >> 3);  // row of the partial tile: tile rows, then the absorbed tail's rows from BM on
+  int sorted_row;
+  if (r < rows_here) sorted_row = t.row_begin + r;
+  else if (r >= BM && r - BM < t.tail_rows) sorted_row = t.tail_begin + (r - BM);
+  else return;
+  constexpr size_t kSlot = (size_t)BN * (BM + kBigTailRows);
+  const float* base = partial + (size_t)(xcd * kBigChunkSlotsPerXcd + su * pl.chunks) * kSlot + r * BN;
   auto total = [&](int col) {
     floatx4_t sum = *reinterpret_cast<const floatx4_t*>(base + col);
-    for (int c = 1; c < pl.chunks; ++c) sum = sum + *reinterpret_cast<const floatx4_t*>(base + (size_t)c * (BN * BM) + col);
+    for (int c = 1; c < pl.chunks; ++c) sum = sum + *reinterpret_cast<const floatx4_t*>(base + (size_t)c * kSlot + col);
     return sum;
   };
-  T* orow = reinterpret_cast<T*>(p.out) + out_row(p, t.row_begin + r) * p.ldo;
+  T* orow = reinterpret_cast<T*>(p.out) + out_row(p, sorted_row) * p.ldo;
   if (MODE == MODE_GATEUP) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -337,7 +425,7 @@ static int launch_ws_m(const GemmParams& p, int64_t max_rows, float* partial, hi
   kern<<<dim3((unsigned)big_grid(n_tiles, m_slots, partial != nullptr)), 768, lds_bytes, st>>>(p, n_tiles, partial);
   int rc = check_launch("grouped_mfma_ws");
   if (rc || !partial) return rc;
-  big_reduce_kernel<T, MODE><<<dim3(8 * 16, BM / 32), 256, 0, st>>>(p, n_tiles, partial);
+  big_reduce_kernel<T, MODE><<<dim3(8 * 16, (BM + kBigTailRows + 31) / 32), 256, 0, st>>>(p, n_tiles, partial);
   return check_launch("big_reduce");
 }
 

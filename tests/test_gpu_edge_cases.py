@@ -182,6 +182,71 @@ def test_streaming_kernel_two_row_tiles_in_one_pass(device, fmt, dtype):
     assert O.rel_l2(got, want) < (1e-3 if dtype == torch.float16 else 8e-3)
 
 
+def _routing_with_rows(rows, T, k, seed):
+    """idx [T,k] (no expert twice in a token) that gives expert e exactly rows[e] pairs; sum(rows) == T*k."""
+    assert sum(rows) == T * k and max(rows) <= T
+    g = torch.Generator().manual_seed(seed)
+    left = list(rows)
+    idx = torch.empty(T, k, dtype=torch.long)
+    for t in range(T):
+        # the k experts with the most pairs left (ties in random order): greedy, always feasible while max(left) <= tokens left
+        order = sorted(range(len(left)), key=lambda e: (-left[e], torch.rand(1, generator=g).item()))
+        pick = order[:k]
+        assert all(left[e] > 0 for e in pick)
+        for j, e in enumerate(pick):
+            left[e] -= 1
+        idx[t] = torch.tensor([pick[i] for i in torch.randperm(k, generator=g).tolist()])
+    assert not any(left)
+    return idx[torch.randperm(T, generator=g)]
+
+
+@pytest.mark.parametrize("fmt,dtype", [("q8_0", torch.float16), ("q4_1", torch.bfloat16), ("fp8", torch.float16)])
+@pytest.mark.parametrize("rows", [
+    [261, 517, 512 + 32, 512 + 33, 256 + 16, 256 + 17, 300, 122],  # absorbed: 5, 5, 32 (two tiles x 16), 16; not: 33, 17
+    [768 + 48, 768 + 1, 256, 255, 1, 0, 270, 257],                  # three full tiles x 16; one-row tails; an expert without rows
+])
+def test_prefill_tails_that_ride_along_with_full_token_tiles(device, fmt, dtype, rows):
+    """Row counts a few rows above a multiple of 256: the prefill kernel lets every full token tile of such an expert take up
+    to 16 of the extra rows along (computed by its loader wavefronts) instead of running a partial token tile for them.
+    Every output row is checked against the oracle, the tail rows also on their own, and the whole result against the
+    vector-ALU kernel."""
+    from sharktank_amd import _hip as hip
+    from sharktank_amd.ops import device_weight
+
+    E, k = len(rows), 2
+    T = sum(rows) // k
+    assert sum(rows) == T * k
+    case = MC.build(MC.Case(T=T, K=512, N=768, E=E, k=k, fmt=fmt, dtype=dtype, seed=4100 + rows[0]))
+    idx = _routing_with_rows(rows, T, k, seed=rows[1])
+    assert torch.bincount(idx.reshape(-1), minlength=E).tolist() == rows
+    x = case.planes["h"]
+    wg, wu, wd = MC.dense_weights(case)
+    ones = torch.ones(T, k, dtype=dtype)
+    N, K = case.N, case.K
+    dws = [device_weight(MC.to_inference_tensor(fmt, case.planes[n], shp, n, device), stacked=True, prepack=True)
+           for n, shp in (("gate", [E, N, K]), ("up", [E, N, K]), ("down", [E, K, N]))]
+    _, offsets, perm, inv = hip.dispatch_build(idx.to(torch.int32).to(device), E)
+    tol = 1e-3 if dtype == torch.float16 else 8e-3
+    y = {}
+    for variant in (hip.VARIANT_MFMA_WS, hip.VARIANT_GENERIC):
+        y[variant] = hip.grouped_ffn(x.to(device), dws[0], dws[1], dws[2], hip.ACT_SILU, offsets, perm, k, variant=variant).cpu()
+    got = y[hip.VARIANT_MFMA_WS]
+    assert O.rel_l2(got.float(), y[hip.VARIANT_GENERIC].float()) < (2e-3 if dtype == torch.float16 else 1.2e-2)
+    # oracle per sorted row: row i belongs to pair perm[i] = t*k + j of expert idx[t, j]
+    perm_c, off_c = perm.cpu().long(), offsets.cpu().long()
+    pair_rows = O.grouped_ffn_pairs(x, idx, wg, wu, wd, case.activation)  # [T, k, K]
+    want = pair_rows.reshape(T * k, K)[perm_c]
+    assert O.rel_l2(got, want) < tol
+    for e in range(E):
+        r = rows[e]
+        c, t = r // 256, r % 256
+        if c >= 1 and 0 < t <= 16 * c:  # an absorbed tail: its rows on their own
+            a, b = int(off_c[e]) + c * 256, int(off_c[e + 1])
+            err = O.rel_l2(got[a:b], want[a:b])
+            assert err < 2 * tol, f"expert {e}: tail rows {a}..{b}: rel-L2 {err:.3e}"
+            assert torch.isfinite(got[a:b].float()).all()
+
+
 def test_random_shapes_automatic_choice_against_vector_alu_kernel(device):
     """Seeded random shapes, formats, routings and activations: the automatically chosen kernels against the vector-ALU
     kernel (an independent implementation of the same arithmetic)."""
