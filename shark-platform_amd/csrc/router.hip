@@ -133,9 +133,12 @@ router_topk_kernel(const T* __restrict__ x, const T* __restrict__ wr, int64_t T_
 #pragma unroll
   for (int e = 0; e < EP; ++e)
     if (e < E) denom += expf(lg[e] - mx);
-
-  // top-k by (logit descending, expert index ascending).  exp is monotone, so this is the order of the
-  // probabilities with ties resolved toward the lower index.
+  // The reference ranks the fp32 probabilities (F.softmax, then torch.topk): so does this kernel, with equal
+  // probabilities ordered by increasing expert index.  Distinct logits whose probabilities round to the same fp32 number
+  // (logits one ulp apart next to the maximum, say) therefore count as a tie, as they do for the reference.
+  float pr[EP];
+#pragma unroll
+  for (int e = 0; e < EP; ++e) pr[e] = (e < E) ? expf(lg[e] - mx) / denom : 0.0f;
   uint64_t taken = 0;
   float vsum = 0.0f;
   float pv[EP];  // selected probabilities in slot order (only the first k are used)
@@ -147,16 +150,15 @@ router_topk_kernel(const T* __restrict__ x, const T* __restrict__ wr, int64_t T_
       float bestv = 0.0f;
 #pragma unroll
       for (int e = 0; e < EP; ++e) {
-        if (e < E && !((taken >> e) & 1ull) && (best < 0 || lg[e] > bestv)) {
+        if (e < E && !((taken >> e) & 1ull) && (best < 0 || pr[e] > bestv)) {
           best = e;
-          bestv = lg[e];
+          bestv = pr[e];
         }
       }
       taken |= 1ull << best;
-      const float p = expf(bestv - mx) / denom;
-      pv[j] = p;
+      pv[j] = bestv;
       pi[j] = best;
-      vsum += p;
+      vsum += bestv;
     }
   }
   if (lane == 0) {
@@ -314,12 +316,13 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
   __syncthreads();
   if (tid != 0) return;
 
-  // fp32 softmax, top-k by (logit descending, index ascending), renormalised gates: same arithmetic and order
-  // as router_topk_kernel.
+  // fp32 softmax, top-k of the probabilities (equal ones by increasing index), renormalised gates: same arithmetic and
+  // order as router_topk_kernel.  The probabilities replace the logits in lg_s.
   float mx = lg_s[0];
   for (int e = 1; e < E; ++e) mx = fmaxf(mx, lg_s[e]);
   float denom = 0.0f;
   for (int e = 0; e < E; ++e) denom += expf(lg_s[e] - mx);
+  for (int e = 0; e < E; ++e) lg_s[e] = expf(lg_s[e] - mx) / denom;
   uint64_t taken = 0;
   float vsum = 0.0f;
   for (int j = 0; j < k; ++j) {
@@ -333,11 +336,10 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
       }
     }
     taken |= 1ull << best;
-    const float p = expf(bestv - mx) / denom;
     idx_out[t * k + j] = best;
     if (idx64_out) idx64_out[t * k + j] = best;
-    part[8 + j] = p;  // part has 64 + 8 floats of room after the partial sums
-    vsum += p;
+    part[8 + j] = bestv;  // part has 64 + 8 floats of room after the partial sums
+    vsum += bestv;
   }
   for (int j = 0; j < k; ++j) gate_out[t * k + j] = Cvt<T>::from_f32(part[8 + j] / vsum);
 

@@ -13,6 +13,12 @@ import moe_cases as MC
 pytestmark = pytest.mark.gpu
 
 TOL = {torch.float32: 1e-5, torch.float16: 1e-3, torch.bfloat16: 1e-3}
+# Limits on the MoE contribution y - h alone (the residual h ~ N(0, 1) is as large as the contribution and would hide an
+# FFN error in a check of y).  fp32 and fp16: the north-star figures.  bf16 keeps 8 significant bits and the gated
+# intermediate, the down projection and the weighted slot values are each rounded to it: two formulations of the oracle
+# itself that differ only in the order of the fp32 sums are 8e-3 apart (tests/test_oracle_golden.py), and that is the
+# figure the kernels are held to.
+MOE_TOL = {torch.float32: 1e-4, torch.float16: 1e-3, torch.bfloat16: 8e-3}
 
 
 def run_block(case, device, variant=0):
@@ -26,18 +32,41 @@ def run_block(case, device, variant=0):
     return y.reshape(case.T, case.K).cpu(), idx.cpu(), gate.cpu()
 
 
-def check_case(case, device, variant=0, tol=None):
+def check_case(case, device, variant=0, tol=None, moe_tol=None):
+    """Routing bit-exact; the layer output y within `tol`; the MoE contribution y - h on its own within `moe_tol`."""
     case = MC.build(case)
     y, idx, gate = run_block(case, device, variant)
     want_y, want_idx, want_gate = MC.oracle_block(case)
     assert torch.equal(idx.long(), want_idx), "routing indices differ"
-    # the residual h dominates y; compare the MoE contribution itself
     h = case.planes["h"]
     err = O.rel_l2(y.float() - h.float(), want_y.float() - h.float())
     err_y = O.rel_l2(y, want_y)
     tol = tol or TOL[case.dtype]
+    moe_tol = moe_tol or MOE_TOL[case.dtype]
     assert err_y < tol, f"layer output rel-L2 {err_y:.3e}"
+    assert err < moe_tol, f"MoE contribution rel-L2 {err:.3e} (limit {moe_tol:.0e})"
     return err, err_y
+
+
+def exact_block(case):
+    """The layer with the oracle's routing and the same quantised operands, every product and sum in float64 and no
+    rounding of intermediates to the activation dtype: what both the reference's arithmetic and the kernels approximate."""
+    case = MC.build(case)
+    wg, wu, wd = (w.double() for w in MC.dense_weights(case))
+    h = case.planes["h"]
+    x = O.rms_norm_ordered(h, case.planes["ffn_norm"], case.eps)
+    idx, gate, _ = O.route(O.router_logits_ordered(x, case.planes["router"]), case.k)
+    xs, zs = case.planes["x_rscale"], case.planes["z_rscale"]
+    xq = (O.fake_quant_per_tensor(x, xs) if xs is not None else x).double()
+    out = torch.zeros(case.T, case.K, dtype=torch.float64)
+    for t in range(case.T):
+        for j in range(case.k):
+            e = int(idx[t, j])
+            z = case.activation(wg[e] @ xq[t]) * (wu[e] @ xq[t])
+            if zs is not None:
+                z = O.fake_quant_per_tensor(z.float(), zs).double()
+            out[t] += gate[t, j].double() * (wd[e] @ z)
+    return out
 
 
 def test_toy_fp32_config(device):
@@ -77,15 +106,26 @@ def test_fp8_weights_and_fp8_activations(device, dtype, T):
 @pytest.mark.parametrize("T", [40, 200, 700])
 def test_fp8_matrix_core_layer(device, dtype, T):
     """The same layers with both operands on the fp8 matrix cores (kernel variant 5): the dot product of the quantised
-    samples is scaled once, skipping the rounding of the dequantised samples to the activation dtype (2^-11 relative
-    for fp16, 2^-8 for bf16, on both operands), so the MoE contribution alone differs from the dequantise-first
-    arithmetic by about 1e-2 (fp16) and 4e-2 (bf16); the layer output is held to the 2e-2 tolerance of the fp8
-    configuration."""
+    samples is scaled once, skipping the reference's rounding of the dequantised samples to the activation dtype (2^-11
+    relative for fp16, 2^-8 for bf16, on both operands).  With fp16 activations the MoE contribution stays within the fp8
+    tolerance of 2e-2 of the reference's arithmetic.  With bf16 activations the two arithmetics are up to 6e-2 apart,
+    and neither is the better one: the gated intermediate is quantised to e4m3 (3 mantissa bits), so a value that the
+    two compute slightly differently lands in a different bucket now and then.  Measured against a float64 evaluation of
+    the same quantised operands both are about 4e-2 off; the kernel must be no further off than the oracle (within 5 %)."""
     from sharktank_amd import _hip
 
     case = MC.Case(T=T, K=512, N=768, fmt="fp8", dtype=dtype, act_quant=True, seed=40 + T)
-    err, err_y = check_case(case, device, variant=_hip.VARIANT_FP8_MFMA, tol=2e-2)
-    assert err < (2e-2 if dtype == torch.float16 else 6e-2), f"MoE contribution rel-L2 {err:.3e}"
+    err, err_y = check_case(case, device, variant=_hip.VARIANT_FP8_MFMA, tol=2e-2, moe_tol=2e-2 if dtype == torch.float16 else 6e-2)
+    if dtype == torch.bfloat16:
+        case = MC.build(case)
+        y, _, _ = run_block(case, device, _hip.VARIANT_FP8_MFMA)
+        want_y, _, _ = MC.oracle_block(case)
+        exact = exact_block(MC.Case(T=T, K=512, N=768, fmt="fp8", dtype=dtype, act_quant=True, seed=40 + T))
+        h = case.planes["h"].double()
+        kernel_vs_exact = O.rel_l2(y.double() - h, exact)
+        oracle_vs_exact = O.rel_l2(want_y.double() - h, exact)
+        print(f"  MoE contribution against float64: kernel {kernel_vs_exact:.2e}, oracle {oracle_vs_exact:.2e}")
+        assert kernel_vs_exact <= oracle_vs_exact * 1.05 + 2e-3
 
 
 @pytest.mark.parametrize("variant_name,down_packed", [("VARIANT_FP8_MFMA", False), ("VARIANT_FP8_MFMA", True), ("VARIANT_FP8_TILE", True)])

@@ -140,6 +140,34 @@ def test_router_ties_lower_index_first(device):
     assert torch.equal(idx.cpu()[pos].long(), torch.tensor([[0, 2, 4]]).expand(int(pos.sum()), 3))
 
 
+@pytest.mark.parametrize("K", [64, 16384])  # one workgroup per token / one wavefront per token (long rows)
+def test_router_distinct_logits_with_equal_probabilities(device, K):
+    """The reference ranks the fp32 softmax probabilities, not the logits (mixture_of_experts_block.py:75-78).  Two fp32
+    logits one ulp apart, 2^-10 and the next number up, have the same probability: exp(-2^-33) rounds to 1.  For the
+    reference that is a tie, which the contract resolves toward the lower expert index, although the higher index holds
+    the larger logit.  The input row is a unit vector, so logit e is exactly the router's entry [e, 0]."""
+    E, k = 8, 2
+    a = torch.tensor(2.0 ** -10, dtype=torch.float32)
+    b = torch.nextafter(a, torch.tensor(1.0))
+    assert b > a and torch.exp(a - b) == 1.0
+    x = torch.zeros(4, K, dtype=torch.float32)
+    x[:, 0] = 1.0
+    wr = torch.full((E, K), 0.0, dtype=torch.float32)
+    wr[:, 0] = -1.0
+    wr[3, 0], wr[5, 0] = a, b  # expert 5 has the larger logit, expert 3 the lower index
+    wr[6, 0] = a - 0.25
+    idx, gate, logits = _hip().router_topk(x.to(device), wr.to(device), k, want_logits=True)
+    assert torch.equal(logits.cpu()[0], wr[:, 0]), "logits are not the router's first column"
+    want_idx, want_gate, probs = O.route(O.router_logits_ordered(x, wr), k)
+    assert probs[0, 3] == probs[0, 5]
+    assert want_idx[0].tolist() == [3, 5]
+    assert torch.equal(idx.cpu().long(), want_idx)
+    assert torch.equal(gate.cpu(), torch.full((4, 2), 0.5))
+    # a third slot takes the next probability down
+    idx3, _, _ = _hip().router_topk(x.to(device), wr.to(device), 3, want_logits=True)
+    assert idx3.cpu()[0].tolist() == [3, 5, 6]
+
+
 @pytest.mark.parametrize("T,k,E", [(1, 2, 8), (32, 2, 8), (2048, 2, 8), (3000, 4, 64), (7, 1, 1)])
 def test_dispatch_bit_exact(device, T, k, E):
     g = torch.Generator().manual_seed(8)
