@@ -15,6 +15,12 @@
  *   - the caller owns all memory, including the workspace; the library
  *     allocates nothing, never synchronises and only enqueues on `stream`
  *     (a hipStream_t passed as void*; NULL is the default stream);
+ *   - host-side state is limited to a thread-local error string, one flag per
+ *     device and kernel that records that the kernel's LDS reservation has been
+ *     raised (hipFuncSetAttribute, on the kernel's first launch on that device:
+ *     run every shape once eagerly before capturing launches into a HIP graph),
+ *     and the per-device address of the built-in workspace of
+ *     stmoe_moe_forward_static;
  *   - the return value is a stmoe_status; stmoe_last_error() returns a
  *     thread-local, human-readable description of the last non-zero status.
  */
@@ -59,7 +65,12 @@ typedef enum {
   STMOE_W_DENSE = 0, /* DefaultPrimitiveTensor: qs = elements of `dtype` */
   STMOE_W_Q8_0 = 1,  /* BlockScaledLayout, block 32: d fp16 [.,K/32], qs int8 [.,K/32,32] */
   STMOE_W_Q4_1 = 2,  /* BlockScaledI4Layout, block 32, unsigned: d,m fp16 [.,K/32], qs u8 [.,K/32,16] */
-                     /* (the matrix-multiply kernels on the packed form assume block scales |d| < 64) */
+                     /* (the matrix-multiply kernels on the PACKED form need finite block scales with |d| < 64:
+                      * they remove the nibbles' exponent bias with one fused multiply-add whose constant term is
+                      * 1024 * d in fp16.  Larger scales give NaN there without an error; the planar form and the
+                      * dequant entry points have no such limit.  The Python binding checks the scale plane once
+                      * before it prepacks a tensor and keeps tensors beyond the limit planar; a C caller that
+                      * cannot rule such scales out does the same.) */
   STMOE_W_FP8 = 3,   /* TensorScaledLayout: qs e4m3fn [.,K], d = d_count scales of `dtype` (f32 or f16) */
   /* The same bytes re-ordered by stmoe_prepack() into the order the matrix-core kernels stream (every wavefront
    * load is one contiguous kilobyte; see stmoe_prepack).  Plane sizes are unchanged. */
@@ -159,7 +170,8 @@ int stmoe_rms_norm(const void* x, int dtype, const void* w, int w_dtype, int64_t
                    void* out, stmoe_stream_t stream);
 
 /* Router of MoeBlock.forward (mixture_of_experts_block.py:70-83): logits = x @ Wr^T rounded to `dtype`,
- * fp32 softmax over E, top-k (descending; equal logits -> lower expert index first), gates renormalised
+ * fp32 softmax over E, top-k of the fp32 probabilities (descending; equal probabilities -> lower expert index first,
+ * also where distinct logits round to one probability), gates renormalised
  * in fp32 then rounded to `dtype`.  Wr [E,K] is given in `dtype`.  K % 8 == 0, E <= 64, k <= E.
  * logits_out ([T,E], `dtype`) and idx64_out ([T,k], int64) may be NULL. */
 int stmoe_router_topk(const void* x, const void* w_router, int dtype, int64_t T, int64_t K, int E, int k,
@@ -169,7 +181,10 @@ int stmoe_router_topk(const void* x, const void* w_router, int dtype, int64_t T,
 /* Token-to-expert dispatch: a stable counting sort of the n_pairs = T*k (token, slot) pairs
  * p = t*k + j by expert id.  counts[E]; offsets[E+1] = exclusive scan; perm[offsets[e]+r] = the r-th
  * pair of expert e in increasing p; inv[perm[i]] = i.  The reference has no such step (it gathers
- * weights per token instead, ffn_moe_block.py:37-41); this is what replaces it. */
+ * weights per token instead, ffn_moe_block.py:37-41); this is what replaces it.
+ * Expert ids outside 0..E-1 are clamped into the range, not reported (the reference's weights[experts] would raise
+ * IndexError): a caller that cannot trust its ids checks them first; the Python layer does when
+ * TURBINE_LLM_DEBUG=enable_nan_checks is set. */
 int stmoe_dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets,
                          int32_t* perm, int32_t* inv, stmoe_stream_t stream);
 

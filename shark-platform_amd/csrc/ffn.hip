@@ -47,8 +47,14 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 //          4 MFMA 256x256 tile (prefill; packed Q8_0), 5 fp8 matrix cores (fp8 weights and quantised activations),
 //          6 MFMA 256x256 tile with specialised producer/consumer wavefronts (prefill; packed formats),
 //          7 fp8 matrix cores, 128x128 tile kernel only (5 uses the 256x256 LDS-direct kernel where it applies)
-// The streaming kernel is chosen when no expert can get more than 32 rows, or when experts get 40 rows or fewer on
-// average (it then walks an expert's rows in passes of 32, re-reading the expert's weights for every pass).
+// Automatic choice of a grouped launch (the host knows the row total and the token count, not the rows per expert):
+// the streaming kernel when no expert can get more than 32 rows (token count <= 32), or when experts get 40 rows or
+// fewer on average (56 with at most 4 experts, 64 with at most 2); everything else goes to the specialised-wavefront
+// prefill kernel.  The streaming kernel walks an expert's rows in passes of 32 and re-reads the expert's weights for every
+// pass, so inside its window a routing that puts all T tokens on a few experts costs those experts ceil(T / 32) passes
+// instead of one or two: at most (experts + rows / 32) weight passes in all against (experts) for a uniform routing,
+// i.e. up to 2.2 x the uniform time at 8 experts and 320 rows; the prefill kernel at those sizes is as fast as the uniform
+// case, so the window ends where the two meet for uniform routing.
 static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
 static constexpr int64_t kSkinnyMaxAvgRows = 40;
 // A single matrix (no grouping): the streaming kernel re-reads the weights once per 32 rows and still wins up to 80 rows

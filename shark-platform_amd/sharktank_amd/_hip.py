@@ -345,6 +345,9 @@ def dispatch_build(idx: torch.Tensor, E: int):
     return counts, offsets, perm, inv
 
 
+Q4_1_PACKED_MAX_SCALE = 64.0
+
+
 class DeviceWeight:
     """An expert-stacked weight `[E, rows, cols]` as the C ABI sees it; keeps its planes alive."""
 
@@ -371,7 +374,18 @@ class DeviceWeight:
 
     def can_prepack(self) -> bool:
         return (self.format in _PACKED_OF and self.rows % 16 == 0 and self.cols % 256 == 0
-                and (self.format != W_FP8 or self.desc.dtype == F32))
+                and (self.format != W_FP8 or self.desc.dtype == F32) and self.q4_scales_in_range())
+
+    def q4_scales_in_range(self) -> bool:
+        """The kernels that read Q4_1 weights in the streaming order fold the removal of their exponent bias into one fused
+        multiply-add, which needs 1024 * |d| to stay finite in fp16: every block scale must be finite and below 64 in
+        magnitude (block scales of real weights are orders of magnitude smaller).  A tensor that breaks the limit keeps the
+        planar order, whose kernels have no such limit.  Checked once per tensor, at load time (one small reduction and a
+        host read)."""
+        if self.format not in (W_Q4_1, W_Q4_1_PACKED):
+            return True
+        d = self.keep[1]
+        return bool(torch.isfinite(d).all()) and float(d.abs().max()) < Q4_1_PACKED_MAX_SCALE
 
     def prepack(self) -> "DeviceWeight":
         """The same weight in the streaming order of stmoe_prepack (new planes; this object is unchanged)."""
@@ -402,9 +416,11 @@ class DeviceWeight:
 GGUF_Q8_0, GGUF_Q4_1 = 0, 1
 
 
-def gguf_ingest(raw: torch.Tensor, gguf_type: int, experts: int, rows: int, cols: int, *, packed: bool) -> DeviceWeight:
+def gguf_ingest(raw: torch.Tensor, gguf_type: int, experts: int, rows: int, cols: int, *, packed: bool,
+                check_scales: bool = True) -> DeviceWeight:
     """Raw ggml blocks (uint8, on the device) -> a DeviceWeight with freshly allocated planes, planar (the reference's
-    planes bit for bit) or in the streaming order of stmoe_prepack."""
+    planes bit for bit) or in the streaming order of stmoe_prepack.  With `check_scales` a Q4_1 tensor whose block scales
+    the packed kernels cannot take (DeviceWeight.q4_scales_in_range) comes back planar even when `packed` is asked for."""
     dev = _dev(raw)
     lib = load_library()
     raw_c = _contig(raw)
@@ -422,6 +438,8 @@ def gguf_ingest(raw: torch.Tensor, gguf_type: int, experts: int, rows: int, cols
     out = DeviceWeight(_PACKED_OF[fmt] if packed else fmt, experts, rows, cols, qs, d, m)
     with torch.cuda.device(dev):
         _check(lib.stmoe_gguf_ingest(_ptr(raw_c), gguf_type, out.ref, _stream(dev)))
+    if packed and check_scales and not out.q4_scales_in_range():
+        return gguf_ingest(raw, gguf_type, experts, rows, cols, packed=False)  # see DeviceWeight.q4_scales_in_range
     return out
 
 

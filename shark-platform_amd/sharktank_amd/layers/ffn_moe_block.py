@@ -14,6 +14,7 @@ import torch.nn.functional as F
 from .. import _hip
 from .. import ops
 from ..ops import device_weight, gather_experts
+from ..utils import debugging
 from ..types import DefaultPrimitiveTensor, PlanarQuantizedTensor, QuantizedTensor, StaticScaledQuantizer, Theta
 from .base import ThetaLayer
 from .linear import LinearLayer
@@ -91,9 +92,23 @@ class PreGatherFFNMOE(ThetaLayer):
     def expert_count(self) -> int:
         return int(self.ffn_gate.shape[0])
 
+    def bigger_mmg(self, inputs, weights, experts):
+        """The reference keeps this alternative to the gather (one matmul against all experts, then a gather of the
+        results; ffn_moe_block.py:43-51) for experiments and never calls it from forward; it has no kernel here."""
+        raise NotImplementedError("PreGatherFFNMOE.bigger_mmg: unused by forward in the reference; not built")
+
+    def one_hot_matmul(self, inputs, weights, experts):
+        """As bigger_mmg with a one-hot selection (ffn_moe_block.py:53-58): unused by the reference's forward; not built."""
+        raise NotImplementedError("PreGatherFFNMOE.one_hot_matmul: unused by forward in the reference; not built")
+
     def forward(self, h: torch.Tensor, experts: torch.Tensor, expert_gate: torch.Tensor):
         wg, wu, wd = self.device_weights()
         T, k = experts.shape
+        if debugging.flags.enable_nan_checks:
+            # The dispatch kernel clamps expert ids into range instead of faulting; the reference's weights[experts] would
+            # raise IndexError.  With the checks switched on (TURBINE_LLM_DEBUG=enable_nan_checks) so does this (one host read).
+            if bool(((experts < 0) | (experts >= wg.experts)).any()):
+                raise IndexError(f"PreGatherFFNMOE: expert index outside 0..{wg.experts - 1}")
         _, offsets, perm, inv = _hip.dispatch_build(experts, wg.experts)
         xs, zs = self.activation_scales()
         y = _hip.grouped_ffn(h, wg, wu, wd, self._act, offsets, perm, k, variant=self.kernel_variant, x_scale=xs, z_scale=zs)

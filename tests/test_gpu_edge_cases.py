@@ -247,6 +247,88 @@ def test_prefill_tails_that_ride_along_with_full_token_tiles(device, fmt, dtype,
             assert torch.isfinite(got[a:b].float()).all()
 
 
+@pytest.mark.parametrize("E", [2, 4, 6])
+@pytest.mark.parametrize("T", [50, 96, 127])
+@pytest.mark.parametrize("routing", ["uniform", "two experts take everything"])
+def test_few_experts_between_100_and_255_rows(device, E, T, routing):
+    """Launches of 100-254 sorted rows with 2-6 experts sit between the streaming kernel (up to 56-64 rows per expert on
+    average) and the prefill kernel, whichever the automatic choice picks from the row total; with all tokens on two
+    experts each of those holds T rows, several passes of the streaming kernel or one partial token tile.  Checked
+    against the oracle pair by pair."""
+    from sharktank_amd import _hip as hip
+    from sharktank_amd.ops import device_weight
+
+    k = 2
+    case = MC.build(MC.Case(T=T, K=512, N=768, E=E, k=k, fmt="q8_0", dtype=torch.float16, seed=900 + E + T))
+    g = torch.Generator().manual_seed(E * 1000 + T)
+    if routing == "uniform":
+        idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    else:
+        idx = torch.tensor([[0, 1], [1, 0]])[torch.randint(0, 2, (T,), generator=g)]
+    x = case.planes["h"]
+    wg, wu, wd = MC.dense_weights(case)
+    N, K = case.N, case.K
+    dws = [device_weight(MC.to_inference_tensor("q8_0", case.planes[n], shp, n, device), stacked=True, prepack=True)
+           for n, shp in (("gate", [E, N, K]), ("up", [E, N, K]), ("down", [E, K, N]))]
+    _, offsets, perm, inv = hip.dispatch_build(idx.to(torch.int32).to(device), E)
+    got = hip.grouped_ffn(x.to(device), dws[0], dws[1], dws[2], hip.ACT_SILU, offsets, perm, k).cpu()
+    want = O.grouped_ffn_pairs(x, idx, wg, wu, wd, case.activation).reshape(T * k, K)[perm.cpu().long()]
+    assert torch.isfinite(got.float()).all()
+    assert O.rel_l2(got, want) < 1e-3
+
+
+def test_q4_1_block_scale_beyond_the_packed_limit_stays_planar(device):
+    """The kernels on packed Q4_1 weights need |d| < 64 (they would give NaN beyond, without an error).  A tensor with one
+    block scale of 100 must keep the planar order when asked to prepack, and the product through ops.matmul must match the
+    oracle; the same tensor with ordinary scales is packed."""
+    from sharktank_amd import _hip as hip
+    from sharktank_amd.ops import device_weight
+
+    g = torch.Generator().manual_seed(77)
+    N, K = 64, 512
+    d, m, qs = O.quantize_q4_1(torch.randn(N, K, generator=g) * 0.02)
+    shape = [N, K]
+    ok = device_weight(MC.to_inference_tensor("q4_1", {"d": d, "m": m, "qs": qs}, shape, "w", device), stacked=False, prepack=True)
+    assert ok.is_packed
+    d_big = d.clone()
+    d_big[3, 5] = 100.0
+    planes = {"d": d_big, "m": m, "qs": qs}
+    dw = device_weight(MC.to_inference_tensor("q4_1", planes, shape, "w", device), stacked=False, prepack=True)
+    assert not dw.is_packed, "a block scale of 100 must keep the tensor off the packed kernels"
+    x = (torch.randn(40, K, generator=g) * 0.1).to(torch.float16)
+    got = hip.mmt(x.to(device), dw).cpu()
+    want = O.mmt(x, MC.dense_from_planes("q4_1", planes, shape, torch.float16))
+    assert torch.isfinite(got.float()).all()
+    assert O.rel_l2(got, want) < 1e-3
+    # raw ggml blocks take the same decision
+    raw = torch.cat([d_big.reshape(-1, 1).view(torch.uint8), m.reshape(-1, 1).view(torch.uint8), qs.reshape(-1, 16)], dim=1).contiguous()
+    ing = hip.gguf_ingest(raw.reshape(-1).to(device), hip.GGUF_Q4_1, 1, N, K, packed=True)
+    assert not ing.is_packed
+
+
+def test_expert_ids_out_of_range_raise_with_checks_on(device):
+    """The dispatch kernel clamps ids into range; with the debug checks on, PreGatherFFNMOE.forward raises IndexError as
+    the reference's weights[experts] would."""
+    from sharktank_amd.layers import PreGatherFFNMOE
+    from sharktank_amd.utils import debugging
+
+    case = MC.build(MC.Case(T=8, K=256, N=256, E=4, k=2, fmt="q8_0", dtype=torch.float16, seed=5))
+    ffn = PreGatherFFNMOE(MC.make_theta(case, device))
+    x = case.planes["h"].to(device)
+    experts = torch.tensor([[0, 1]] * 7 + [[2, 4]], dtype=torch.int32, device=device)
+    gate = torch.full((8, 2), 0.5, dtype=torch.float16, device=device)
+    old = debugging.flags.enable_nan_checks
+    try:
+        debugging.flags.enable_nan_checks = True
+        with pytest.raises(IndexError):
+            ffn(x, experts, gate)
+        debugging.flags.enable_nan_checks = False
+        y = ffn(x, experts, gate)  # clamped: finite output, no fault
+        assert torch.isfinite(y.float()).all()
+    finally:
+        debugging.flags.enable_nan_checks = old
+
+
 def test_random_shapes_automatic_choice_against_vector_alu_kernel(device):
     """Seeded random shapes, formats, routings and activations: the automatically chosen kernels against the vector-ALU
     kernel (an independent implementation of the same arithmetic)."""

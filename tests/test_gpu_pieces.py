@@ -416,7 +416,8 @@ def test_gguf_raw_blocks_to_planes(device, fmt, shape):
     assert torch.equal(d.cpu().view(torch.int16), want_d.contiguous().view(torch.int16))
     assert torch.equal(qs.cpu().view(torch.uint8), want_qs.contiguous().view(torch.uint8))
     if rows % 16 == 0 and cols % 256 == 0:
-        direct = H.gguf_ingest(raw.to(device), gt, E, rows, cols, packed=True)
+        # random bit patterns as block scales: the byte permutation is what is tested, not the scale limit of the kernels
+        direct = H.gguf_ingest(raw.to(device), gt, E, rows, cols, packed=True, check_scales=False)
         via = planar.prepack()
         for a, b in zip(direct.keep, via.keep):
             assert (a is None) == (b is None)

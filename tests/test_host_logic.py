@@ -113,3 +113,36 @@ def test_unknown_activation_is_rejected():
 
     with pytest.raises(NotImplementedError):
         activation_enum(torch.tanh)
+
+
+def _tiny_theta(**extra):
+    E, N, K = 2, 32, 64
+    tensors = {
+        "ffn_gate_inp.weight": ST.DefaultPrimitiveTensor(name="ffn_gate_inp.weight", data=torch.zeros(E, K)),
+        "ffn_norm.weight": ST.DefaultPrimitiveTensor(name="ffn_norm.weight", data=torch.ones(K)),
+        "ffn_gate_exps.weight": ST.DefaultPrimitiveTensor(name="ffn_gate_exps.weight", data=torch.zeros(E, N, K)),
+        "ffn_up_exps.weight": ST.DefaultPrimitiveTensor(name="ffn_up_exps.weight", data=torch.zeros(E, N, K)),
+        "ffn_down_exps.weight": ST.DefaultPrimitiveTensor(name="ffn_down_exps.weight", data=torch.zeros(E, K, N)),
+    }
+    tensors.update(extra)
+    return ST.Theta(tensors)
+
+
+def test_router_with_bias_is_refused():
+    """The fused forward reads the router matrix only; a bias that a LinearLayer would add must not vanish silently."""
+    from sharktank_amd.layers import MoeBlock
+
+    MoeBlock(_tiny_theta(), 2, 1, 1e-5)  # a plain router builds
+    bias = ST.DefaultPrimitiveTensor(name="ffn_gate_inp.bias", data=torch.zeros(2))
+    with pytest.raises(NotImplementedError, match="ffn_gate_inp"):
+        MoeBlock(_tiny_theta(**{"ffn_gate_inp.bias": bias}), 2, 1, 1e-5)
+
+
+def test_unused_reference_alternatives_are_named():
+    """PreGatherFFNMOE.bigger_mmg / one_hot_matmul exist in the reference and are never called by its forward."""
+    from sharktank_amd.layers import PreGatherFFNMOE
+
+    ffn = PreGatherFFNMOE(_tiny_theta())
+    for fn in (ffn.bigger_mmg, ffn.one_hot_matmul):
+        with pytest.raises(NotImplementedError, match="unused by forward"):
+            fn(None, None, None)
