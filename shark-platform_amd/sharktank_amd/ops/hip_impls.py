@@ -38,6 +38,47 @@ def device_weight(w, *, stacked: bool, prepack: bool = False) -> _hip.DeviceWeig
     return dw
 
 
+def _planes_key(w):
+    """What a cached descriptor of `w` depends on: the identity, shape and version of every plane."""
+    if isinstance(w, torch.Tensor):
+        ts = (w,)
+    elif isinstance(w, (Q8_0, Q4_1)):
+        ts = (w.raw,)
+    else:
+        ts = tuple(w.globals.values())
+    return tuple((t.data_ptr(), tuple(t.shape), t.dtype, t._version) for t in ts)
+
+
+_TENSOR_CACHE = {}  # id(torch.Tensor) -> (weakref to it, {(stacked, prepack, dtype): (planes key, descriptor)})
+
+
+def cached_device_weight(w, *, stacked: bool, prepack: bool = True, cast_to: torch.dtype = None) -> _hip.DeviceWeight:
+    """device_weight(w) built once per weight and kept with it: the planes are made contiguous and (where the shape allows)
+    re-ordered into the kernels' streaming order on the first call; later calls with unchanged planes reuse the result.
+    InferenceTensors carry their descriptors themselves; plain torch tensors are tracked through weak references.  `cast_to`
+    (dense weights only) is the dtype the kernels need, cast once as well."""
+    if isinstance(w, torch.Tensor):
+        ent = _TENSOR_CACHE.get(id(w))
+        if ent is None or ent[0]() is not w:
+            import weakref
+
+            wid = id(w)
+            ent = (weakref.ref(w, lambda _, wid=wid: _TENSOR_CACHE.pop(wid, None)), {})
+            _TENSOR_CACHE[wid] = ent
+        store = ent[1]
+    else:
+        store = w.__dict__.setdefault("_stmoe_descriptors", {})
+    slot, key = (stacked, prepack, cast_to), _planes_key(w)
+    hit = store.get(slot)
+    if hit is None or hit[0] != key:
+        src = w
+        if cast_to is not None and not isinstance(w, QuantizedTensor):
+            src = unbox_tensor(w).to(cast_to)
+        hit = (key, device_weight(src, stacked=stacked, prepack=prepack))
+        store[slot] = hit
+    return hit[1]
+
+
 def _device_weight_planar(w, *, stacked: bool) -> _hip.DeviceWeight:
     shape = list(w.shape)
     if stacked:
@@ -124,16 +165,18 @@ def matmul_tensor_quantized(lhs, rhs: QuantizedTensor, *, transpose_rhs: bool):
     lhs = unbox_tensor(lhs)
     if not transpose_rhs or len(rhs.shape) != 2 or lhs.dtype not in _FLOAT_DTYPES:
         return NotImplemented
-    return _mmt_2d(lhs, device_weight(rhs, stacked=False))
+    # the descriptor (contiguous planes, streaming order) is built on the first product and kept with the weight
+    return _mmt_2d(lhs, cached_device_weight(rhs, stacked=False))
 
 
 @matmul.override(Tensor, Tensor)
 def matmul_tensor_tensor(lhs, rhs, *, transpose_rhs: bool):
     lhs = unbox_tensor(lhs)
+    holder = rhs  # the object the cast copy is kept with: the PrimitiveTensor, or the torch tensor itself
     rhs = unbox_tensor(rhs)
     if not transpose_rhs or rhs.dim() != 2 or lhs.dtype not in _FLOAT_DTYPES:
         return NotImplemented
-    return _mmt_2d(lhs, device_weight(rhs.to(lhs.dtype), stacked=False))
+    return _mmt_2d(lhs, cached_device_weight(holder, stacked=False, cast_to=lhs.dtype))
 
 
 def _linear(input, weight, bias, *, accum_dtype=None):
@@ -142,10 +185,7 @@ def _linear(input, weight, bias, *, accum_dtype=None):
     input = unbox_tensor(input)
     if isinstance(weight, QuantizedTensor):
         return matmul(input, weight, transpose_rhs=True)
-    weight = unbox_tensor(weight)
-    if weight.dtype != input.dtype:
-        weight = weight.to(dtype=input.dtype)
-    return matmul(input, weight, transpose_rhs=True)
+    return matmul(input, weight, transpose_rhs=True)  # a dense weight is cast to the input's dtype once and kept
 
 
 linear.override(Tensor, Tensor)(_linear)
@@ -195,12 +235,29 @@ def get_index_quantized_experts(tensor: QuantizedTensor, key):
     return gather_experts(tensor, experts)
 
 
+_LAST_DISPATCH = None  # (weakref to the experts tensor, its planes key, expert count, (offsets, perm))
+
+
+def _dispatch_of(experts: torch.Tensor, E: int):
+    """The dispatch arrays of an index tensor.  The three einsums of one PreGatherFFNMOE forward index with the same tensor:
+    the arrays are built for the first and reused by the other two."""
+    global _LAST_DISPATCH
+    import weakref
+
+    key = _planes_key(experts)
+    last = _LAST_DISPATCH
+    if last is not None and last[0]() is experts and last[1] == key and last[2] == E:
+        return last[3]
+    _, offsets, perm, _ = _hip.dispatch_build(experts, E)
+    _LAST_DISPATCH = (weakref.ref(experts), key, E, (offsets, perm))
+    return offsets, perm
+
+
 def _gathered_state(g: GatheredExpertsTensor):
     if g._device_weight is None:
-        g._device_weight = device_weight(g.weights, stacked=True)
+        g._device_weight = cached_device_weight(g.weights, stacked=True)
     if g._dispatch is None:
-        _, offsets, perm, _ = _hip.dispatch_build(g.experts, g._device_weight.experts)
-        g._dispatch = (offsets, perm)
+        g._dispatch = _dispatch_of(g.experts, g._device_weight.experts)
     return g._device_weight, g._dispatch
 
 

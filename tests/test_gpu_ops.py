@@ -10,8 +10,12 @@ pytestmark = pytest.mark.gpu
 
 
 def test_mmt_block_scaled_q8_reference_generator(device):
-    """Shapes, generators and tolerances of sharktank/tests/kernels/mmt_block_scaled_q8_test.py:24-41 (seed 42):
-    a [4,16,3200], d [3200,100,1], qs [3200,100,32]; expected = a @ (d*qs).flatten(1).T, atol 1e-3 (scaled), rtol 1e-5."""
+    """The shapes and the seed of sharktank/tests/kernels/mmt_block_scaled_q8_test.py:24-41 (a [4,16,3200], d [3200,100,1],
+    qs [3200,100,32], seed 42; expected = a @ (d*qs).flatten(1).T) through ops.matmul, with two stated changes: a and d
+    are drawn as rand / 64 where the reference draws rand * 64 (with * 64 every fp16 output is +inf, which compares equal
+    and checks nothing; test_kernels_mmt_block_scaled_q8 below runs the reference's own * 64 generator in fp32), and the
+    tolerances are atol 1e-2 with rtol 1e-4 (fp32) / 2e-3 (fp16) instead of atol 1e-3, rtol 1e-5: the reference compares
+    an fp32 kernel with an fp32 matmul, here the fp16 case rounds the dequantised weights and the result to fp16."""
     from sharktank_amd import ops, types as ST
 
     torch.manual_seed(42)
@@ -246,3 +250,79 @@ def test_kernels_einsum_2args_q4(device, a_dtype, es):
     assert O.rel_l2(got.float().cpu(), want) < (1e-5 if a_dtype == torch.float32 else 1e-3)
     with pytest.raises(NotImplementedError):
         kernels.einsum_2args_q4(a.to(device), d.to(device), qs.to(device), m.to(device), "ij,jk->ik")
+
+
+def test_quantized_matmul_descriptor_is_built_once_and_packed(device):
+    """ops.matmul / ops.linear / LinearLayer on a quantized weight build the device descriptor on the first call (planes made
+    contiguous, re-ordered into the streaming order) and reuse it afterwards, so they run the packed kernels; a changed
+    plane invalidates it."""
+    from sharktank_amd import ops, types as ST
+    from sharktank_amd.layers import LinearLayer
+
+    g = torch.Generator().manual_seed(12)
+    N, K = 512, 1024
+    d, qs = O.quantize_q8_0(torch.randn(N, K, generator=g) * 0.02)
+    w = ST.PlanarQuantizedTensor(name="weight", shape=[N, K], layout=ST.BlockScaledLayout([N, K], d.to(device), qs.to(device)))
+    x = torch.randn(3, 40, K, generator=g).to(torch.float16)
+    y1 = ops.matmul(x.to(device), w, transpose_rhs=True)
+    store = w.__dict__["_stmoe_descriptors"]
+    (key, dw), = store.values()
+    assert dw.is_packed
+    y2 = LinearLayer(ST.Theta({"weight": w}))(x.to(device))
+    assert next(iter(store.values()))[1] is dw, "the descriptor must be reused, not rebuilt"
+    want = O.mmt(x, O.dequant_block_scaled(d, qs).reshape(N, K).to(torch.float16))
+    assert torch.equal(y1, y2) and O.rel_l2(y1.cpu(), want) < 1e-3
+    # an in-place change of a plane gives a new descriptor and the new product
+    w.unpack().d.mul_(2.0)
+    y3 = ops.matmul(x.to(device), w, transpose_rhs=True)
+    assert next(iter(store.values()))[1] is not dw
+    assert O.rel_l2(y3.cpu(), O.mmt(x, O.dequant_block_scaled(d * 2, qs).reshape(N, K).to(torch.float16))) < 1e-3
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1"])
+@pytest.mark.parametrize("M", [1, 32, 2048])
+def test_ffn_layer_llama_shape(device, fmt, M):
+    """FFN (sharktank/sharktank/layers/ffn_block.py:21-51) at a Llama-8B shape, hidden 4096, FFN 14336, quantized weights:
+    the gated form on the fused kernels against the closed form down(silu(gate x) * up x) of the oracle, row by row."""
+    import moe_cases as MC
+    from sharktank_amd import types as ST
+    from sharktank_amd.layers import FFN
+
+    K, N = 4096, 14336
+    gg = torch.Generator(device=device).manual_seed(20)
+    planes, tensors = {}, {}
+    for name, shape in (("ffn_gate", [N, K]), ("ffn_up", [N, K]), ("ffn_down", [K, N])):
+        w = torch.randn(shape, generator=gg, device=device) * 0.02
+        q = O.quantize_q8_0(w) if fmt == "q8_0" else O.quantize_q4_1(w)
+        p = {"d": q[0], "qs": q[1]} if fmt == "q8_0" else {"d": q[0], "m": q[1], "qs": q[2]}
+        planes[name] = {k: v.cpu() for k, v in p.items()}
+        tensors[f"{name}.weight"] = MC.to_inference_tensor(fmt, p, shape, f"{name}.weight", device)
+    ffn = FFN(ST.Theta(tensors))
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(21)).to(torch.float16)
+    got = ffn(x.reshape(1, M, K).to(device)).reshape(M, K).cpu()
+    rows = list(range(M)) if M <= 32 else [0, 1, 255, 256, 257, 1023, 1024, 2047]
+    xs = x[rows]
+    dense = {n: MC.dense_from_planes(fmt, planes[n], [N, K] if n != "ffn_down" else [K, N], torch.float16) for n in planes}
+    z = torch.nn.functional.silu(O._mm_rt(xs, dense["ffn_gate"])) * O._mm_rt(xs, dense["ffn_up"])
+    want = O._mm_rt(z, dense["ffn_down"])
+    assert torch.isfinite(got.float()).all()
+    assert O.rel_l2(got[rows], want) < 1e-3
+
+
+def test_ffn_layer_ungated_and_with_bias(device):
+    """The forms without a fused kernel compose the linears as the reference does: un-gated FFN, and a gated one whose
+    down projection has a bias... which ops.linear has no kernel for: the error names the missing implementation."""
+    import moe_cases as MC
+    from sharktank_amd import types as ST
+    from sharktank_amd.layers import FFN
+
+    g = torch.Generator().manual_seed(22)
+    K, N, M = 256, 512, 24
+    up = torch.randn(N, K, generator=g) * 0.05
+    down = torch.randn(K, N, generator=g) * 0.05
+    theta = ST.Theta({"ffn_up.weight": ST.DefaultPrimitiveTensor(name="ffn_up.weight", data=up.to(torch.float16).to(device)),
+                      "ffn_down.weight": ST.DefaultPrimitiveTensor(name="ffn_down.weight", data=down.to(torch.float16).to(device))})
+    x = torch.randn(M, K, generator=g).to(torch.float16)
+    got = FFN(theta, is_gated=False, activation_fn=torch.nn.functional.gelu)(x.to(device)).cpu()
+    want = O._mm_rt(torch.nn.functional.gelu(O._mm_rt(x, up.to(torch.float16))), down.to(torch.float16))
+    assert O.rel_l2(got, want) < 1e-3
