@@ -338,3 +338,36 @@ def test_single_token_forward_equals_staged_calls(device, E, k, dtype):
     y = _hip.grouped_ffn(xn, wg, wu, wd, block.experts._act, offsets, perm, k)
     staged = _hip.combine(y, gate, inv, 1, k, residual=h)
     assert torch.equal(staged.view(torch.int16), fused.reshape(1, case.K).view(torch.int16))
+
+
+@pytest.mark.parametrize("T", [2, 31, 32, 200, 256, 257])
+@pytest.mark.parametrize("E,k", [(8, 2), (64, 6)])
+def test_small_batch_forward_equals_staged_calls(device, T, E, k):
+    """The fused forward (one C-ABI call, one workspace) must give the same bits as router, dispatch_build, grouped_ffn and
+    combine called one after the other, also when called again on the same workspace and whatever the workspace held
+    before (nothing in it needs an initial value)."""
+    from sharktank_amd import _hip
+    from sharktank_amd.layers import MoeBlock
+    from sharktank_amd.types import unbox_tensor
+
+    dtype = torch.float16
+    case = MC.build(MC.Case(T=T, K=512, N=256, E=E, k=k, fmt="q8_0", dtype=dtype, seed=800 + T + E))
+    theta = MC.make_theta(case, device)
+    block = MoeBlock(theta, expert_count=E, expert_used_count=k, rms_epsilon=case.eps)
+    wg, wu, wd = block.experts.device_weights()
+    h = case.planes["h"].to(device)
+    block.reserve_workspace(T, dtype, device)
+    block._workspace.fill_(0xFF)
+    fused, idx_f, gate_f = block(h.reshape(1, T, case.K), return_routing=True)
+    again = block(h.reshape(1, T, case.K))
+    block._workspace.fill_(0x01)
+    third = block(h.reshape(1, T, case.K))
+
+    xn = _hip.rms_norm(h, unbox_tensor(block.ffn_norm.weight), case.eps)
+    idx, gate, _ = _hip.router_topk(xn, block._router_weight(dtype), k)
+    assert torch.equal(idx.cpu().to(torch.int64), idx_f.cpu().to(torch.int64)) and torch.equal(gate, gate_f)
+    counts, offsets, perm, inv = _hip.dispatch_build(idx, E)
+    y = _hip.grouped_ffn(xn, wg, wu, wd, block.experts._act, offsets, perm, k)
+    staged = _hip.combine(y, gate, inv, T, k, residual=h)
+    for got in (fused, again, third):
+        assert torch.equal(staged.view(torch.int16), got.reshape(T, case.K).view(torch.int16))
