@@ -125,6 +125,20 @@ int stmoe_dequant_tensor_scaled(const void* qs, int qs_dtype, const void* d, con
 int stmoe_quantize_fp8(const void* x, int x_dtype, const float* rscale, int64_t n, void* out_fp8,
                        stmoe_stream_t stream);
 
+/* StaticScaledQuantizer per-axis quantize to fp8 (sharktank/sharktank/types/quantizers.py:184-230): with j the index along
+ * the scaled axis (`axis_len` entries, `inner` elements behind it: element i has j = (i / inner) % axis_len),
+ * out = e4m3fn(clamp(x * scale[j], -448, 448)); the product is computed in the dtype eager torch gives the two tensors'
+ * product: x's dtype when the scales have it, fp32 otherwise (scale_dtype f32).  The matching TensorScaledLayout holds
+ * d = reciprocal scales, broadcast along the same axis: stmoe_dequant_tensor_scaled_per_axis. */
+int stmoe_quantize_fp8_per_axis(const void* x, int x_dtype, const void* scale, int scale_dtype, int64_t axis_len,
+                                int64_t inner, int64_t n, void* out_fp8, stmoe_stream_t stream);
+
+/* TensorScaledLayout.dequant (layouts.py:163-181) with d (and m) of `axis_len` values broadcast along one axis that has
+ * `inner` elements behind it: out = ((D(qs) - m[j]) * d[j]).to(out_dtype), j = (i / inner) % axis_len, D = d_dtype. */
+int stmoe_dequant_tensor_scaled_per_axis(const void* qs, int qs_dtype, const void* d, const void* m /*nullable*/,
+                                         int d_dtype, int64_t axis_len, int64_t inner, int64_t n, void* out,
+                                         int out_dtype, stmoe_stream_t stream);
+
 /* DynamicScaledQuantizer._quantize_raw_tensor for float8_e4m3fn (sharktank/sharktank/types/quantizers.py:368-389):
  * amax = max|x|; scale = T(448 / max(amax, eps)), eps = finfo(float8_e4m3fn).eps = 0.125; rscale = T(1 / scale);
  * out = e4m3fn(clamp(T(x * scale))), every step in x's dtype T as eager torch computes it.  scale_rscale_out receives

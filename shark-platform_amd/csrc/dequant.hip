@@ -69,10 +69,10 @@ promote_i4_kernel(const uint8_t* __restrict__ packed, int64_t n_bytes, int is_si
 template <typename DD, typename OUT>
 __global__ void __launch_bounds__(256)
 dequant_tensor_scaled_kernel(const void* __restrict__ qs, int qs_dtype, const DD* __restrict__ d,
-                             const DD* __restrict__ m, int64_t per_scale, int64_t n, OUT* __restrict__ out) {
+                             const DD* __restrict__ m, int64_t per_scale, int64_t d_count, int64_t n, OUT* __restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const int64_t j = i / per_scale;
+  const int64_t j = (i / per_scale) % d_count;  // scale index along the scaled axis (axes before it repeat the scales)
   float q = round_to<DD>(load_as_f32(qs, qs_dtype, i));
   const float dv = Cvt<DD>::to_f32(d[j]);
   if (m) q = round_to<DD>(__fsub_rn(q, Cvt<DD>::to_f32(m[j])));
@@ -241,18 +241,18 @@ extern "C" int stmoe_promote_i4(const uint8_t* qs_packed, int64_t n_bytes, int i
 
 template <typename DD>
 static int launch_tensor_scaled(const void* qs, int qs_dtype, const void* d, const void* m, int64_t per_scale,
-                                int64_t n, void* out, int out_dtype, hipStream_t st) {
+                                int64_t d_count, int64_t n, void* out, int out_dtype, hipStream_t st) {
   const int64_t blocks = (n + 255) / 256;
   dim3 g((unsigned)blocks);
   switch (out_dtype) {
     case STMOE_F32:
-      dequant_tensor_scaled_kernel<DD, float><<<g, 256, 0, st>>>(qs, qs_dtype, (const DD*)d, (const DD*)m, per_scale, n, (float*)out);
+      dequant_tensor_scaled_kernel<DD, float><<<g, 256, 0, st>>>(qs, qs_dtype, (const DD*)d, (const DD*)m, per_scale, d_count, n, (float*)out);
       break;
     case STMOE_F16:
-      dequant_tensor_scaled_kernel<DD, f16_t><<<g, 256, 0, st>>>(qs, qs_dtype, (const DD*)d, (const DD*)m, per_scale, n, (f16_t*)out);
+      dequant_tensor_scaled_kernel<DD, f16_t><<<g, 256, 0, st>>>(qs, qs_dtype, (const DD*)d, (const DD*)m, per_scale, d_count, n, (f16_t*)out);
       break;
     case STMOE_BF16:
-      dequant_tensor_scaled_kernel<DD, bf16_t><<<g, 256, 0, st>>>(qs, qs_dtype, (const DD*)d, (const DD*)m, per_scale, n, (bf16_t*)out);
+      dequant_tensor_scaled_kernel<DD, bf16_t><<<g, 256, 0, st>>>(qs, qs_dtype, (const DD*)d, (const DD*)m, per_scale, d_count, n, (bf16_t*)out);
       break;
     default:
       return set_error(STMOE_ERR_DTYPE, "dequant_tensor_scaled: out_dtype %d is not f32/f16/bf16", out_dtype);
@@ -271,11 +271,66 @@ extern "C" int stmoe_dequant_tensor_scaled(const void* qs, int qs_dtype, const v
                 "dequant_tensor_scaled: %lld scales do not divide %lld elements", (long long)d_count, (long long)n);
   const int64_t per_scale = n / d_count;
   switch (d_dtype) {
-    case STMOE_F32: return launch_tensor_scaled<float>(qs, qs_dtype, d, m, per_scale, n, out, out_dtype, as_stream(stream));
-    case STMOE_F16: return launch_tensor_scaled<f16_t>(qs, qs_dtype, d, m, per_scale, n, out, out_dtype, as_stream(stream));
-    case STMOE_BF16: return launch_tensor_scaled<bf16_t>(qs, qs_dtype, d, m, per_scale, n, out, out_dtype, as_stream(stream));
+    case STMOE_F32: return launch_tensor_scaled<float>(qs, qs_dtype, d, m, per_scale, d_count, n, out, out_dtype, as_stream(stream));
+    case STMOE_F16: return launch_tensor_scaled<f16_t>(qs, qs_dtype, d, m, per_scale, d_count, n, out, out_dtype, as_stream(stream));
+    case STMOE_BF16: return launch_tensor_scaled<bf16_t>(qs, qs_dtype, d, m, per_scale, d_count, n, out, out_dtype, as_stream(stream));
     default: return set_error(STMOE_ERR_DTYPE, "dequant_tensor_scaled: scale dtype %d is not f32/f16/bf16", d_dtype);
   }
+}
+
+extern "C" int stmoe_dequant_tensor_scaled_per_axis(const void* qs, int qs_dtype, const void* d, const void* m, int d_dtype,
+                                                    int64_t axis_len, int64_t inner, int64_t n, void* out, int out_dtype,
+                                                    stmoe_stream_t stream) {
+  STMOE_REQUIRE(n >= 0, STMOE_ERR_SHAPE, "dequant_tensor_scaled_per_axis: n %lld < 0", (long long)n);
+  if (n == 0) return STMOE_OK;
+  STMOE_REQUIRE(qs && d && out, STMOE_ERR_NULL, "dequant_tensor_scaled_per_axis: NULL pointer");
+  STMOE_REQUIRE(qs_dtype >= STMOE_F32 && qs_dtype <= STMOE_U8, STMOE_ERR_DTYPE, "dequant_tensor_scaled_per_axis: qs dtype %d", qs_dtype);
+  STMOE_REQUIRE(axis_len >= 1 && inner >= 1 && n % (axis_len * inner) == 0, STMOE_ERR_SHAPE,
+                "dequant_tensor_scaled_per_axis: an axis of %lld with %lld elements behind it does not divide %lld elements",
+                (long long)axis_len, (long long)inner, (long long)n);
+  switch (d_dtype) {
+    case STMOE_F32: return launch_tensor_scaled<float>(qs, qs_dtype, d, m, inner, axis_len, n, out, out_dtype, as_stream(stream));
+    case STMOE_F16: return launch_tensor_scaled<f16_t>(qs, qs_dtype, d, m, inner, axis_len, n, out, out_dtype, as_stream(stream));
+    case STMOE_BF16: return launch_tensor_scaled<bf16_t>(qs, qs_dtype, d, m, inner, axis_len, n, out, out_dtype, as_stream(stream));
+    default: return set_error(STMOE_ERR_DTYPE, "dequant_tensor_scaled_per_axis: scale dtype %d is not f32/f16/bf16", d_dtype);
+  }
+}
+
+// Per-axis static quantisation: x * scale[j] with j the index along the scaled axis, in the dtype eager torch gives the
+// product of the two tensors (P = T when the scales have x's dtype, fp32 otherwise), clamped and cast.
+template <typename T, typename S, typename P>
+__global__ void __launch_bounds__(256)
+quantize_fp8_per_axis_kernel(const T* __restrict__ x, const S* __restrict__ scale, int64_t axis_len, int64_t inner, int64_t n,
+                             uint8_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int64_t j = (i / inner) % axis_len;
+  float q = round_to<P>(__fmul_rn(Cvt<T>::to_f32(x[i]), Cvt<S>::to_f32(scale[j])));
+  q = fminf(fmaxf(q, -448.0f), 448.0f);
+  if (q != q) q = __uint_as_float(0x7fc00000u);
+  out[i] = f32_to_fp8_e4m3fn(q);
+}
+
+extern "C" int stmoe_quantize_fp8_per_axis(const void* x, int x_dtype, const void* scale, int scale_dtype, int64_t axis_len,
+                                           int64_t inner, int64_t n, void* out_fp8, stmoe_stream_t stream) {
+  STMOE_REQUIRE(n >= 0, STMOE_ERR_SHAPE, "quantize_fp8_per_axis: n %lld < 0", (long long)n);
+  if (n == 0) return STMOE_OK;
+  STMOE_REQUIRE(x && scale && out_fp8, STMOE_ERR_NULL, "quantize_fp8_per_axis: NULL pointer");
+  STMOE_REQUIRE(axis_len >= 1 && inner >= 1 && n % (axis_len * inner) == 0, STMOE_ERR_SHAPE,
+                "quantize_fp8_per_axis: an axis of %lld with %lld elements behind it does not divide %lld elements",
+                (long long)axis_len, (long long)inner, (long long)n);
+  dim3 g((unsigned)((n + 255) / 256));
+  hipStream_t st = as_stream(stream);
+#define STMOE_QPA(TT, SS, PP)                                                                                            \
+  quantize_fp8_per_axis_kernel<TT, SS, PP><<<g, 256, 0, st>>>((const TT*)x, (const SS*)scale, axis_len, inner, n, (uint8_t*)out_fp8)
+  if (x_dtype == STMOE_F32 && scale_dtype == STMOE_F32) STMOE_QPA(float, float, float);
+  else if (x_dtype == STMOE_F16 && scale_dtype == STMOE_F32) STMOE_QPA(f16_t, float, float);
+  else if (x_dtype == STMOE_BF16 && scale_dtype == STMOE_F32) STMOE_QPA(bf16_t, float, float);
+  else if (x_dtype == STMOE_F16 && scale_dtype == STMOE_F16) STMOE_QPA(f16_t, f16_t, f16_t);
+  else if (x_dtype == STMOE_BF16 && scale_dtype == STMOE_BF16) STMOE_QPA(bf16_t, bf16_t, bf16_t);
+  else return set_error(STMOE_ERR_DTYPE, "quantize_fp8_per_axis: x dtype %d with scale dtype %d not implemented", x_dtype, scale_dtype);
+#undef STMOE_QPA
+  return check_launch("quantize_fp8_per_axis");
 }
 
 extern "C" int stmoe_quantize_fp8(const void* x, int x_dtype, const float* rscale, int64_t n, void* out_fp8,

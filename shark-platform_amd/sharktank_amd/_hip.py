@@ -75,6 +75,9 @@ SIGNATURES = {
     "stmoe_unpack": (c_int, [POINTER(StmoeWeight), POINTER(StmoeWeight), c_void_p]),
     "stmoe_gguf_ingest": (c_int, [c_void_p, c_int, POINTER(StmoeWeight), c_void_p]),
     "stmoe_quantize_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
+    "stmoe_quantize_fp8_per_axis": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
+    "stmoe_dequant_tensor_scaled_per_axis": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p,
+                                                     c_int, c_void_p]),
     "stmoe_dynamic_quantize_fp8_scratch_bytes": (c_size_t, []),
     "stmoe_dynamic_quantize_fp8": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "stmoe_fake_quant_fp8": (c_int, [c_void_p, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
@@ -235,17 +238,54 @@ def dequant_tensor_scaled(qs, d, m, dtype: torch.dtype) -> torch.Tensor:
     m_c = None if m is None else _contig(m).to(d_c.dtype)
     n = qs_c.numel()
     d_count = d_c.numel()
-    if d_count != 1:
-        # per-axis scales broadcast along one axis: only a leading-axis broadcast maps to contiguous runs
-        lead = qs_c.shape[0] if qs_c.dim() else 1
-        if d_count != lead or tuple(d_c.shape) not in ((lead,), (lead,) + (1,) * (qs_c.dim() - 1)):
-            raise NotImplementedError(f"TensorScaledLayout dequant: scale shape {tuple(d.shape)} for qs {tuple(qs.shape)}")
     if m_c is not None and m_c.numel() != d_count:
         raise NotImplementedError("TensorScaledLayout dequant: offset and scale must have the same shape")
     out = torch.empty(qs_c.shape, dtype=dtype, device=dev)
+    axis = _broadcast_axis(d_c, qs_c) if d_count != 1 else None
     with torch.cuda.device(dev):
-        _check(lib.stmoe_dequant_tensor_scaled(_ptr(qs_c), dtype_enum(qs_c.dtype), _ptr(d_c), _ptr(m_c), dtype_enum(d_c.dtype),
-                                               d_count, n, _ptr(out), dtype_enum(dtype), _stream(dev)))
+        if axis is None:
+            _check(lib.stmoe_dequant_tensor_scaled(_ptr(qs_c), dtype_enum(qs_c.dtype), _ptr(d_c), _ptr(m_c), dtype_enum(d_c.dtype),
+                                                   1, n, _ptr(out), dtype_enum(dtype), _stream(dev)))
+        else:
+            inner = 1
+            for s_ in qs_c.shape[axis + 1:]:
+                inner *= s_
+            _check(lib.stmoe_dequant_tensor_scaled_per_axis(_ptr(qs_c), dtype_enum(qs_c.dtype), _ptr(d_c), _ptr(m_c),
+                                                            dtype_enum(d_c.dtype), d_count, inner, n, _ptr(out),
+                                                            dtype_enum(dtype), _stream(dev)))
+    return out
+
+
+def _broadcast_axis(d: torch.Tensor, qs: torch.Tensor) -> int:
+    """The axis of `qs` along which the scales `d` vary: `d` is [A] (then the leading axis, the per-expert case) or has
+    qs's rank with ones everywhere but on one axis (the per-axis quantizer's broadcast shape)."""
+    if d.dim() == 1:
+        if qs.dim() and qs.shape[0] == d.shape[0]:
+            return 0
+    elif d.dim() == qs.dim():
+        axes = [i for i, s_ in enumerate(d.shape) if s_ != 1]
+        if len(axes) == 1 and d.shape[axes[0]] == qs.shape[axes[0]]:
+            return axes[0]
+    raise NotImplementedError(f"TensorScaledLayout dequant: scale shape {tuple(d.shape)} for qs {tuple(qs.shape)}")
+
+
+def quantize_fp8_per_axis(x: torch.Tensor, scale: torch.Tensor, axis: int) -> torch.Tensor:
+    """StaticScaledQuantizer's per-axis branch: e4m3fn(clamp(x * scale broadcast along `axis`))."""
+    dev = _dev(x, scale)
+    lib = load_library()
+    x_c, s_c = _contig(x), _contig(scale).reshape(-1)
+    axis = axis % x_c.dim()
+    if s_c.numel() != x_c.shape[axis]:
+        raise ValueError(f"per-axis scale of {s_c.numel()} values for axis {axis} of {tuple(x_c.shape)}")
+    if s_c.dtype != x_c.dtype and s_c.dtype != torch.float32:
+        s_c = s_c.to(torch.float32)  # eager torch would promote the product of two 16-bit dtypes to fp32 as well
+    inner = 1
+    for s_ in x_c.shape[axis + 1:]:
+        inner *= s_
+    out = torch.empty(x_c.shape, dtype=torch.float8_e4m3fn, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_quantize_fp8_per_axis(_ptr(x_c), dtype_enum(x_c.dtype), _ptr(s_c), dtype_enum(s_c.dtype), s_c.numel(),
+                                               inner, x_c.numel(), _ptr(out), _stream(dev)))
     return out
 
 

@@ -15,7 +15,8 @@ from .. import _hip
 from .. import ops
 from ..ops import device_weight, gather_experts
 from ..utils import debugging
-from ..types import DefaultPrimitiveTensor, PlanarQuantizedTensor, QuantizedTensor, StaticScaledQuantizer, Theta
+from ..types import (DefaultPrimitiveTensor, DynamicScaledQuantizer, PlanarQuantizedTensor, QuantizedTensor,
+                     StaticScaledQuantizer, Theta)
 from .base import ThetaLayer
 from .linear import LinearLayer
 
@@ -45,8 +46,14 @@ class PreGatherFFNMOE(ThetaLayer):
         self.q_input = theta.optional_tensor("ffn_gate_exps", "q_input")
         self.q_intermediate = theta.optional_tensor("ffn_down_exps", "q_input")
         for q in (self.q_input, self.q_intermediate):
-            if q is not None and not isinstance(q, StaticScaledQuantizer):
+            if q is not None and not isinstance(q, (StaticScaledQuantizer, DynamicScaledQuantizer)):
                 raise NotImplementedError(f"PreGatherFFNMOE: activation quantizer {type(q).__name__} has no kernel")
+        # Inside the fused kernels the intermediate exists only tile by tile, so its quantizer must be known before the
+        # launch: static and per tensor.  The input quantizer may also be per axis or dynamic (see forward).
+        qz = self.q_intermediate
+        if qz is not None and (not isinstance(qz, StaticScaledQuantizer) or qz.axis is not None):
+            raise NotImplementedError("PreGatherFFNMOE: the quantizer of the gated intermediate (ffn_down_exps.q_input) must be "
+                                      "static and per tensor; a dynamic or per-axis one needs the whole intermediate first")
         self.activation = activation
         self._act = activation_enum(activation)
         self._dw = None
@@ -83,10 +90,24 @@ class PreGatherFFNMOE(ThetaLayer):
         return torch.sum(ffn_down, dim=1)
 
     def activation_scales(self):
-        """(reciprocal scale of the input quantizer, of the intermediate quantizer); None where there is none."""
-        xs = self.q_input.reciprocal_scale if self.q_input is not None else None
+        """(reciprocal scale of the input quantizer, of the intermediate quantizer) as the kernels take them: one device
+        float each; None where there is no quantizer or where `quantized_input` has to apply it before the launch."""
+        q = self.q_input
+        xs = q.reciprocal_scale if isinstance(q, StaticScaledQuantizer) and q.axis is None else None
         zs = self.q_intermediate.reciprocal_scale if self.q_intermediate is not None else None
         return xs, zs
+
+    def quantized_input(self, h: torch.Tensor):
+        """(h', x_scale): how the input quantizer reaches the kernels.  Static per tensor: the kernels quantise themselves
+        (h, reciprocal scale).  Per axis or dynamic: h is quantised and dequantised here with the quantizer's own
+        arithmetic (x * scale, not x / reciprocal scale), as LinearLayer does with a q_input
+        (sharktank/sharktank/layers/linear.py:72-78), and the kernels see plain activations."""
+        q = self.q_input
+        if q is None:
+            return h, None
+        if isinstance(q, StaticScaledQuantizer) and q.axis is None:
+            return h, q.reciprocal_scale
+        return q.quantize(h).unpack().dequant(h.dtype), None
 
     @property
     def expert_count(self) -> int:
@@ -110,7 +131,8 @@ class PreGatherFFNMOE(ThetaLayer):
             if bool(((experts < 0) | (experts >= wg.experts)).any()):
                 raise IndexError(f"PreGatherFFNMOE: expert index outside 0..{wg.experts - 1}")
         _, offsets, perm, inv = _hip.dispatch_build(experts, wg.experts)
-        xs, zs = self.activation_scales()
+        _, zs = self.activation_scales()
+        h, xs = self.quantized_input(h)
         y = _hip.grouped_ffn(h, wg, wu, wd, self._act, offsets, perm, k, variant=self.kernel_variant, x_scale=xs, z_scale=zs)
         return _hip.combine(y, expert_gate.to(h.dtype), inv, T, k)
 

@@ -23,22 +23,30 @@ class QuantizerTensor(InferenceTensor):
 
 
 class StaticScaledQuantizer(QuantizerTensor):
+    """Mirror of sharktank/sharktank/types/quantizers.py:83-260 for float8_e4m3fn without offsets: per tensor (0-d scale:
+    `saturate_cast(t / reciprocal_scale)`) or per axis (1-d scale: `saturate_cast(t * scale)` with the scale broadcast
+    along `axis`), both producing a TensorScaledLayout whose `d` is the reciprocal scale."""
+
     def __init__(self, *, scale: torch.Tensor, dtype: torch.dtype, axis: Optional[int] = None,
                  reciprocal_scale: Optional[torch.Tensor] = None, offset: Optional[torch.Tensor] = None,
                  disable_saturate: bool = False, name: str = UnnamedTensorName):
         super().__init__(shape=scale.shape, name=name)
-        if axis is not None or offset is not None or disable_saturate:
-            raise NotImplementedError("StaticScaledQuantizer: only the per-tensor, offset-free, saturating form has a kernel")
+        if offset is not None or disable_saturate:
+            raise NotImplementedError("StaticScaledQuantizer: only the offset-free, saturating forms have kernels")
         if dtype != torch.float8_e4m3fn:
             raise NotImplementedError(f"StaticScaledQuantizer: target dtype {dtype} has no kernel (gfx950 MFMA consumes float8_e4m3fn)")
-        assert len(scale.shape) == 0, "Expected per-tensor scale to be 0D"
+        if axis is None:
+            assert len(scale.shape) == 0, "Expected per-tensor scale to be 0D"
+        else:
+            assert len(scale.shape) == 1, "Expected per-axis scale to be 1D"
+        self._axis = axis
         self._scale = scale
         self._reciprocal_scale = reciprocal_scale if reciprocal_scale is not None else 1.0 / scale
         self._dtype = dtype
 
     @property
     def axis(self):
-        return None
+        return self._axis
 
     @property
     def offset(self):
@@ -61,17 +69,26 @@ class StaticScaledQuantizer(QuantizerTensor):
         return {f"{self.name}:d": self._scale, f"{self.name}:rscale": self._reciprocal_scale}
 
     def _clone_with_globals(self, new_globals):
-        return StaticScaledQuantizer(name=self.name, scale=new_globals[f"{self.name}:d"],
+        return StaticScaledQuantizer(name=self.name, scale=new_globals[f"{self.name}:d"], axis=self._axis,
                                      reciprocal_scale=new_globals[f"{self.name}:rscale"], dtype=self._dtype)
 
     def _quantize_raw_tensor(self, t: torch.Tensor, *, name: str) -> QuantizedTensor:
         from .. import _hip
 
-        qs = _hip.quantize_fp8(t, self._reciprocal_scale)
         shape = list(t.shape)
+        if self._axis is None:
+            qs = _hip.quantize_fp8(t, self._reciprocal_scale)
+            d = self._reciprocal_scale
+        else:
+            axis = self._axis
+            assert 0 <= axis < len(shape), f"Per-axis scale {axis} out of bounds of shape {shape}"
+            qs = _hip.quantize_fp8_per_axis(t, self._scale, axis)
+            scale_shape = [1] * len(shape)
+            scale_shape[axis] = self._scale.shape[0]
+            d = self._reciprocal_scale.reshape(scale_shape)
         return PlanarQuantizedTensor(
             shape=shape, name=name,
-            layout=TensorScaledLayout(shape=shape, d=self._reciprocal_scale, qs=qs, m=None, dtype=t.dtype),
+            layout=TensorScaledLayout(shape=shape, d=d, qs=qs, m=None, dtype=t.dtype),
         )
 
 

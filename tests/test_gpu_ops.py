@@ -326,3 +326,67 @@ def test_ffn_layer_ungated_and_with_bias(device):
     got = FFN(theta, is_gated=False, activation_fn=torch.nn.functional.gelu)(x.to(device)).cpu()
     want = O._mm_rt(torch.nn.functional.gelu(O._mm_rt(x, up.to(torch.float16))), down.to(torch.float16))
     assert O.rel_l2(got, want) < 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("scale_dtype", ["same", torch.float32])
+@pytest.mark.parametrize("shape,axis", [((40, 96), 1), ((40, 96), 0), ((3, 17, 64), 1), ((3, 17, 64), 2)])
+def test_static_scaled_quantizer_per_axis(device, dtype, scale_dtype, shape, axis):
+    """StaticScaledQuantizer with a 1-d scale (sharktank/sharktank/types/quantizers.py:184-230): samples bit for bit those
+    of the oracle's per-axis branch (the product in the dtype torch promotes the two tensors to), and the layout's dequant
+    with the broadcast reciprocal scale bit for bit the oracle's TensorScaledLayout dequant."""
+    from sharktank_amd import types as ST
+
+    g = torch.Generator().manual_seed(31 + axis)
+    sdt = dtype if scale_dtype == "same" else scale_dtype
+    t = (torch.randn(shape, generator=g) * 3).to(dtype)
+    t.view(-1)[0] = 1000.0  # saturates
+    scale = (torch.rand(shape[axis], generator=g) * 60 + 20).to(sdt)
+    q = ST.StaticScaledQuantizer(scale=scale.to(device), dtype=torch.float8_e4m3fn, axis=axis)
+    assert q.axis == axis
+    qt = q.quantize(t.to(device))
+    layout = qt.unpack()
+    want_qs, want_d, _ = O.static_quantize_per_axis(t, scale, axis, torch.float8_e4m3fn)
+    assert torch.equal(layout.qs.cpu().view(torch.uint8), want_qs.view(torch.uint8))
+    assert list(layout.d.shape) == list(want_d.shape) and torch.equal(layout.d.cpu(), want_d)
+    want = O.dequant_tensor_scaled(want_d, want_qs, layout_dtype=dtype)
+    got = layout.dequant()
+    assert got.dtype == want.dtype
+    view = torch.int32 if want.dtype == torch.float32 else torch.int16
+    assert torch.equal(got.cpu().view(view), want.view(view))
+
+
+@pytest.mark.parametrize("kind", ["dynamic", "per_axis"])
+def test_pre_gather_ffn_moe_with_dynamic_and_per_axis_input_quantizers(device, kind):
+    """ffn_gate_exps.q_input as a DynamicScaledQuantizer (scale from the input's own maximum) or as a per-axis static
+    quantizer (one scale per hidden feature): the layer quantises and dequantises its input with the quantizer's own
+    arithmetic and must match the oracle fed with the same fake-quantised input."""
+    import moe_cases as MC
+    from sharktank_amd import types as ST
+    from sharktank_amd.layers import PreGatherFFNMOE
+
+    case = MC.build(MC.Case(T=48, K=512, N=768, fmt="q8_0", dtype=torch.float16, seed=61))
+    x = case.planes["h"]
+    g = torch.Generator().manual_seed(62)
+    idx = torch.stack([torch.randperm(case.E, generator=g)[:case.k] for _ in range(case.T)])
+    gate = torch.full((case.T, case.k), 0.5, dtype=torch.float16)
+    flat = MC.make_theta(case, device).flatten()
+    if kind == "dynamic":
+        flat["ffn_gate_exps.q_input"] = ST.DynamicScaledQuantizer(name="ffn_gate_exps.q_input", dtype=torch.float8_e4m3fn)
+        qs, rscale = O.dynamic_quantize(x, torch.float8_e4m3fn)
+        xq = O.dequant_tensor_scaled(rscale, qs, layout_dtype=torch.float16)
+    else:
+        scale = (torch.rand(case.K, generator=g) * 40 + 60).to(torch.float32)
+        flat["ffn_gate_exps.q_input"] = ST.StaticScaledQuantizer(name="ffn_gate_exps.q_input", scale=scale.to(device),
+                                                                 dtype=torch.float8_e4m3fn, axis=1)
+        qs, d, _ = O.static_quantize_per_axis(x, scale, 1, torch.float8_e4m3fn)
+        xq = O.dequant_tensor_scaled(d, qs, layout_dtype=torch.float16).to(torch.float16)
+    ffn = PreGatherFFNMOE(ST.Theta(flat))
+    got = ffn(x.to(device), idx.to(device), gate.to(device)).cpu()
+    wg, wu, wd = MC.dense_weights(case)
+    want = O.grouped_ffn_moe(xq.to(torch.float16), idx, gate, wg, wu, wd, case.activation)
+    assert O.rel_l2(got, want) < 1e-3
+    # a dynamic quantizer of the intermediate is refused by name
+    flat["ffn_down_exps.q_input"] = ST.DynamicScaledQuantizer(name="ffn_down_exps.q_input", dtype=torch.float8_e4m3fn)
+    with pytest.raises(NotImplementedError, match="intermediate"):
+        PreGatherFFNMOE(ST.Theta(flat))
