@@ -114,6 +114,21 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     };
     // Converts register set SET (the weights of a K step s) into weight stage STAGE; with TAIL the tail's MFMAs of step s
     // follow each piece's conversion (token operands: register set s % 2 = TXSET).
+    auto store_piece = [&](auto set_tag, auto stage_tag, auto tail_tag, auto txset_tag, int j) {
+      constexpr int SET = decltype(set_tag)::value, STAGE = decltype(stage_tag)::value, TXSET = decltype(txset_tag)::value;
+      constexpr bool TAIL = decltype(tail_tag)::value != 0;
+      uint32_t v[8];
+      wreg[SET][j].landed();  // awaited by the previous step's vm_wait (or the prologue's)
+      wreg[SET][j].template convert<T>(waddr[j], v);
+      uint16_t* row = w_st + STAGE * WSTAGE + piece_row(j) * BIG_LS;
+      const u32x4_t lo = (u32x4_t){v[0], v[1], v[2], v[3]}, hi = (u32x4_t){v[4], v[5], v[6], v[7]};
+      *reinterpret_cast<u32x4_t*>(row + st_swz0) = lo;
+      *reinterpret_cast<u32x4_t*>(row + st_swz1) = hi;
+      if constexpr (TAIL) {
+        tacc[j] = mfma16b<T>(lo, tx[TXSET][0], tacc[j]);
+        tacc[j] = mfma16b<T>(hi, tx[TXSET][1], tacc[j]);
+      }
+    };
     auto store_w = [&](auto set_tag, auto stage_tag, auto tail_tag, auto txset_tag) {
       constexpr int SET = decltype(set_tag)::value, STAGE = decltype(stage_tag)::value, TXSET = decltype(txset_tag)::value;
       constexpr bool TAIL = decltype(tail_tag)::value != 0;
@@ -122,19 +137,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
         vm_landed(tx[TXSET][1]);
       }
 #pragma unroll
-      for (int j = 0; j < WPIECES; ++j) {
-        uint32_t v[8];
-        wreg[SET][j].landed();  // awaited by the previous step's vm_wait (or the prologue's)
-        wreg[SET][j].template convert<T>(waddr[j], v);
-        uint16_t* row = w_st + STAGE * WSTAGE + piece_row(j) * BIG_LS;
-        const u32x4_t lo = (u32x4_t){v[0], v[1], v[2], v[3]}, hi = (u32x4_t){v[4], v[5], v[6], v[7]};
-        *reinterpret_cast<u32x4_t*>(row + st_swz0) = lo;
-        *reinterpret_cast<u32x4_t*>(row + st_swz1) = hi;
-        if constexpr (TAIL) {
-          tacc[j] = mfma16b<T>(lo, tx[TXSET][0], tacc[j]);
-          tacc[j] = mfma16b<T>(hi, tx[TXSET][1], tacc[j]);
-        }
-      }
+      for (int j = 0; j < WPIECES; ++j) store_piece(set_tag, stage_tag, tail_tag, txset_tag, j);
     };
     auto load_x = [&](auto xstage_tag, int kt) {
       constexpr int XS = decltype(xstage_tag)::value;
@@ -162,17 +165,40 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     // joins.  That matters because the loads into registers are invisible to the compiler: a register copy or a spill that
     // it placed where two paths with different register assignments meet would move a register whose load has not landed.
     const int last = nkt - 1;
+    // The loads of a step are spread between the conversions of its four weight pieces instead of following them in one
+    // burst: the compute unit's one vector-memory path takes a wavefront's 1 KB request about every 13 cycles, and the 64
+    // requests of a step (4 producers x 16) queue up behind each other; a producer that issues them back to back sits in
+    // that queue for 800 cycles after its 1200 cycles of conversion, one that feeds them in between does both at once.
+    // Piece j's registers are free once it is converted, so its reload (step kt + 4) follows directly, then two of the
+    // step's eight token loads.  All loads of a step are therefore younger than all loads of the step before, and the
+    // wait at the end of a step lets exactly this step's loads stay in flight.
     auto k_step = [&](auto r_tag, auto tail_tag, int kt) {
       constexpr int R = decltype(r_tag)::value;
       constexpr bool TAIL = decltype(tail_tag)::value != 0;
       constexpr int TLOADS = TAIL ? 2 : 0;
+      constexpr int XS = (R + 2) % 3;
       using Set = WsInt<(R + 1) % 3>;
       using TxSet = WsInt<(R + 1) % 2>;
-      if (kt < last) store_w(Set{}, WsInt<(R + 1) % 2>{}, tail_tag, TxSet{});
+      using Stage = WsInt<(R + 1) % 2>;
+      const char* xsrc = reinterpret_cast<const char*>(p.a) + (kt0 + min(kt + 2, last)) * (BIG_BK * 2);
+      const int ktw = kt0 + min(kt + 4, last);
+      const bool conv = kt < last;
+      if constexpr (TAIL) {
+        vm_landed(tx[TxSet::value][0]);
+        vm_landed(tx[TxSet::value][1]);
+      }
+#pragma unroll
+      for (int j = 0; j < WPIECES; ++j) {
+        if (conv) store_piece(Set{}, Stage{}, tail_tag, TxSet{}, j);
+        __builtin_amdgcn_sched_barrier(0);
+        wreg[Set::value][j].load_async(waddr[j], ktw);
+#pragma unroll
+        for (int i = 2 * j; i < 2 * j + 2; ++i)
+          vm_load16_to_lds(xsrc, xoff[i], x_lds0 + (uint32_t)((XS * XSTAGE + 32 * i * BIG_LS) * 2));
+        __builtin_amdgcn_sched_barrier(0);
+      }
       if constexpr (TAIL) load_tx(TxSet{}, min(kt + 3, last));
-      load_x(WsInt<(R + 2) % 3>{}, min(kt + 2, last));
-      load_w(Set{}, min(kt + 4, last));
-      vm_wait<2 * WLOADS + XLOADS + TLOADS>();
+      vm_wait<WLOADS + XLOADS + TLOADS>();
       __syncthreads();
     };
     auto run = [&](auto tail_tag) {
