@@ -322,29 +322,49 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     __builtin_amdgcn_sched_group_barrier(0x008, 2 * NTJ, 0);
   };
   __syncthreads();  // first stage filled
-  auto k_loop = [&](auto ntj_tag) {
+  // The two consumers of a SIMD share its matrix pipe, and the SIMD issues the older wavefront's instruction whenever both
+  // have one ready: left alone, wavefronts 0-3 run at the pace their own operand reads allow (about 1500 cycles for the
+  // 1024 cycles of MFMAs of a K step), wavefronts 4-7 only fill the gaps and then run the rest of their step alone, where
+  // nobody covers their waits for LDS (2500 cycles; every barrier waits for them).  Issue priorities hand the pipe over in
+  // the middle of the step instead: the first group runs its first K half above the second group and its second K half
+  // below it, so each group has one half in which it is served first and one in which it fills the other's gaps, and both
+  // reach the barrier within a few hundred cycles of each other (2575 instead of 2680 cycles per step).  The priority
+  // changes sit between the two halves, outside the pinned MFMA / LDS-read sequences; a change inside one (after 40-48 of
+  // the 64 MFMAs, nearer the balance point) disturbs that order and gains nothing.
+  auto k_loop = [&](auto ntj_tag, auto group_tag) {
+    constexpr bool FIRST = decltype(group_tag)::value == 0;
+    if (!FIRST) __builtin_amdgcn_s_setprio(1);
     int xs = 0;
     for (int kt = 0; kt < nkt; kt += 2) {
+      if (FIRST) __builtin_amdgcn_s_setprio(2);
       compute(WsInt<0>{}, ntj_tag, xs, 0);
+      if (FIRST) __builtin_amdgcn_s_setprio(0);
       compute(WsInt<0>{}, ntj_tag, xs, 1);
       __syncthreads();
       xs = xs == 2 ? 0 : xs + 1;
       if (kt + 1 < nkt) {
+        if (FIRST) __builtin_amdgcn_s_setprio(2);
         compute(WsInt<1>{}, ntj_tag, xs, 0);
+        if (FIRST) __builtin_amdgcn_s_setprio(0);
         compute(WsInt<1>{}, ntj_tag, xs, 1);
         __syncthreads();
         xs = xs == 2 ? 0 : xs + 1;
       }
     }
+    __builtin_amdgcn_s_setprio(0);
+  };
+  auto k_loop_of_group = [&](auto ntj_tag) {
+    if (wave < 4) k_loop(ntj_tag, WsInt<0>{});
+    else k_loop(ntj_tag, WsInt<1>{});
   };
   if (!active) {
     for (int kt = 0; kt < nkt; ++kt) __syncthreads();
   } else if (ntj == 1) {
-    k_loop(WsInt<1>{});
+    k_loop_of_group(WsInt<1>{});
   } else if (ntj == 2) {
-    k_loop(WsInt<2>{});
+    k_loop_of_group(WsInt<2>{});
   } else {
-    k_loop(WsInt<4>{});
+    k_loop_of_group(WsInt<4>{});
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------------
