@@ -209,6 +209,26 @@ __device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_t
   }
   return big_unit(p, lane_off, BM, n_tiles, pl, unit, t, absorb);
 }
+// Item j of an XCD's work list: the whole units first, then the chunks of the split ones (the same numbering as the
+// workgroup index j of big_tile_id), from a plan and offsets fetched once: for workgroups that walk several items.
+__device__ __forceinline__ bool big_item(const GemmParams& p, int lane_off, int BM, int n_tiles, const BigPlan& pl, int xcd, int j, BigTile& t,
+                                         bool absorb = false) {
+  int unit;
+  if (j < pl.whole) {
+    unit = j;
+    t.chunk = 0;
+    t.nchunks = 1;
+    t.chunk_slot = 0;
+  } else {
+    const int c = j - pl.whole;
+    if (c >= pl.rest * pl.chunks) return false;
+    unit = pl.whole + c / pl.chunks;
+    t.chunk = c % pl.chunks;
+    t.nchunks = pl.chunks;
+    t.chunk_slot = xcd * kBigChunkSlotsPerXcd + c;
+  }
+  return big_unit(p, lane_off, BM, n_tiles, pl, unit, t, absorb);
+}
 // Grid size that covers every XCD's share for at most `slots_bound` token tiles (a split adds up to 24 workgroups).
 static inline int big_grid(int n_tiles, int slots_bound, bool allow_split) {
   return 8 * ((n_tiles * slots_bound + 7) / 8 + 2 + (allow_split ? 24 : 0));

@@ -24,21 +24,66 @@ namespace stmoe {
 
 template <int V> struct WsInt { static constexpr int value = V; };
 
+// Token of pair id `pair` = pair / k_top; the usual top-k values without the 40 instructions of an integer division.
+__device__ __forceinline__ int pair_token(int pair, int k_top) {
+  if (k_top == 1) return pair;
+  if (k_top == 2) return pair >> 1;
+  if (k_top == 4) return pair >> 2;
+  if (k_top == 8) return pair >> 3;
+  return pair / k_top;
+}
+
+struct WsArgs {
+  GemmParams p;
+  int n_tiles;
+  int wgs_per_xcd;  // grid size / 8
+  float* partial;
+};
+
 template <typename T, int WF, int MODE>
 __global__ void __launch_bounds__(768, 1)
-grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
+grouped_mfma_ws_kernel(WsArgs args) {
   constexpr int BN = 256, BM = 256;
   constexpr int WSTAGE = BN * BIG_LS, XSTAGE = BM * BIG_LS;  // elements
   constexpr int WPIECES = 4;   // packed weight pieces per producer per K step (16 row tiles / 4 producers)
   constexpr int XLOADS = 8;    // direct token loads per producer per K step (32 blocks of 8 rows / 4 producers)
   constexpr int WLOADS = BigPiece<WF>::LOADS * WPIECES;
   extern __shared__ __align__(16) uint16_t lds[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for all lanes: everything derived from it can live in scalar registers
-  const int g = lane >> 4, n_in = lane & 15;
 
+  // A workgroup walks its XCD's work list: item `wg`, then every (workgroups per XCD)-th one after it, shifted by half a
+  // round in odd rounds (in a block of 32 units the first half belongs to an expert's first token tile, the second half to
+  // its second; ride-along rows mostly sit on the first, and a workgroup that always drew the same half would collect
+  // them).  The loaders of a unit are done one K step before the consumers and then start the next unit (tile lookup,
+  // gather offsets, first loads and conversion) while the consumers still multiply and store: all of LDS is free after the
+  // last barrier of a unit.
+  // Carried from unit to unit: the round number, this wavefront's index and the experts' row offsets (one per lane).
+  // Everything else a unit needs, the plan of the XCD's list included, is derived again inside the loop from values the
+  // compiler cannot see through (an opaque zero, the opaque address of the kernel arguments): otherwise it computes the
+  // loop-invariant part of every unit's set-up once, in front of the loop, and keeps some hundred values alive through the
+  // K loops, whose registers are all taken.
+  const int wave_id = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int offsets_by_lane = big_lane_offsets(args.p);
+  for (int round = 0;; ++round) {
+  int zero = 0, wave = wave_id, lane_off = offsets_by_lane;
+  asm volatile("" : "+s"(zero), "+s"(wave), "+v"(lane_off));
+  const int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, (unsigned)zero));
+  const int tid = wave * 64 + lane;
+  // A unit's set-up by the loaders (tile lookup, gather offsets, first loads, first conversion) is what its consumers wait
+  // for, while the consumers of the previous unit still multiply and store: the loaders go first at the issue stage.
+  if (wave >= 8) __builtin_amdgcn_s_setprio(3);
+  const int g = lane >> 4, n_in = lane & 15;
+  auto kernarg = __builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(kernarg));
+  const WsArgs& ka = *reinterpret_cast<const WsArgs*>((const void*)kernarg);
+  const GemmParams& p = ka.p;
+  const int n_tiles = ka.n_tiles;
+  float* const partial = ka.partial;
+  const int xcd = blockIdx.x & 7, wg = blockIdx.x >> 3, wgs = ka.wgs_per_xcd;
+  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, partial != nullptr, true);
+  int slot = wg + (round & 1) * (wgs >> 1);
+  if (slot >= wgs) slot -= wgs;
   BigTile tile;
-  if (!big_tile_id(p, BM, n_tiles, partial != nullptr, tile, true)) return;
+  if (!big_item(p, lane_off, BM, n_tiles, pl, xcd, round * wgs + slot, tile, true)) return;
   const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
   // Rows per token-row group: the rows of a partial tile are spread evenly (in multiples of 16) over the four groups,
@@ -81,7 +126,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
       const int lr = pw * 8 + 32 * j + (lane >> 3);
       const int r = min((lr >> 6) * rpg + min(lr & 63, rpg - 1), rows_here - 1);
       const int i = row_begin + r;
-      const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
+      const int64_t src = p.perm ? (int64_t)pair_token(p.perm[i], p.k_top) : (int64_t)i;
       xoff[j] = (uint32_t)((src * p.lda + (((lane & 7) ^ (lr & 7)) << 3)) * 2);
     }
     const uint32_t lds_addr0 = (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)lds);
@@ -98,7 +143,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     uint32_t toff = 0;
     if (tile.tail_rows > 0) {
       const int i = tile.tail_begin + min(n_in, tile.tail_rows - 1);
-      const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
+      const int64_t src = p.perm ? (int64_t)pair_token(p.perm[i], p.k_top) : (int64_t)i;
       toff = (uint32_t)((src * p.lda + g * 16) * 2);
     }
     u32x4_t tx[2][2];  // [register set = K step % 2][half of the lane's 16 elements]
@@ -204,17 +249,16 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     auto run = [&](auto tail_tag) {
       constexpr bool TAIL = decltype(tail_tag)::value != 0;
       constexpr int TLOADS = TAIL ? 2 : 0;
-      if constexpr (TAIL) {
-        load_tx(WsInt<0>{}, 0);
-        load_tx(WsInt<1>{}, min(1, last));
-      }
+      // what step 0 waits for goes first: a unit's first requests queue behind each other for the CU's one vector-memory path
+      if constexpr (TAIL) load_tx(WsInt<0>{}, 0);
       load_w(WsInt<0>{}, 0);
-      load_w(WsInt<1>{}, min(1, last));
       load_x(WsInt<0>{}, 0);
-      load_w(WsInt<2>{}, min(2, last));
+      if constexpr (TAIL) load_tx(WsInt<1>{}, min(1, last));
+      load_w(WsInt<1>{}, min(1, last));
       load_x(WsInt<1>{}, min(1, last));
-      // the weights of step 0 (and the tail operands of steps 0, 1) are older than everything else issued so far
-      vm_wait<2 * WLOADS + 2 * XLOADS>();
+      load_w(WsInt<2>{}, min(2, last));
+      // the weights of step 0 (and the tail operands of step 0) are older than everything else issued so far
+      vm_wait<2 * WLOADS + 2 * XLOADS + TLOADS>();
       store_w(WsInt<0>{}, WsInt<0>{}, tail_tag, WsInt<0>{});
       if constexpr (TAIL) load_tx(WsInt<0>{}, min(2, last));
       load_w(WsInt<0>{}, min(3, last));
@@ -223,6 +267,10 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
       // step 1 and the tail operands of step 2
       vm_wait<2 * WLOADS + XLOADS + TLOADS>();
       __syncthreads();
+      // With a tail the loaders carry 8 MFMAs per K step on top of their conversions and are the wavefronts every step
+      // waits for; served first at the issue stage they lose less time to the consumers' instructions (measured:
+      // tail-carrying tiles 4 % faster; without a tail a raised priority made the consumers 2-4 % slower).
+      __builtin_amdgcn_s_setprio(TAIL ? 2 : 0);
       for (int kt = 0;; kt += 6) {
         k_step(WsInt<0>{}, tail_tag, kt);
         if (kt + 1 >= nkt) break;
@@ -241,12 +289,8 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
     };
     if (tile.tail_rows == 0) {
       run(WsInt<0>{});
-      return;
+      continue;
     }
-    // With a tail the producers carry 8 MFMAs per K step on top of their conversions and are the wavefronts every step waits
-    // for; given priority at the issue stage they lose less time to the consumers' instructions (measured: tail-carrying
-    // tiles 4 % faster; without a tail a higher priority made the consumers 2-4 % slower and is left alone).
-    __builtin_amdgcn_s_setprio(2);
     run(WsInt<1>{});
     // ---- the tail's results: lane (n_in, g) holds, for token row tail_begin + n_in, features 4 g .. 4 g + 3 of each block
     if (n_in < tile.tail_rows) {
@@ -272,7 +316,8 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
               make_uint2(pack2<T>(tacc[bi][0], tacc[bi][1]), pack2<T>(tacc[bi][2], tacc[bi][3]));
       }
     }
-    return;
+    __builtin_amdgcn_s_setprio(0);
+    continue;
   }
 
   // =================================== consumer ===================================
@@ -414,6 +459,7 @@ grouped_mfma_ws_kernel(GemmParams p, int n_tiles, float* partial) {
       }
     }
   }
+  }  // next item
 }
 
 // Adds the chunks of every split unit in chunk order and writes the rows: DOWN: the sums; GATEUP: the gated product of
@@ -472,7 +518,9 @@ static int launch_ws_m(const GemmParams& p, int64_t max_rows, float* partial, hi
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;
-  kern<<<dim3((unsigned)big_grid(n_tiles, m_slots, partial != nullptr)), 768, lds_bytes, st>>>(p, n_tiles, partial);
+  // one workgroup per CU (it takes all of the CU's LDS), fewer when an XCD's list cannot be longer than that
+  const int per_xcd = std::min(kBigCusPerXcd, big_grid(n_tiles, m_slots, partial != nullptr) / 8);
+  kern<<<dim3((unsigned)(8 * per_xcd)), 768, lds_bytes, st>>>(WsArgs{p, n_tiles, per_xcd, partial});
   int rc = check_launch("grouped_mfma_ws");
   if (rc || !partial) return rc;
   big_reduce_kernel<T, MODE><<<dim3(8 * 16, (BM + kBigTailRows + 31) / 32), 256, 0, st>>>(p, n_tiles, partial);
