@@ -379,6 +379,7 @@ def main():
     ap.add_argument("--decode-tokens", type=int, default=32)
     ap.add_argument("--cpu-sample", type=int, default=16, help="tokens timed on the CPU baseline (0 to skip)")
     ap.add_argument("--no-configs", action="store_true", help="skip the legs of the other BASELINE configurations")
+    ap.add_argument("--no-probe", action="store_true", help="skip the matrix-core ceiling probe")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (5 times) so that rocprofv3 FETCH_SIZE/WRITE_SIZE readings "
                          "of the kernels can be scaled by what the same counters read for a copy of known size")
@@ -425,6 +426,22 @@ def main():
                      "algorithmic_unit": "expert-weight bytes per launch"},
     }
 
+    # What the matrix cores of this very machine sustain on nothing but MFMA instructions (the chip lowers its clock with
+    # their activity and with the switching of the operand bits): the practical ceiling beside the data-sheet one.
+    probe = None
+    if not args.no_probe:
+        from sharktank_amd import _hip
+
+        probe = {
+            "f16_random_operands_TFLOPs": round(_hip.probe_mfma(dev, 0, True), 1),
+            "f16_constant_operands_TFLOPs": round(_hip.probe_mfma(dev, 0, False), 1),
+            "fp8_random_operands_TFLOPs": round(_hip.probe_mfma(dev, 1, True), 1),
+            "fp8_constant_operands_TFLOPs": round(_hip.probe_mfma(dev, 1, False), 1),
+            "what": "256 workgroups x 8 wavefronts of independent v_mfma_f32_16x16x32_f16 / v_mfma_scale_f32_32x32x64_f8f6f4 "
+                    "on register operands; 8 timed launches of 20000 loop passes after 12 untimed ones",
+        }
+        roofline["frac_of_mfma_only_probe"] = round(achieved / probe["f16_random_operands_TFLOPs"], 4)
+
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -455,7 +472,7 @@ def main():
         "layer_tflops": round(layer_flops / (ms * 1e-3) / 1e12, 2),
         "e2e_ms_per_step": round(e2e_ms, 4),
         "stage_ms": {k: round(v, 4) for k, v in st.items()},
-        "roofline": roofline, "decode": decode, "cpu_baseline": cpu, "configs": configs,
+        "roofline": roofline, "mfma_only_probe": probe, "decode": decode, "cpu_baseline": cpu, "configs": configs,
     }
     print(json.dumps(line))
 

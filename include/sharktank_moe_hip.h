@@ -287,6 +287,15 @@ int stmoe_moe_forward_static(const void* h, int dtype, int64_t T, int64_t K, int
                              const float* z_scale /*nullable*/, void* out, int32_t* idx_out, void* gate_out,
                              int variant, stmoe_stream_t stream);
 
+/* Measurement aid, no counterpart in the reference: one launch of nothing but independent matrix-core instructions on
+ * operands held in registers (kind 0: v_mfma_f32_16x16x32_f16, kind 1: v_mfma_scale_f32_32x32x64_f8f6f4 on e4m3 bytes;
+ * random_operands 0: constant bits, 1: hashed bits), 2 wavefronts per SIMD on 256 CUs, `iters` (a multiple of 4) loop
+ * passes.  *flop (host, nullable) receives the floating-point operations of the launch; the caller times it.  The chip
+ * lowers its clock with the matrix cores' activity and with the switching of the operand bits, so this rate, not the
+ * data-sheet one, is what a matrix-core-bound kernel can approach on this machine.  `sink`: 4 writable device bytes. */
+int stmoe_probe_mfma(int kind, int random_operands, int iters, float* sink, double* flop /*host, nullable*/,
+                     stmoe_stream_t stream);
+
 /* x @ W^T for one quantised (or dense) matrix W [rows, cols]: the operand set of the reference's
  * `mmt_block_scaled_q8(a,d,qs)` (sharktank/sharktank/kernels/mmt_block_scaled_q8.py:30) and
  * `mmt_block_scaled_offset_q4_unsigned(a,d,qs,m)` (mmt_block_scaled_offset_q4.py:31), reached from

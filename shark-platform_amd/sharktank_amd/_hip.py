@@ -102,6 +102,7 @@ SIGNATURES = {
                                          POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_int, c_void_p]),
     "stmoe_mmt": (c_int, [c_void_p, c_int, c_int64, POINTER(StmoeWeight), c_void_p, c_int, c_void_p]),
+    "stmoe_probe_mfma": (c_int, [c_int, c_int, c_int, c_void_p, POINTER(ctypes.c_double), c_void_p]),
 }
 STATIC_SCRATCH_BYTES = 16 << 20  # STMOE_STATIC_SCRATCH_BYTES
 
@@ -616,3 +617,24 @@ def mmt(a: torch.Tensor, w: DeviceWeight, *, variant: int = VARIANT_AUTO) -> tor
     with torch.cuda.device(dev):
         _check(lib.stmoe_mmt(_ptr(a_c), dtype_enum(a_c.dtype), M, w.ref, _ptr(out), variant, _stream(dev)))
     return out
+
+
+def probe_mfma(device, kind: int = 0, random_operands: bool = True, iters: int = 20000, launches: int = 8,
+               warm_launches: int = 12) -> float:
+    """TFLOP/s of launches of nothing but independent matrix-core instructions (stmoe_probe_mfma; kind 0: fp16, 1: fp8),
+    timed with events on the current stream.  The untimed launches in front (some tens of milliseconds) let the chip's
+    power management settle: a short burst after idle runs at a clock the chip does not hold."""
+    lib = load_library()
+    dev = torch.device(device)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    flop = ctypes.c_double(0.0)
+    with torch.cuda.device(dev):
+        for _ in range(warm_launches):
+            _check(lib.stmoe_probe_mfma(kind, int(random_operands), iters, _ptr(sink), None, _stream(dev)))
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(launches):
+            _check(lib.stmoe_probe_mfma(kind, int(random_operands), iters, _ptr(sink), ctypes.byref(flop), _stream(dev)))
+        stop.record()
+        stop.synchronize()
+    return launches * flop.value / (start.elapsed_time(stop) * 1e-3) / 1e12
