@@ -1,23 +1,28 @@
-// Prefill kernel with specialised wavefronts: 256 x 256 workgroup tile, 8 consumer + 4 producer wavefronts.
+// Prefill kernel with specialised wavefronts: 256 weight rows x 256 token rows per unit, one workgroup of 12 wavefronts
+// per CU that walks its XCD's list of units.
 //
+//   units of 129..256 token rows: 8 consumer + 4 loader wavefronts
 //   consumers (wavefronts 0-7: 2 weight-row halves x 4 token-row groups): 128 weight rows x 64 token rows each (GATEUP: 64 gate + the same 64 up rows);
 //             a K step is nothing but LDS operand reads and 64 MFMAs, so both consumers of a SIMD keep the matrix
 //             pipe fed all the time
-//   producers (wavefronts 8-11, one per SIMD): per K step each loads 4 packed 1 KB weight pieces into registers
-//             (three K steps before they are needed), dequantises them and writes 16-bit rows into the next weight
+//   loaders   (wavefronts 8-11, one per SIMD): per K step each loads 4 packed 1 KB weight pieces into registers
+//             (four K steps before they are needed), dequantises them and writes 16-bit rows into the next weight
 //             stage, and issues 8 direct global->LDS loads of token rows (two K steps ahead)
+//   units of at most 128 token rows: 4 consumers (wavefronts 0-3, one per SIMD, the same 128 x 64 each) + 8 loaders
+//             (wavefronts 4-11, two weight pieces and two token loads each): such a unit still converts its whole weight slab
+//             while its consumers have half the work, and four loaders cannot convert faster than in 2200 cycles per K step
 //   LDS (160 KB): 2 weight stages + 3 token stages of 32 KB, rows of 128 bytes XOR-swizzled in 16-byte units;
 //             one barrier per K step
 //   registers: 12 wavefronts leave 168 per lane; the consumers hold 128 accumulators and 20 operand registers
 //
 //   tails:    a full token tile may take up to 16 more rows of its expert along (an absorbed tail, see big_tail_absorbed):
-//             the four producers multiply those rows themselves, each against 64 of the tile's 256 weight rows, with the
+//             the four loaders multiply those rows themselves, each against 64 of the tile's 256 weight rows, with the
 //             weight operands taken from the registers they have just converted and the token operands straight from
-//             global memory (two K steps ahead, two register sets); 8 MFMAs per producer and K step, no LDS traffic
+//             global memory (two K steps ahead, two register sets); 8 MFMAs per loader and K step, no LDS traffic
 //
-// All loads of the producers are inline assembly with a wave-uniform base in scalar registers and are awaited by hand
-// (see ffn_mfma_common.h); per K step a producer issues the tail's token loads (if any), then XLOADS token loads, then
-// WLOADS weight loads, always in this order and always all of them.
+// All loads of the loaders are inline assembly with a wave-uniform base in scalar registers and are awaited by hand
+// (see ffn_mfma_common.h); per K step a loader issues, piece by piece, WLOADS weight loads and XLOADS token loads, then
+// the tail's token loads (if any), always in this order and always all of them.
 #include "ffn_mfma_common.h"
 
 namespace stmoe {
@@ -45,9 +50,6 @@ __global__ void __launch_bounds__(768, 1)
 grouped_mfma_ws_kernel(WsArgs args) {
   constexpr int BN = 256, BM = 256;
   constexpr int WSTAGE = BN * BIG_LS, XSTAGE = BM * BIG_LS;  // elements
-  constexpr int WPIECES = 4;   // packed weight pieces per producer per K step (16 row tiles / 4 producers)
-  constexpr int XLOADS = 8;    // direct token loads per producer per K step (32 blocks of 8 rows / 4 producers)
-  constexpr int WLOADS = BigPiece<WF>::LOADS * WPIECES;
   extern __shared__ __align__(16) uint16_t lds[];
 
   // A workgroup walks its XCD's work list: item `wg`, then every (workgroups per XCD)-th one after it, shifted by half a
@@ -61,6 +63,12 @@ grouped_mfma_ws_kernel(WsArgs args) {
   // compiler cannot see through (an opaque zero, the opaque address of the kernel arguments): otherwise it computes the
   // loop-invariant part of every unit's set-up once, in front of the loop, and keeps some hundred values alive through the
   // K loops, whose registers are all taken.
+  // Two shapes of unit.  FULL (129..256 token rows): wavefronts 0-7 consume, 8-11 load.  HALF (at most 128 token rows): the
+  // consumers' work is halved but a unit still streams and converts its whole 256 x K weight slab, which four loaders
+  // cannot do faster than in 2200 cycles per K step; so wavefronts 0-3 consume (one per SIMD, 128 weight rows x 64 token
+  // rows each, as in FULL) and wavefronts 4-11 load, two weight pieces each instead of four.  A wavefront's role can
+  // change from unit to unit (4-7), which costs nothing: every unit starts from scratch and every wavefront owns the same
+  // 168 registers.
   const int wave_id = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int offsets_by_lane = big_lane_offsets(args.p);
   for (int round = 0;; ++round) {
@@ -80,50 +88,67 @@ grouped_mfma_ws_kernel(WsArgs args) {
   float* const partial = ka.partial;
   const int xcd = blockIdx.x & 7, wg = blockIdx.x >> 3, wgs = ka.wgs_per_xcd;
   const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, partial != nullptr, true);
-  int slot = wg + (round & 1) * (wgs >> 1);
-  if (slot >= wgs) slot -= wgs;
+  // Which item of round `round` (wgs consecutive items of the XCD's list) this workgroup takes: its own index shifted
+  // by half a round plus one per round.  Neighbouring items differ systematically in cost (in a block of 32 full units the
+  // first half belongs to an expert's first token tile, which carries most ride-along rows; partial units cycle through
+  // the experts, some of which have 30 rows and some 250), and a workgroup that drew the same place in every round would
+  // collect one kind: the launch ends when the slowest workgroup does.
+  const int slot = (wg + round * ((wgs >> 1) + 1)) % wgs;
   BigTile tile;
   if (!big_item(p, lane_off, BM, n_tiles, pl, xcd, round * wgs + slot, tile, true)) return;
   const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
-  // Rows per token-row group: the rows of a partial tile are spread evenly (in multiples of 16) over the four groups,
-  // so all consumers share the work and each only multiplies the 16-row column blocks it really has.  Tile row
-  // grp * rpg + i (i < rpg) lives in LDS row grp * 64 + i.  Full tiles: rpg = 64, the identity.
-  const int rpg = min(64, ((rows_here + 3) / 4 + 15) / 16 * 16);
   // this workgroup's K steps: all of them, or one chunk of a split unit
   const int kt0 = (int)((p.kred >> 6) * tile.chunk / tile.nchunks);
   const int nkt = (int)((p.kred >> 6) * (tile.chunk + 1) / tile.nchunks) - kt0;
+
+  auto unit = [&](auto loader_tag, auto half_tag) {
+  constexpr bool LOADER = decltype(loader_tag)::value != 0;
+  constexpr bool HALF = decltype(half_tag)::value != 0;
+  constexpr int NLOADERS = HALF ? 8 : 4;
+  constexpr int WPIECES = 16 / NLOADERS;                     // packed 16-row weight pieces per loader and K step
+  constexpr int XLOADS = (HALF ? 16 : 32) / NLOADERS;        // direct token loads (8 rows each) per loader and K step
+  constexpr int XPER = XLOADS / WPIECES;                     // token loads issued after each piece
+  constexpr int XROWS = 8 * NLOADERS;                        // LDS rows between a loader's consecutive token loads
+  constexpr int GROUPS = HALF ? 2 : 4;                       // token-row groups of 64 LDS rows
+  constexpr int WLOADS = BigPiece<WF>::LOADS * WPIECES;
+  if constexpr (LOADER) __builtin_amdgcn_s_setprio(3);  // (wavefronts 4-7, which learn their role only here)
+  // Rows per token-row group: the rows of a partial tile are spread evenly (in multiples of 16) over the groups, so all
+  // consumers share the work and each only multiplies the 16-row column blocks it really has.  Tile row
+  // grp * rpg + i (i < rpg) lives in LDS row grp * 64 + i.  Full tiles: rpg = 64, the identity.
+  const int rpg = min(64, ((rows_here + GROUPS - 1) / GROUPS + 15) / 16 * 16);
 
   uint16_t* const Wbase = lds;               // [2][BN][64]
   uint16_t* const Xbase = lds + 2 * WSTAGE;  // [3][BM][64]
   const int sw = n_in & 7;
 
-  if (wave >= 8) {
+  if constexpr (LOADER) {
     // =================================== producer ===================================
-    const int pw = wave - 8;
-    // This producer's four 16-row weight blocks, as rows of the workgroup tile: GATEUP: gate blocks 2 pw, 2 pw + 1 and the up
-    // blocks of the same features (so that an absorbed tail's gate and up sums meet in one lane); DOWN: blocks 4 pw .. 4 pw + 3
-    auto piece_row = [&](int j) { return MODE == MODE_GATEUP ? (j < 2 ? 0 : BN / 2) + (2 * pw + (j & 1)) * 16 : (4 * pw + j) * 16; };
+    const int pw = wave - (HALF ? 4 : 8);
+    // This loader's 16-row weight blocks, as rows of the workgroup tile.  GATEUP: WPIECES / 2 gate blocks and the up blocks
+    // of the same features (so that an absorbed tail's gate and up sums meet in one lane); DOWN: WPIECES blocks in a row.
+    auto piece_block = [&](int j) { return MODE == MODE_GATEUP ? (WPIECES / 2) * pw + j % (WPIECES / 2) : WPIECES * pw + j; };
+    auto piece_row = [&](int j) { return (MODE == MODE_GATEUP && j >= WPIECES / 2 ? BN / 2 : 0) + piece_block(j) * 16; };
     BigAddr<WF> waddr[WPIECES];
 #pragma unroll
     for (int j = 0; j < WPIECES; ++j) {
       int64_t row0;
       const WeightView* wv;
       if (MODE == MODE_GATEUP) {
-        wv = j >= 2 ? &p.w1 : &p.w0;
-        row0 = (int64_t)e * wv->rows + (int64_t)ntile * (BN / 2) + (2 * pw + (j & 1)) * 16;
+        wv = j >= WPIECES / 2 ? &p.w1 : &p.w0;
+        row0 = (int64_t)e * wv->rows + (int64_t)ntile * (BN / 2) + piece_block(j) * 16;
       } else {
         wv = &p.w0;
         row0 = (int64_t)e * wv->rows + (int64_t)ntile * BN + piece_row(j);
       }
       waddr[j].init(*wv, row0 >> 4, e, lane, p.kred);
     }
-    // token rows: lane l of direct load j fills LDS row pw*8 + 32*j + l/8, unit l%8, from global unit (l%8) ^ (row & 7);
+    // token rows: lane l of direct load j fills LDS row pw*8 + XROWS*j + l/8, unit l%8, from global unit (l%8) ^ (row & 7);
     // LDS rows that hold no tile row re-read a valid row (their outputs are never stored)
     uint32_t xoff[XLOADS];
 #pragma unroll
     for (int j = 0; j < XLOADS; ++j) {
-      const int lr = pw * 8 + 32 * j + (lane >> 3);
+      const int lr = pw * 8 + XROWS * j + (lane >> 3);
       const int r = min((lr >> 6) * rpg + min(lr & 63, rpg - 1), rows_here - 1);
       const int i = row_begin + r;
       const int64_t src = p.perm ? (int64_t)pair_token(p.perm[i], p.k_top) : (int64_t)i;
@@ -189,7 +214,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
       const char* xsrc = reinterpret_cast<const char*>(p.a) + (kt0 + kt) * (BIG_BK * 2);  // the step's columns: a scalar add
 #pragma unroll
       for (int j = 0; j < XLOADS; ++j)
-        vm_load16_to_lds(xsrc, xoff[j], x_lds0 + (uint32_t)((XS * XSTAGE + 32 * j * BIG_LS) * 2));
+        vm_load16_to_lds(xsrc, xoff[j], x_lds0 + (uint32_t)((XS * XSTAGE + XROWS * j * BIG_LS) * 2));
     };
     auto load_tx = [&](auto set_tag, int kt) {
       constexpr int SET = decltype(set_tag)::value;
@@ -238,8 +263,8 @@ grouped_mfma_ws_kernel(WsArgs args) {
         __builtin_amdgcn_sched_barrier(0);
         wreg[Set::value][j].load_async(waddr[j], ktw);
 #pragma unroll
-        for (int i = 2 * j; i < 2 * j + 2; ++i)
-          vm_load16_to_lds(xsrc, xoff[i], x_lds0 + (uint32_t)((XS * XSTAGE + 32 * i * BIG_LS) * 2));
+        for (int i = XPER * j; i < XPER * j + XPER; ++i)
+          vm_load16_to_lds(xsrc, xoff[i], x_lds0 + (uint32_t)((XS * XSTAGE + XROWS * i * BIG_LS) * 2));
         __builtin_amdgcn_sched_barrier(0);
       }
       if constexpr (TAIL) load_tx(TxSet{}, min(kt + 3, last));
@@ -287,10 +312,11 @@ grouped_mfma_ws_kernel(WsArgs args) {
       }
       vm_wait<0>();  // the requests past the last step: nothing may land in registers or LDS after this wavefront is done
     };
-    if (tile.tail_rows == 0) {
+    if (HALF || tile.tail_rows == 0) {
       run(WsInt<0>{});
-      continue;
+      return;
     }
+    if constexpr (!HALF) {
     run(WsInt<1>{});
     // ---- the tail's results: lane (n_in, g) holds, for token row tail_begin + n_in, features 4 g .. 4 g + 3 of each block
     if (n_in < tile.tail_rows) {
@@ -317,12 +343,12 @@ grouped_mfma_ws_kernel(WsArgs args) {
       }
     }
     __builtin_amdgcn_s_setprio(0);
-    continue;
-  }
-
+    }  // !HALF
+  } else {
   // =================================== consumer ===================================
   // Wavefront w runs on SIMD w % 4.  Token-row groups (wm) are spread so that a partial tile, where only the first
-  // groups have rows, still uses several SIMDs: wm 0 -> SIMDs 0,1; wm 1 -> SIMDs 2,3; wm 2 -> 0,1; wm 3 -> 2,3.
+  // groups have rows, still uses several SIMDs: wm 0 -> SIMDs 0,1; wm 1 -> SIMDs 2,3; wm 2 -> 0,1; wm 3 -> 2,3 (HALF: two
+  // groups, wm 0 -> SIMDs 0,1; wm 1 -> 2,3).
   const int wn = wave & 1, wm = wave >> 1;
   const uint16_t* a_rd[2];  // K half ks: weight row (wavefront base + n_in), unit ks*4 + g
   const uint16_t* b_rd[2];
@@ -398,8 +424,10 @@ grouped_mfma_ws_kernel(WsArgs args) {
     }
     __builtin_amdgcn_s_setprio(0);
   };
+  // HALF: one consumer per SIMD, nothing to hand over; it stays above the two loaders it shares the SIMD with.
   auto k_loop_of_group = [&](auto ntj_tag) {
-    if (wave < 4) k_loop(ntj_tag, WsInt<0>{});
+    if constexpr (HALF) k_loop(ntj_tag, WsInt<1>{});
+    else if (wave < 4) k_loop(ntj_tag, WsInt<0>{});
     else k_loop(ntj_tag, WsInt<1>{});
   };
   if (!active) {
@@ -458,6 +486,15 @@ grouped_mfma_ws_kernel(WsArgs args) {
               make_uint2(pack2<T>(acc[ti][tj][0], acc[ti][tj][1]), pack2<T>(acc[ti][tj][2], acc[ti][tj][3]));
       }
     }
+  }
+  }  // consumer
+  };  // unit
+  if (rows_here <= BM / 2) {
+    if (wave < 4) unit(WsInt<0>{}, WsInt<1>{});
+    else unit(WsInt<1>{}, WsInt<1>{});
+  } else {
+    if (wave < 8) unit(WsInt<0>{}, WsInt<0>{});
+    else unit(WsInt<1>{}, WsInt<0>{});
   }
   }  // next item
 }

@@ -204,12 +204,14 @@ def _routing_with_rows(rows, T, k, seed):
 @pytest.mark.parametrize("rows", [
     [261, 517, 512 + 32, 512 + 33, 256 + 16, 256 + 17, 300, 122],  # absorbed: 5, 5, 32 (two tiles x 16), 16; not: 33, 17
     [768 + 48, 768 + 1, 256, 255, 1, 0, 270, 257],                  # three full tiles x 16; one-row tails; an expert without rows
+    [128, 129, 127, 1, 18, 64, 256 + 128, 256 + 129],               # token tiles of at most 128 rows (8 loaders, 4 consumers) and both sides of that limit
 ])
 def test_prefill_tails_that_ride_along_with_full_token_tiles(device, fmt, dtype, rows):
     """Row counts a few rows above a multiple of 256: the prefill kernel lets every full token tile of such an expert take up
     to 16 of the extra rows along (computed by its loader wavefronts) instead of running a partial token tile for them.
-    Every output row is checked against the oracle, the tail rows also on their own, and the whole result against the
-    vector-ALU kernel."""
+    Token tiles of at most 128 rows run with eight loader and four consumer wavefronts instead of four and eight.
+    Every output row is checked against the oracle, every expert's rows and the tail rows also on their own, and the whole
+    result against the vector-ALU kernel."""
     from sharktank_amd import _hip as hip
     from sharktank_amd.ops import device_weight
 
@@ -239,6 +241,10 @@ def test_prefill_tails_that_ride_along_with_full_token_tiles(device, fmt, dtype,
     assert O.rel_l2(got, want) < tol
     for e in range(E):
         r = rows[e]
+        if r > 0:
+            a, b = int(off_c[e]), int(off_c[e + 1])
+            err = O.rel_l2(got[a:b], want[a:b])
+            assert err < 2 * tol, f"expert {e} ({r} rows): rel-L2 {err:.3e}"
         c, t = r // 256, r % 256
         if c >= 1 and 0 < t <= 16 * c:  # an absorbed tail: its rows on their own
             a, b = int(off_c[e]) + c * 256, int(off_c[e + 1])
