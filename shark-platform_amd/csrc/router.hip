@@ -187,8 +187,8 @@ struct SingleTokenDispatch {
   int32_t *counts, *offsets, *perm, *inv;
 };
 
-template <typename T, typename W, bool FUSE_NORM>
-__global__ void __launch_bounds__(512)
+template <typename T, typename W, bool FUSE_NORM, int PRE>
+__global__ void __launch_bounds__(512, PRE ? 4 : 8)
 router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float eps, T* __restrict__ xn,
                  const T* __restrict__ wr, int64_t K, int E, int k, T* __restrict__ logits_out,
                  int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out, T* __restrict__ gate_out,
@@ -205,11 +205,12 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
   // latency runs in parallel with the norm (they do not depend on it).  PRE chunks of 512 elements are kept in registers.
   // Rows of at least NC * 512 elements (the usual case) take their first loads without a bounds test per load: loads
   // under separate conditions are waited for one by one, those of a straight line are all in flight together.
-  constexpr int PRE = 4;
+  // PRE = 4 for launches of few tokens (latency); PRE = 0 for many tokens, where the 16 registers of the prefetch cost a
+  // quarter of the workgroups a CU can hold and throughput counts.
   constexpr int NC = 8;
   const bool long_row = K >= (int64_t)NC * 512;
-  uint4 wpre[PRE];
-  if (sizeof(T) == 2 && wave < E) {  // 16-bit rows (a chunk of 8 elements is one 16-byte load)
+  uint4 wpre[PRE ? PRE : 1];
+  if (PRE > 0 && sizeof(T) == 2 && wave < E) {  // 16-bit rows (a chunk of 8 elements is one 16-byte load)
     const T* wrow = wr + (int64_t)wave * K;
     if (long_row) {
 #pragma unroll
@@ -297,7 +298,7 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) acc = __fadd_rn(acc, __fmul_rn(xv.v[jj], wv.v[jj]));
     };
-    const bool pre_ok = sizeof(T) == 2 && e == wave;
+    const bool pre_ok = PRE > 0 && sizeof(T) == 2 && e == wave;
 #pragma unroll
     for (int j = 0; j < PRE; ++j) {  // chunks in increasing order, as the summation order requires
       const int64_t k0 = (int64_t)lane * 8 + (int64_t)j * 512;
@@ -367,8 +368,12 @@ static int launch_router_wg(const void* x, const void* norm_w, float eps, void* 
                             SingleTokenDispatch disp = SingleTokenDispatch{nullptr, nullptr, nullptr, nullptr}) {
   const size_t lds = ((K * sizeof(T) + 15) / 16) * 16 + (64 + 8 + 64) * sizeof(float);
   if (lds > 64 * 1024) return set_error(STMOE_ERR_UNSUPPORTED, "router: K=%lld does not fit the per-token LDS row", (long long)K);
-  router_wg_kernel<T, W, FUSE_NORM><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
-      (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
+  if (T_tokens <= 512)
+    router_wg_kernel<T, W, FUSE_NORM, 4><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
+        (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
+  else
+    router_wg_kernel<T, W, FUSE_NORM, 0><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
+        (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
   return check_launch("router_wg");
 }
 
