@@ -48,15 +48,18 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 //          6 MFMA 256x256 tile with specialised producer/consumer wavefronts (prefill; packed formats),
 //          7 fp8 matrix cores, 128x128 tile kernel only (5 uses the 256x256 LDS-direct kernel where it applies)
 // Automatic choice of a grouped launch (the host knows the row total and the token count, not the rows per expert):
-// the streaming kernel when no expert can get more than 32 rows (token count <= 32), or when experts get 40 rows or
+// the streaming kernel when no expert can get more than 32 rows (token count <= 32), or when experts get 20 rows or
 // fewer on average (56 with at most 4 experts, 64 with at most 2); everything else goes to the specialised-wavefront
-// prefill kernel.  The streaming kernel walks an expert's rows in passes of 32 and re-reads the expert's weights for every
+// prefill kernel (measured on the Mixtral layer, 8 experts, top-2, Q8_0 fp16 / Q4_1 bf16, whole layer: 80 tokens streaming
+// 341 / 328 us, 96 tokens 363 / 358 us against 317 us (Q8_0) for the prefill kernel, 112 tokens 432 / 422 against 325 us,
+// 160 tokens 567 / 563 against 336 / 346 us: since token tiles of at most 128 rows run with eight loader wavefronts the prefill kernel is nearly flat
+// from 32 to 256 tokens).  The streaming kernel walks an expert's rows in passes of 32 and re-reads the expert's weights for every
 // pass, so inside its window a routing that puts all T tokens on a few experts costs those experts ceil(T / 32) passes
 // instead of one or two: at most (experts + rows / 32) weight passes in all against (experts) for a uniform routing,
 // i.e. up to 2.2 x the uniform time at 8 experts and 320 rows; the prefill kernel at those sizes is as fast as the uniform
 // case, so the window ends where the two meet for uniform routing.
 static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
-static constexpr int64_t kSkinnyMaxAvgRows = 40;
+static constexpr int64_t kSkinnyMaxAvgRows = 20;
 // A single matrix (no grouping): the streaming kernel re-reads the weights once per 32 rows and still wins up to 80 rows
 // (38 / 45 / 66 us at 48 / 64 / 96 rows of a [14336, 4096] Q8_0 matrix, against 60 / 64 / 64 us for the 256 x 256 kernel
 // and 77 us for the 128 x 128 one); beyond that the 256 x 256 kernel is the fastest at every size.
@@ -125,7 +128,7 @@ static FfnWs carve_ffn(int64_t T, int k, int64_t K, int64_t N, int dtype) {
   w.zq = w.xa + align_up((size_t)T * K * es, 256);
   w.split = w.zq + align_up((size_t)T * k * N, 256);
   // fp32 partial tiles of split reductions (prefill kernels only)
-  w.total = w.split + (T * k >= 256 ? align_up(mfma_ws_partial_bytes(), 256) : 0);
+  w.total = w.split + (T * k > 160 ? align_up(mfma_ws_partial_bytes(), 256) : 0);  // from where 8 experts leave the streaming window
   return w;
 }
 
