@@ -48,22 +48,24 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 //          6 MFMA 256x256 tile with specialised producer/consumer wavefronts (prefill; packed formats),
 //          7 fp8 matrix cores, 128x128 tile kernel only (5 uses the 256x256 LDS-direct kernel where it applies)
 // Automatic choice of a grouped launch (the host knows the row total and the token count, not the rows per expert):
-// the streaming kernel when no expert can get more than 32 rows (token count <= 32), or when experts get 20 rows or
-// fewer on average (56 with at most 4 experts, 64 with at most 2); everything else goes to the specialised-wavefront
-// prefill kernel (measured on the Mixtral layer, 8 experts, top-2, Q8_0 fp16 / Q4_1 bf16, whole layer: 80 tokens streaming
-// 341 / 328 us, 96 tokens 363 / 358 us against 317 us (Q8_0) for the prefill kernel, 112 tokens 432 / 422 against 325 us,
-// 160 tokens 567 / 563 against 336 / 346 us: since token tiles of at most 128 rows run with eight loader wavefronts the prefill kernel is nearly flat
-// from 32 to 256 tokens).  The streaming kernel walks an expert's rows in passes of 32 and re-reads the expert's weights for every
-// pass, so inside its window a routing that puts all T tokens on a few experts costs those experts ceil(T / 32) passes
-// instead of one or two: at most (experts + rows / 32) weight passes in all against (experts) for a uniform routing,
-// i.e. up to 2.2 x the uniform time at 8 experts and 320 rows; the prefill kernel at those sizes is as fast as the uniform
-// case, so the window ends where the two meet for uniform routing.
+// the streaming kernel when no expert can get more than 32 rows (token count <= 32), when the launch has at most 128 rows
+// in all (such launches get no scratch for split reductions, without which the prefill kernel leaves most CUs idle), or
+// when experts get 16 rows or fewer on average (28 with at most 4 experts); everything else goes to the
+// specialised-wavefront prefill kernel.  Measured on the Mixtral layer (top-2, Q8_0 fp16, whole layer, us; streaming /
+// prefill kernel with split scratch): 8 experts at 64 / 80 / 96 / 128 / 160 tokens 297 / 340 / 360 / 436 / 559 against
+// 307 / 310 / 315 / 321 / 331 (Q4_1 bf16: 285 / 330 / 358 / 434 / 565 against 332 / 334 / 335 / 339 / 346); 4 experts at
+// 48 / 56 / 64 / 80 tokens 168 / 172 / 235 / 295 against 183 / 184 / 186 / 190; 2 experts at 40 / 64 tokens 171 / 185
+// against 127 / 131 (with scratch, which launches of that size do not get).  Since token tiles of at most 128 rows run
+// with eight loader wavefronts the prefill kernel is nearly flat from 48 to 256 tokens.
+// The streaming kernel walks an expert's rows in passes of 32 and re-reads the expert's weights for every pass, so inside
+// its window a routing that puts all T tokens on a few experts costs those experts ceil(T / 32) passes instead of one.
 static constexpr int64_t kSkinnyMaxRowsPerExpert = 32;
-static constexpr int64_t kSkinnyMaxAvgRows = 20;
-// A single matrix (no grouping): the streaming kernel re-reads the weights once per 32 rows and still wins up to 80 rows
-// (38 / 45 / 66 us at 48 / 64 / 96 rows of a [14336, 4096] Q8_0 matrix, against 60 / 64 / 64 us for the 256 x 256 kernel
-// and 77 us for the 128 x 128 one); beyond that the 256 x 256 kernel is the fastest at every size.
-static constexpr int64_t kSkinnyMaxRowsSingle = 80;
+static constexpr int64_t kSkinnyMaxRows = 128;  // == the largest T * k without split scratch (carve_ffn)
+static inline int64_t skinny_max_avg_rows(int E) { return E <= 4 ? 28 : 16; }
+// A single matrix (no grouping): the streaming kernel re-reads the weights once per 32 rows and wins up to 48 rows
+// (24 / 38 / 45 / 58 us at 32 / 48 / 64 / 80 rows of a [14336, 4096] Q8_0 matrix, against 37 / 38 / 40 / 48 us for the
+// 256 x 256 kernel, which takes 50 us at 96-128 rows and 74-82 us from 129 to 512).
+static constexpr int64_t kSkinnyMaxRowsSingle = 48;
 // fp8 activations x fp8 weights on the fp8 matrix cores: the 256 x 256 kernel for packed weights and launches with
 // enough rows to fill its tiles (variant 5), the 128 x 128 kernel otherwise (and always with variant 7).
 static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
@@ -79,12 +81,8 @@ static int run_projection(int variant, int dtype, int wtag, int mode, const Gemm
     if (dtype == STMOE_F32) variant = 1;
     else if (!p.offsets && p.E == 1) variant = max_rows <= kSkinnyMaxRowsSingle ? 3 : 6;
     else if (p.offsets && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
-                           max_rows <= kSkinnyMaxAvgRows * p.E || (p.E <= 2 && max_rows <= 64 * p.E) ||
-                           (p.E <= 4 && max_rows <= 56 * p.E))) variant = 3;
+                           max_rows <= kSkinnyMaxRows || max_rows <= skinny_max_avg_rows(p.E) * p.E)) variant = 3;
     // Everything else goes to the 256 x 256 kernel (which hands shapes it does not take down to the 128 x 128 one).
-    // With few experts a launch can have more than 40 rows per expert and still fewer than 256 rows in all: measured
-    // there (2 / 4 / 6 experts, 100-254 rows, Q8_0 Mixtral shapes) the 128 x 128 kernel took 405-780 us per layer, the
-    // 256 x 256 one 295-440 us, and streaming 185-336 us up to 64 rows per expert with 2 experts or 56 with 4.
     else variant = 6;
   }
   if (variant == 6) {
@@ -128,7 +126,7 @@ static FfnWs carve_ffn(int64_t T, int k, int64_t K, int64_t N, int dtype) {
   w.zq = w.xa + align_up((size_t)T * K * es, 256);
   w.split = w.zq + align_up((size_t)T * k * N, 256);
   // fp32 partial tiles of split reductions (prefill kernels only)
-  w.total = w.split + (T * k > 160 ? align_up(mfma_ws_partial_bytes(), 256) : 0);  // from where 8 experts leave the streaming window
+  w.total = w.split + (T * k > 128 ? align_up(mfma_ws_partial_bytes(), 256) : 0);  // kSkinnyMaxRows: smaller launches stream
   return w;
 }
 

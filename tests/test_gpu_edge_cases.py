@@ -257,8 +257,8 @@ def test_prefill_tails_that_ride_along_with_full_token_tiles(device, fmt, dtype,
 @pytest.mark.parametrize("T", [50, 96, 127])
 @pytest.mark.parametrize("routing", ["uniform", "two experts take everything"])
 def test_few_experts_between_100_and_255_rows(device, E, T, routing):
-    """Launches of 100-254 sorted rows with 2-6 experts sit between the streaming kernel (up to 56-64 rows per expert on
-    average) and the prefill kernel, whichever the automatic choice picks from the row total; with all tokens on two
+    """Launches of 100-254 sorted rows with 2-6 experts sit between the streaming kernel (up to 128 rows in all, or 16-28
+    rows per expert on average) and the prefill kernel, whichever the automatic choice picks from the row total; with all tokens on two
     experts each of those holds T rows, several passes of the streaming kernel or one partial token tile.  Checked
     against the oracle pair by pair."""
     from sharktank_amd import _hip as hip

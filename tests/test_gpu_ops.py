@@ -71,7 +71,7 @@ def test_linear_and_dense_matmul(device):
 @pytest.mark.parametrize("M,N", [(1, 96), (7, 96), (16, 256), (17, 96), (32, 256), (33, 96), (40, 256), (64, 256), (80, 96), (81, 256)])
 def test_quantized_linear_few_rows(device, fmt, dtype, M, N):
     """One quantized matrix times a handful of rows (a Llama-style projection at decode): the streaming kernel runs
-    without an expert offsets array (up to 80 rows by itself, beyond that on request), from planar and from packed
+    without an expert offsets array (up to 48 rows by itself, beyond that on request), from planar and from packed
     planes, with the same bits from both."""
     import moe_cases as MC
     from sharktank_amd import _hip
@@ -89,7 +89,7 @@ def test_quantized_linear_few_rows(device, fmt, dtype, M, N):
         auto = _hip.mmt(x.to(device), dw)
         assert O.rel_l2(auto.cpu(), ref) < (1e-3 if dtype == torch.float16 else 8e-3)
         forced = _hip.mmt(x.to(device), dw, variant=_hip.VARIANT_SKINNY)
-        if M <= 80:  # the automatic choice for so few rows is the streaming kernel (N = 256: its LDS-sharing form)
+        if M <= 48:  # the automatic choice for so few rows is the streaming kernel (N = 256: its LDS-sharing form)
             assert torch.equal(auto.view(torch.int16), forced.view(torch.int16))
         else:
             assert O.rel_l2(forced.cpu(), ref) < (1e-3 if dtype == torch.float16 else 8e-3)
