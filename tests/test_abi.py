@@ -56,6 +56,9 @@ def test_argument_validation_without_a_gpu():
                                None, None, None, None, None, None, 0, 0, None)
     assert rc == 2 and b"32" in lib.stmoe_last_error()  # Q8_0 needs cols % 32 == 0
     assert lib.stmoe_dynamic_quantize_fp8_scratch_bytes() == 4096
+    assert lib.stmoe_probe_mfma(0, 1, 400, None, None, None) == 1  # NULL sink
+    assert lib.stmoe_probe_mfma(2, 1, 400, 16, None, None) == 2  # unknown kind
+    assert lib.stmoe_probe_mfma(0, 1, 402, 16, None, None) == 2  # iters not a multiple of 4
     assert lib.stmoe_dynamic_quantize_fp8(None, _hip.F16, 8, None, 16, 16, 16, None) == 6  # scratch too small
     assert lib.stmoe_dynamic_quantize_fp8(None, _hip.F16, 8, None, 16, 16, 4096, None) == 1  # NULL x
     # raw GGUF blocks: shape, format pairing and streaming-order constraints are checked before any launch

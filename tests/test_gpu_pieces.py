@@ -493,3 +493,16 @@ def test_dynamic_quantizer_bit_exact(device, dtype, n, kind):
     assert torch.equal(lay.qs.cpu().reshape(-1).view(torch.uint8), want_qs.reshape(-1).view(torch.uint8))
     # and the layout dequantises as the reference's TensorScaledLayout does
     assert torch.equal(lay.dequant().cpu().reshape(-1), O.dequant_tensor_scaled(want_rscale, want_qs, layout_dtype=dtype).reshape(-1))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", [0, 1])
+def test_matrix_core_probe_runs(device, kind):
+    """The ceiling probe (a launch of nothing but MFMA instructions) completes and reports a rate between a tenth of the
+    published peak and the peak itself (fp16 2500, fp8 5000 TFLOP/s): a measurement aid, so only its plausibility is checked."""
+    from sharktank_amd import _hip
+
+    peak = 2500.0 if kind == 0 else 5000.0
+    for random_operands in (True, False):
+        rate = _hip.probe_mfma(device, kind, random_operands, iters=2000, launches=2, warm_launches=2)
+        assert 0.1 * peak < rate <= 1.02 * peak, f"kind {kind}, random {random_operands}: {rate:.0f} TFLOP/s"
