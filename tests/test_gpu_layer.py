@@ -340,7 +340,7 @@ def test_single_token_forward_equals_staged_calls(device, E, k, dtype):
     assert torch.equal(staged.view(torch.int16), fused.reshape(1, case.K).view(torch.int16))
 
 
-@pytest.mark.parametrize("T", [2, 31, 32, 200, 256, 257])
+@pytest.mark.parametrize("T", [2, 31, 32, 200, 256, 257, 700])
 @pytest.mark.parametrize("E,k", [(8, 2), (64, 6)])
 def test_small_batch_forward_equals_staged_calls(device, T, E, k):
     """The fused forward (one C-ABI call, one workspace) must give the same bits as router, dispatch_build, grouped_ffn and

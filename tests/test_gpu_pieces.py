@@ -108,7 +108,11 @@ def test_rms_norm(device, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("T,K,E,k", [(64, 512, 8, 2), (33, 4096, 8, 2), (5, 1000 * 8, 16, 4), (1, 64, 3, 3)])
+@pytest.mark.parametrize("T,K,E,k", [(64, 512, 8, 2), (33, 4096, 8, 2), (5, 1000 * 8, 16, 4), (1, 64, 3, 3),
+                                     # more than 512 tokens (launches that fill the chip several times over), rows longer
+                                     # than the per-token LDS row of the one-workgroup-per-token kernel
+                                     (700, 4096, 8, 2), (1100, 6144, 8, 2), (600, 1024, 16, 4), (512 * 66 + 5, 512, 8, 2),
+                                     (520, 8192 + 512, 8, 2)])
 def test_router_bit_exact(device, dtype, T, K, E, k):
     g = torch.Generator().manual_seed(5)
     x = torch.randn(T, K, generator=g).to(dtype)
@@ -125,6 +129,31 @@ def test_router_bit_exact(device, dtype, T, K, E, k):
     ref_idx, _, _ = O.route(O.router_logits(x, wr), k)
     mism = int((ref_idx != want_idx).any(dim=1).sum())
     assert mism <= max(1, T // 100), f"{mism} of {T} tokens route differently from torch.matmul logits"
+
+
+@pytest.mark.parametrize("T", [3, 700])
+def test_router_fp16_subnormal_and_large_operands(device, T):
+    """Subnormal, tiny and large fp16 operands: the logits' bits must still be the oracle's (exact conversions to fp32,
+    products and sums rounded one by one in the documented order)."""
+    g = torch.Generator().manual_seed(11)
+    K, E, k = 1024, 8, 2
+    def operands(rows, scale):
+        v = torch.randn(rows, K, generator=g) * scale
+        sub = torch.randint(1, 1024, (rows, K), generator=g).to(torch.int16).view(torch.float16).float()  # fp16 subnormals
+        sub = sub * torch.where(torch.rand(rows, K, generator=g) < 0.5, -1.0, 1.0)
+        kind = torch.randint(0, 4, (rows, K), generator=g)
+        v = torch.where(kind == 0, sub, v)
+        v = torch.where(kind == 1, v * 1e-4, v)
+        v = torch.where(kind == 2, v * 30.0, v)
+        return v.to(torch.float16)
+    x, wr = operands(T, 1.0), operands(E, 0.02)
+    assert bool((x.float().abs() < 6.2e-5).any()) and bool(torch.isfinite(x.float()).all())
+    idx, gate, logits = _hip().router_topk(x.to(device), wr.to(device), k, want_logits=True, index_dtype=torch.int64)
+    want_logits = O.router_logits_ordered(x, wr.float())
+    assert bool(torch.isfinite(want_logits.float()).all())
+    assert torch.equal(logits.cpu().view(torch.int16), want_logits.view(torch.int16))
+    # (no index check here: logits of this size put many probabilities within an ulp of each other, where the exponential
+    # of the device and the host's may order them differently; test_router_distinct_logits_with_equal_probabilities covers that)
 
 
 def test_router_ties_lower_index_first(device):
