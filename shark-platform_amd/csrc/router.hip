@@ -205,8 +205,8 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
   // latency runs in parallel with the norm (they do not depend on it).  PRE chunks of 512 elements are kept in registers.
   // Rows of at least NC * 512 elements (the usual case) take their first loads without a bounds test per load: loads
   // under separate conditions are waited for one by one, those of a straight line are all in flight together.
-  // PRE = 4 for launches of few tokens (latency); PRE = 0 for many tokens, where the 16 registers of the prefetch cost a
-  // quarter of the workgroups a CU can hold and throughput counts.
+  // PRE = 8 (a whole row of 4096) for launches of at most 64 tokens and 4 up to 512 tokens (latency); PRE = 0 for more
+  // tokens, where the 16 registers of the prefetch cost a quarter of the workgroups a CU can hold and throughput counts.
   constexpr int NC = 8;
   const bool long_row = K >= (int64_t)NC * 512;
   uint4 wpre[PRE ? PRE : 1];
@@ -315,49 +315,60 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
     }
   }
   __syncthreads();
-  if (tid != 0) return;
+  if (wave != 0) return;
 
   // fp32 softmax, top-k of the probabilities (equal ones by increasing index), renormalised gates: same arithmetic and
-  // order as router_topk_kernel.  The probabilities replace the logits in lg_s.
-  float mx = lg_s[0];
-  for (int e = 1; e < E; ++e) mx = fmaxf(mx, lg_s[e]);
+  // order as router_topk_kernel, done by the first wavefront.  Lane e holds expert e: the exponentials and the divisions
+  // are computed side by side; everything whose order matters (the sum of the exponentials, the choice with its
+  // lower-index-first rule, the sum of the chosen probabilities) is the serial loop over values read from the lanes, which
+  // every lane runs alike.
+  const float l = lane < E ? lg_s[lane] : 0.0f;
+  float mx = __shfl(l, 0);
+  for (int e = 1; e < E; ++e) mx = fmaxf(mx, __shfl(l, e));
+  const float ex = expf(l - mx);
   float denom = 0.0f;
-  for (int e = 0; e < E; ++e) denom += expf(lg_s[e] - mx);
-  for (int e = 0; e < E; ++e) lg_s[e] = expf(lg_s[e] - mx) / denom;
+  for (int e = 0; e < E; ++e) denom += __shfl(ex, e);
+  const float pr = ex / denom;
   uint64_t taken = 0;
   float vsum = 0.0f;
+  int my_best = 0;        // lane j: the j-th choice
+  float my_bestv = 0.0f;
   for (int j = 0; j < k; ++j) {
     int best = -1;
     float bestv = 0.0f;
     for (int e = 0; e < E; ++e) {
-      const float v = lg_s[e];
+      const float v = __shfl(pr, e);
       if (!((taken >> e) & 1ull) && (best < 0 || v > bestv)) {
         best = e;
         bestv = v;
       }
     }
     taken |= 1ull << best;
-    idx_out[t * k + j] = best;
-    if (idx64_out) idx64_out[t * k + j] = best;
-    part[8 + j] = bestv;  // part has 64 + 8 floats of room after the partial sums
+    if (lane == j) {
+      my_best = best;
+      my_bestv = bestv;
+    }
     vsum += bestv;
   }
-  for (int j = 0; j < k; ++j) gate_out[t * k + j] = Cvt<T>::from_f32(part[8 + j] / vsum);
+  if (lane < k) {
+    idx_out[t * k + lane] = my_best;
+    if (idx64_out) idx64_out[t * k + lane] = my_best;
+    gate_out[t * k + lane] = Cvt<T>::from_f32(my_bestv / vsum);
+  }
 
   // A launch of one token can also write that token's dispatch (what dispatch_build_kernel would compute from idx):
   // every chosen expert has one row, the rows are ordered by expert id, pair j sits at the number of chosen experts
   // with a smaller id.  Saves a kernel launch where a forward is a handful of short launches.
   if (disp.counts) {
-    for (int e = 0; e < E; ++e) {
-      disp.counts[e] = (int32_t)((taken >> e) & 1ull);
-      disp.offsets[e] = (int32_t)__popcll(taken & ((1ull << e) - 1ull));
+    if (lane < E) {
+      disp.counts[lane] = (int32_t)((taken >> lane) & 1ull);
+      disp.offsets[lane] = (int32_t)__popcll(taken & ((1ull << lane) - 1ull));
     }
-    disp.offsets[E] = k;
-    for (int j = 0; j < k; ++j) {
-      const int e = idx_out[j];
-      const int pos = (int)__popcll(taken & ((1ull << e) - 1ull));
-      disp.perm[pos] = j;
-      disp.inv[j] = pos;
+    if (lane == 0) disp.offsets[E] = k;
+    if (lane < k) {
+      const int pos = (int)__popcll(taken & ((1ull << my_best) - 1ull));
+      disp.perm[pos] = lane;
+      disp.inv[lane] = pos;
     }
   }
 }
@@ -368,7 +379,10 @@ static int launch_router_wg(const void* x, const void* norm_w, float eps, void* 
                             SingleTokenDispatch disp = SingleTokenDispatch{nullptr, nullptr, nullptr, nullptr}) {
   const size_t lds = ((K * sizeof(T) + 15) / 16) * 16 + (64 + 8 + 64) * sizeof(float);
   if (lds > 64 * 1024) return set_error(STMOE_ERR_UNSUPPORTED, "router: K=%lld does not fit the per-token LDS row", (long long)K);
-  if (T_tokens <= 512)
+  if (T_tokens <= 64)
+    router_wg_kernel<T, W, FUSE_NORM, 8><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
+        (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
+  else if (T_tokens <= 512)
     router_wg_kernel<T, W, FUSE_NORM, 4><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
         (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
   else
