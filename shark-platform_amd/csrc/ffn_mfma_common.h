@@ -51,6 +51,32 @@ __device__ __forceinline__ bool big_tail_absorbed(int rows, int BM, bool absorb)
   const int c = rows / BM, t = rows - c * BM;
   return absorb && t > 0 && t <= kBigTailRows * c;
 }
+// Token tiles of an expert with `rows` rows.  Usually rows / BM full tiles and, if rows remain that no full tile takes
+// along, one partial tile, which is listed with the other experts' partial tiles at the end of the launch.  With `balance`
+// an expert whose remainder is more than half a tile gets rows / BM + 1 tiles of equal size instead (470 rows: 235 + 235
+// instead of 256 + 214), all of them listed like full tiles: the same work, but the workgroups that take the same feature
+// tile of the two token tiles then run side by side at the same pace and the second one finds the weight tile in L2 (a
+// full tile and its expert's partial tile, half a launch apart, both fetch it from memory).
+struct BigExpertTiles {
+  int main;     // tiles in the main list (full tiles, or the equal-sized ones)
+  int partial;  // 1: a partial tile in the list of partial tiles
+  bool even;    // main tiles are the equal-sized ones: tile s = rows [s rows / main, (s + 1) rows / main)
+};
+__device__ __forceinline__ BigExpertTiles big_expert_tiles(int rows, int BM, bool absorb, bool balance) {
+  const int c = rows / BM, t = rows - c * BM;
+  BigExpertTiles x;
+  x.main = c;
+  x.partial = 0;
+  x.even = false;
+  if (t == 0 || big_tail_absorbed(rows, BM, absorb)) return x;
+  if (balance && c == 1 && 2 * t > BM) {
+    x.main = c + 1;
+    x.even = true;
+  } else {
+    x.partial = 1;
+  }
+  return x;
+}
 // A launch whose units do not fill a whole number of rounds over the 32 CUs of an XCD leaves most CUs idle while the
 // last few units run.  With `allow_split` those last units (the partial token tiles come last) are cut along the
 // reduction into up to 4 chunks (as many as keep units x chunks within the 32 CUs) that run on separate CUs and write
@@ -68,19 +94,21 @@ __device__ __forceinline__ int big_lane_offsets(const GemmParams& p) {
   return (p.offsets && lane <= p.E) ? p.offsets[lane] : 0;
 }
 __device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int lane_off, int BM, int n_tiles, int xcd, bool allow_split,
-                                            bool absorb = false) {
+                                            bool absorb = false, bool balance = false) {
   BigPlan pl;
   pl.F = 0;
   pl.R = 0;
   if (p.offsets) {
     for (int e = 0; e < p.E; ++e) {
       const int rows = __builtin_amdgcn_readlane(lane_off, e + 1) - __builtin_amdgcn_readlane(lane_off, e);
-      pl.F += rows / BM;
-      pl.R += (rows % BM) != 0 && !big_tail_absorbed(rows, BM, absorb);
+      const BigExpertTiles x = big_expert_tiles(rows, BM, absorb, balance);
+      pl.F += x.main;
+      pl.R += x.partial;
     }
   } else {
-    pl.F = (int)(p.fixed_rows / BM);
-    pl.R = (p.fixed_rows % BM) != 0 && !big_tail_absorbed((int)p.fixed_rows, BM, absorb);
+    const BigExpertTiles x = big_expert_tiles((int)p.fixed_rows, BM, absorb, balance);
+    pl.F = x.main;
+    pl.R = x.partial;
   }
   const int UF = pl.F * n_tiles, UR = pl.R * n_tiles;
   pl.f0 = (int)((int64_t)UF * xcd / 8);
@@ -126,8 +154,21 @@ __device__ __forceinline__ void big_set_tail(int b, int rows, int BM, int s, boo
   t.tail_begin = b + first;
   t.tail_rows = min(kBigTailRows, rows - first);
 }
+// Rows of main tile s of an expert (first row b, `rows` rows) and the tail rows it takes along.
+__device__ __forceinline__ void big_main_tile(int b, int rows, int BM, int s, const BigExpertTiles& x, bool absorb, BigTile& t) {
+  if (x.even) {
+    t.row_begin = b + (int)((int64_t)rows * s / x.main);
+    t.row_end = b + (int)((int64_t)rows * (s + 1) / x.main);
+    t.tail_begin = 0;
+    t.tail_rows = 0;
+  } else {
+    t.row_begin = b + s * BM;
+    t.row_end = t.row_begin + BM;
+    big_set_tail(b, rows, BM, s, absorb, t);
+  }
+}
 __device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int BM, int n_tiles, const BigPlan& pl, int unit, BigTile& t,
-                                         bool absorb = false) {
+                                         bool absorb = false, bool balance = false) {
   int u;
   bool partial;
   t.tail_begin = 0;
@@ -145,28 +186,25 @@ __device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int 
     t.e = 0;
     if (partial) {
       t.ntile = u;
-      t.row_begin = pl.F * BM;
+      t.row_begin = (int)(p.fixed_rows / BM) * BM;
       t.row_end = (int)p.fixed_rows;
     } else {
       int s;
       big_full_unit(u, pl.F, n_tiles, s, t.ntile);
-      t.row_begin = s * BM;
-      t.row_end = t.row_begin + BM;
-      big_set_tail(0, (int)p.fixed_rows, BM, s, absorb, t);
+      big_main_tile(0, (int)p.fixed_rows, BM, s, big_expert_tiles((int)p.fixed_rows, BM, absorb, balance), absorb, t);
     }
     return true;
   }
   if (!partial) {
     for (int e = 0; e < p.E; ++e) {
       const int b = __builtin_amdgcn_readlane(lane_off, e), rows = __builtin_amdgcn_readlane(lane_off, e + 1) - b;
-      const int c = rows / BM, units = c * n_tiles;
+      const BigExpertTiles x = big_expert_tiles(rows, BM, absorb, balance);
+      const int units = x.main * n_tiles;
       if (u < units) {
         int s;
-        big_full_unit(u, c, n_tiles, s, t.ntile);
+        big_full_unit(u, x.main, n_tiles, s, t.ntile);
         t.e = e;
-        t.row_begin = b + s * BM;
-        t.row_end = t.row_begin + BM;
-        big_set_tail(b, rows, BM, s, absorb, t);
+        big_main_tile(b, rows, BM, s, x, absorb, t);
         return true;
       }
       u -= units;
@@ -177,7 +215,7 @@ __device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int 
   int s = u - t.ntile * pl.R;
   for (int e = 0; e < p.E; ++e) {
     const int b = __builtin_amdgcn_readlane(lane_off, e), rows = __builtin_amdgcn_readlane(lane_off, e + 1) - b;
-    if (rows % BM && !big_tail_absorbed(rows, BM, absorb)) {
+    if (big_expert_tiles(rows, BM, absorb, balance).partial) {
       if (s == 0) {
         t.e = e;
         t.row_begin = b + rows / BM * BM;
@@ -212,7 +250,7 @@ __device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_t
 // Item j of an XCD's work list: the whole units first, then the chunks of the split ones (the same numbering as the
 // workgroup index j of big_tile_id), from a plan and offsets fetched once: for workgroups that walk several items.
 __device__ __forceinline__ bool big_item(const GemmParams& p, int lane_off, int BM, int n_tiles, const BigPlan& pl, int xcd, int j, BigTile& t,
-                                         bool absorb = false) {
+                                         bool absorb = false, bool balance = false) {
   int unit;
   if (j < pl.whole) {
     unit = j;
@@ -227,7 +265,7 @@ __device__ __forceinline__ bool big_item(const GemmParams& p, int lane_off, int 
     t.nchunks = pl.chunks;
     t.chunk_slot = xcd * kBigChunkSlotsPerXcd + c;
   }
-  return big_unit(p, lane_off, BM, n_tiles, pl, unit, t, absorb);
+  return big_unit(p, lane_off, BM, n_tiles, pl, unit, t, absorb, balance);
 }
 // Grid size that covers every XCD's share for at most `slots_bound` token tiles (a split adds up to 24 workgroups).
 static inline int big_grid(int n_tiles, int slots_bound, bool allow_split) {

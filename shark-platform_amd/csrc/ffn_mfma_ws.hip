@@ -87,7 +87,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
   const int n_tiles = ka.n_tiles;
   float* const partial = ka.partial;
   const int xcd = blockIdx.x & 7, wg = blockIdx.x >> 3, wgs = ka.wgs_per_xcd;
-  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, partial != nullptr, true);
+  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, partial != nullptr, true, true);
   // Which item of round `round` (wgs consecutive items of the XCD's list) this workgroup takes: its own index shifted
   // by half a round plus one per round.  Neighbouring items differ systematically in cost (in a block of 32 full units the
   // first half belongs to an expert's first token tile, which carries most ride-along rows; partial units cycle through
@@ -95,7 +95,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
   // collect one kind: the launch ends when the slowest workgroup does.
   const int slot = (wg + round * ((wgs >> 1) + 1)) % wgs;
   BigTile tile;
-  if (!big_item(p, lane_off, BM, n_tiles, pl, xcd, round * wgs + slot, tile, true)) return;
+  if (!big_item(p, lane_off, BM, n_tiles, pl, xcd, round * wgs + slot, tile, true, true)) return;
   const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
   // this workgroup's K steps: all of them, or one chunk of a split unit
@@ -507,10 +507,10 @@ __global__ void __launch_bounds__(256) big_reduce_kernel(GemmParams p, int n_til
   constexpr int BN = 256, BM = 256;
   const int xcd = blockIdx.x >> 4, su = blockIdx.x & 15;
   const int lane_off = big_lane_offsets(p);
-  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, true, true);
+  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, true, true, true);
   if (su >= pl.rest) return;
   BigTile t;
-  if (!big_unit(p, lane_off, BM, n_tiles, pl, pl.whole + su, t, true)) return;
+  if (!big_unit(p, lane_off, BM, n_tiles, pl, pl.whole + su, t, true, true)) return;
   const int rows_here = t.row_end - t.row_begin;
   const int r = blockIdx.y * 32 + (threadIdx.x >> 3);  // row of the partial tile: tile rows, then the absorbed tail's rows from BM on
   int sorted_row;
