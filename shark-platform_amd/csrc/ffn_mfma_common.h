@@ -56,20 +56,23 @@ __device__ __forceinline__ bool big_tail_absorbed(int rows, int BM, bool absorb)
 // an expert whose remainder is more than half a tile gets rows / BM + 1 tiles of equal size instead (470 rows: 235 + 235
 // instead of 256 + 214), all of them listed like full tiles: the same work, but the workgroups that take the same feature
 // tile of the two token tiles then run side by side at the same pace and the second one finds the weight tile in L2 (a
-// full tile and its expert's partial tile, half a launch apart, both fetch it from memory).
+// full tile and its expert's partial tile, half a launch apart, both fetch it from memory).  balance = 1 does that for
+// experts with one full tile, balance = 2 for any number of full tiles (650 rows: 3 x 217 instead of 256 + 256 + 138),
+// which pays where a tile with fewer rows is a faster unit (Q8_0: Mixtral layer at 4096 tokens 2 % faster) and costs
+// where the loaders set the pace of a unit whatever its rows (Q4_1: Grok-shape skewed prefill 2.4 % slower).
 struct BigExpertTiles {
   int main;     // tiles in the main list (full tiles, or the equal-sized ones)
   int partial;  // 1: a partial tile in the list of partial tiles
   bool even;    // main tiles are the equal-sized ones: tile s = rows [s rows / main, (s + 1) rows / main)
 };
-__device__ __forceinline__ BigExpertTiles big_expert_tiles(int rows, int BM, bool absorb, bool balance) {
+__device__ __forceinline__ BigExpertTiles big_expert_tiles(int rows, int BM, bool absorb, int balance) {
   const int c = rows / BM, t = rows - c * BM;
   BigExpertTiles x;
   x.main = c;
   x.partial = 0;
   x.even = false;
   if (t == 0 || big_tail_absorbed(rows, BM, absorb)) return x;
-  if (balance && c == 1 && 2 * t > BM) {
+  if (2 * t > BM && (balance == 2 ? c > 0 : balance == 1 && c == 1)) {
     x.main = c + 1;
     x.even = true;
   } else {
@@ -94,7 +97,7 @@ __device__ __forceinline__ int big_lane_offsets(const GemmParams& p) {
   return (p.offsets && lane <= p.E) ? p.offsets[lane] : 0;
 }
 __device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int lane_off, int BM, int n_tiles, int xcd, bool allow_split,
-                                            bool absorb = false, bool balance = false) {
+                                            bool absorb = false, int balance = 0) {
   BigPlan pl;
   pl.F = 0;
   pl.R = 0;
@@ -131,18 +134,16 @@ __device__ __forceinline__ BigPlan big_plan(const GemmParams& p, int lane_off, i
   return pl;
 }
 // Unit number `unit` of the XCD's list: full units, then partial ones.
-// Full units are listed expert by expert, and inside an expert in blocks of about 32 units (one round over an XCD's
-// CUs) made of all of the expert's full token tiles x as many neighbouring feature tiles as fit: the workgroups that run
-// together on an XCD then share a few token tiles and a few weight tiles through its L2 instead of each fetching its own
-// (with 4 token tiles per expert: 4 + 8 operand streams for 32 workgroups).  Partial units: feature tile by feature
-// tile, one unit per expert that has a partial token tile.
+// Full units are listed expert by expert, and inside an expert feature tile by feature tile with the expert's token
+// tiles of one feature tile next to each other: the 32 workgroups of an XCD that run consecutive units then share a few
+// token tiles and a few weight tiles through its L2 instead of each fetching its own (with 4 token tiles per expert:
+// 4 + 8 operand streams for 32 workgroups), and the workgroups that need the same weight tile start together whatever
+// the number of token tiles (blocks of all token tiles x 32 / tiles feature tiles, listed token tile by token tile, gave
+// the same sets only when the tile count divides 32: with 3 token tiles the partners drifted into different rounds).
+// Partial units: feature tile by feature tile, one unit per expert that has a partial token tile.
 __device__ __forceinline__ void big_full_unit(int u, int c, int n_tiles, int& token_tile, int& ntile) {
-  const int bn0 = c >= kBigCusPerXcd ? 1 : kBigCusPerXcd / c;  // feature tiles per block
-  const int per = c * bn0;
-  const int b = u / per, v = u - b * per;
-  const int bn = min(bn0, n_tiles - b * bn0);
-  token_tile = v / bn;
-  ntile = b * bn0 + v - token_tile * bn;
+  ntile = u / c;
+  token_tile = u - ntile * c;
 }
 // Tail rows that full token tile s of an expert (first row b, `rows` rows) takes along.
 __device__ __forceinline__ void big_set_tail(int b, int rows, int BM, int s, bool absorb, BigTile& t) {
@@ -168,7 +169,7 @@ __device__ __forceinline__ void big_main_tile(int b, int rows, int BM, int s, co
   }
 }
 __device__ __forceinline__ bool big_unit(const GemmParams& p, int lane_off, int BM, int n_tiles, const BigPlan& pl, int unit, BigTile& t,
-                                         bool absorb = false, bool balance = false) {
+                                         bool absorb = false, int balance = 0) {
   int u;
   bool partial;
   t.tail_begin = 0;
@@ -250,7 +251,7 @@ __device__ __forceinline__ bool big_tile_id(const GemmParams& p, int BM, int n_t
 // Item j of an XCD's work list: the whole units first, then the chunks of the split ones (the same numbering as the
 // workgroup index j of big_tile_id), from a plan and offsets fetched once: for workgroups that walk several items.
 __device__ __forceinline__ bool big_item(const GemmParams& p, int lane_off, int BM, int n_tiles, const BigPlan& pl, int xcd, int j, BigTile& t,
-                                         bool absorb = false, bool balance = false) {
+                                         bool absorb = false, int balance = 0) {
   int unit;
   if (j < pl.whole) {
     unit = j;

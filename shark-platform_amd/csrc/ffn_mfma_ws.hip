@@ -38,6 +38,9 @@ __device__ __forceinline__ int pair_token(int pair, int k_top) {
   return pair / k_top;
 }
 
+// Which experts get equal-sized token tiles (see big_expert_tiles).
+constexpr int ws_balance(int wf) { return wf == WF_Q8_0_P ? 2 : 1; }
+
 struct WsArgs {
   GemmParams p;
   int n_tiles;
@@ -49,6 +52,7 @@ template <typename T, int WF, int MODE>
 __global__ void __launch_bounds__(768, 1)
 grouped_mfma_ws_kernel(WsArgs args) {
   constexpr int BN = 256, BM = 256;
+  constexpr int kBalance = ws_balance(WF);
   constexpr int WSTAGE = BN * BIG_LS, XSTAGE = BM * BIG_LS;  // elements
   extern __shared__ __align__(16) uint16_t lds[];
 
@@ -87,7 +91,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
   const int n_tiles = ka.n_tiles;
   float* const partial = ka.partial;
   const int xcd = blockIdx.x & 7, wg = blockIdx.x >> 3, wgs = ka.wgs_per_xcd;
-  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, partial != nullptr, true, true);
+  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, partial != nullptr, true, kBalance);
   // Which item of round `round` (wgs consecutive items of the XCD's list) this workgroup takes: its own index shifted
   // by half a round plus one per round.  Neighbouring items differ systematically in cost (in a block of 32 full units the
   // first half belongs to an expert's first token tile, which carries most ride-along rows; partial units cycle through
@@ -95,7 +99,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
   // collect one kind: the launch ends when the slowest workgroup does.
   const int slot = (wg + round * ((wgs >> 1) + 1)) % wgs;
   BigTile tile;
-  if (!big_item(p, lane_off, BM, n_tiles, pl, xcd, round * wgs + slot, tile, true, true)) return;
+  if (!big_item(p, lane_off, BM, n_tiles, pl, xcd, round * wgs + slot, tile, true, kBalance)) return;
   const int e = tile.e, row_begin = tile.row_begin, row_end = tile.row_end, ntile = tile.ntile;
   const int rows_here = row_end - row_begin;
   // this workgroup's K steps: all of them, or one chunk of a split unit
@@ -502,15 +506,15 @@ grouped_mfma_ws_kernel(WsArgs args) {
 // Adds the chunks of every split unit in chunk order and writes the rows: DOWN: the sums; GATEUP: the gated product of
 // the gate sums (columns 0..127 of the partial tile) and the up sums (columns 128..255).  Grid: (8 XCDs x 16 split
 // units, 8 blocks of 32 rows); the unit list is recomputed with the same plan as the main kernel.
-template <typename T, int MODE>
+template <typename T, int MODE, int BALANCE>
 __global__ void __launch_bounds__(256) big_reduce_kernel(GemmParams p, int n_tiles, const float* partial) {
   constexpr int BN = 256, BM = 256;
   const int xcd = blockIdx.x >> 4, su = blockIdx.x & 15;
   const int lane_off = big_lane_offsets(p);
-  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, true, true, true);
+  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, true, true, BALANCE);
   if (su >= pl.rest) return;
   BigTile t;
-  if (!big_unit(p, lane_off, BM, n_tiles, pl, pl.whole + su, t, true, true)) return;
+  if (!big_unit(p, lane_off, BM, n_tiles, pl, pl.whole + su, t, true, BALANCE)) return;
   const int rows_here = t.row_end - t.row_begin;
   const int r = blockIdx.y * 32 + (threadIdx.x >> 3);  // row of the partial tile: tile rows, then the absorbed tail's rows from BM on
   int sorted_row;
@@ -560,7 +564,7 @@ static int launch_ws_m(const GemmParams& p, int64_t max_rows, float* partial, hi
   kern<<<dim3((unsigned)(8 * per_xcd)), 768, lds_bytes, st>>>(WsArgs{p, n_tiles, per_xcd, partial});
   int rc = check_launch("grouped_mfma_ws");
   if (rc || !partial) return rc;
-  big_reduce_kernel<T, MODE><<<dim3(8 * 16, (BM + kBigTailRows + 31) / 32), 256, 0, st>>>(p, n_tiles, partial);
+  big_reduce_kernel<T, MODE, ws_balance(WF)><<<dim3(8 * 16, (BM + kBigTailRows + 31) / 32), 256, 0, st>>>(p, n_tiles, partial);
   return check_launch("big_reduce");
 }
 

@@ -205,7 +205,7 @@ def _routing_with_rows(rows, T, k, seed):
     [261, 517, 512 + 32, 512 + 33, 256 + 16, 256 + 17, 300, 122],  # absorbed: 5, 5, 32 (two tiles x 16), 16; not: 33, 17
     [768 + 48, 768 + 1, 256, 255, 1, 0, 270, 257],                  # three full tiles x 16; one-row tails; an expert without rows
     [128, 129, 127, 1, 18, 64, 256 + 128, 256 + 129],               # token tiles of at most 128 rows (8 loaders, 4 consumers) and both sides of that limit
-    [470, 511, 385, 384, 256 + 128 + 1, 512 + 200, 491, 130],       # one full tile and more than half of another: two equal tiles (235 + 235, 256 + 255, 193 + 192); not: 384, 712
+    [470, 511, 385, 384, 256 + 128 + 1, 512 + 200, 491, 130],       # a full tile and more than half of another: equal tiles (235 + 235, 256 + 255, 193 + 192; Q8_0 also 712 = 3 x 237+); not: 384
 ])
 def test_prefill_tails_that_ride_along_with_full_token_tiles(device, fmt, dtype, rows):
     """Row counts a few rows above a multiple of 256: the prefill kernel lets every full token tile of such an expert take up
