@@ -447,4 +447,30 @@ template <> struct BigPiece<WF_Q4_1_P> {
   }
 };
 
+// ---- output rows in whole cache lines ---------------------------------------------------------------------
+// An MFMA result leaves lane (n, g) with 4 consecutive features of token row n per 16-feature block: features
+// 16 i + 4 g .. + 3 of block i.  Stored as they are, a wavefront instruction writes 32 bytes to each of 16 rows and a
+// 128-byte line of the output is touched by four instructions.  A 4 x 4 transpose over the lane groups (register i of group g
+// <-> register g of group i; two v_permlane32_swap and two v_permlane16_swap per dword) gives lane (n, g) the 16 consecutive
+// features 16 g .. 16 g + 15 of the four blocks' 64: 32 bytes per lane, a whole line per row and instruction pair.
+// Every lane of the wavefront must take part.
+__device__ __forceinline__ void lane_group_transpose4(uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3) {
+  typedef uint32_t pair_t __attribute__((ext_vector_type(2)));
+  const pair_t a = __builtin_amdgcn_permlane32_swap(r0, r2, false, false);
+  const pair_t b = __builtin_amdgcn_permlane32_swap(r1, r3, false, false);
+  const pair_t c = __builtin_amdgcn_permlane16_swap(a.x, b.x, false, false);
+  const pair_t d = __builtin_amdgcn_permlane16_swap(a.y, b.y, false, false);
+  r0 = c.x; r1 = c.y; r2 = d.x; r3 = d.y;
+}
+// q[i] = this lane's 4 features (two packed 16-bit pairs) of block i; afterwards q[0..3] are 16 consecutive features.
+__device__ __forceinline__ void lane_group_transpose4(uint2 (&q)[4]) {
+  lane_group_transpose4(q[0].x, q[1].x, q[2].x, q[3].x);
+  lane_group_transpose4(q[0].y, q[1].y, q[2].y, q[3].y);
+}
+__device__ __forceinline__ void store_16_features(void* dst, const uint2 (&q)[4]) {
+  uint4* d = reinterpret_cast<uint4*>(dst);
+  d[0] = make_uint4(q[0].x, q[0].y, q[1].x, q[1].y);
+  d[1] = make_uint4(q[2].x, q[2].y, q[3].x, q[3].y);
+}
+
 }  // namespace stmoe

@@ -445,12 +445,27 @@ grouped_mfma_ws_kernel(WsArgs args) {
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------------
+  // Rows are written in whole 128-byte lines (see lane_group_transpose4; the launcher checks their alignment).
   auto store_gateup = [&](auto act_tag) {
     constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
       const int r = wm * rpg + tj * 16 + n_in;
-      if (tj * 16 + n_in < my_rows) {
+      const bool mine = tj * 16 + n_in < my_rows;
+      if constexpr (ACT == STMOE_ACT_SILU) {
+        uint2 q[4];
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti) {
+          const float gq[4] = {acc[ti][tj][0], acc[ti][tj][1], acc[ti][tj][2], acc[ti][tj][3]};
+          const float uq[4] = {acc[ti + 4][tj][0], acc[ti + 4][tj][1], acc[ti + 4][tj][2], acc[ti + 4][tj][3]};
+          q[ti] = gateup_quad<T, ACT>(gq, uq);
+        }
+        lane_group_transpose4(q);
+        if (mine)
+          store_16_features(reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo + (int64_t)ntile * (BN / 2) + wn * 64 + 16 * g, q);
+        __builtin_amdgcn_sched_barrier(0);  // one column block at a time: the accumulators leave no room for more
+      } else if (mine) {
+        // (erf-GELU: its branches keep too much alive next to four finished blocks; every block is stored as it is done)
         T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo + (int64_t)ntile * (BN / 2) + wn * 64 + 4 * g;
 #pragma unroll
         for (int ti = 0; ti < 4; ++ti) {
@@ -482,12 +497,19 @@ grouped_mfma_ws_kernel(WsArgs args) {
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
       const int r = wm * rpg + tj * 16 + n_in;
-      if (tj * 16 + n_in < my_rows) {
-        T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo;
+      const bool mine = tj * 16 + n_in < my_rows;
 #pragma unroll
-        for (int ti = 0; ti < 8; ++ti)
-          *reinterpret_cast<uint2*>(orow + (int64_t)ntile * BN + wn * 128 + ti * 16 + 4 * g) =
-              make_uint2(pack2<T>(acc[ti][tj][0], acc[ti][tj][1]), pack2<T>(acc[ti][tj][2], acc[ti][tj][3]));
+      for (int half = 0; half < 2; ++half) {
+        uint2 q[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const floatx4_t v = acc[4 * half + i][tj];
+          q[i] = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
+        }
+        lane_group_transpose4(q);
+        if (mine)
+          store_16_features(reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo + (int64_t)ntile * BN + wn * 128 + half * 64 + 16 * g, q);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
@@ -583,8 +605,8 @@ int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64
   if (p.offsets && p.E >= 64) return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: at most 63 experts");
   if (wtag != WF_Q8_0_P && wtag != WF_Q4_1_P && wtag != WF_FP8_F32D_P)
     return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs weights in a packed streaming order");
-  if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0 || p.n_out % (mode == MODE_GATEUP ? 128 : 256) != 0)
-    return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs K %% 256 == 0 and output features in whole tiles");
+  if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 8 != 0 || !aligned16(p.out) || p.n_out % (mode == MODE_GATEUP ? 128 : 256) != 0)
+    return set_error(STMOE_ERR_UNSUPPORTED, "mfma ws kernel: needs K %% 256 == 0, output features in whole tiles and 16-byte aligned output rows");
   {
     // token rows are addressed with 32-bit byte offsets from the activation base
     const int64_t src_rows = p.perm ? (max_rows + p.k_top - 1) / p.k_top : max_rows;
