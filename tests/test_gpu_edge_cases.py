@@ -206,6 +206,7 @@ def _routing_with_rows(rows, T, k, seed):
     [768 + 48, 768 + 1, 256, 255, 1, 0, 270, 257],                  # three full tiles x 16; one-row tails; an expert without rows
     [128, 129, 127, 1, 18, 64, 256 + 128, 256 + 129],               # token tiles of at most 128 rows (8 loaders, 4 consumers) and both sides of that limit
     [470, 511, 385, 384, 256 + 128 + 1, 512 + 200, 491, 130],       # a full tile and more than half of another: equal tiles (235 + 235, 256 + 255, 193 + 192; Q8_0 also 712 = 3 x 237+); not: 384
+    [900, 1100, 650, 1290, 770, 1024 + 200, 768 + 129, 301],        # several full tiles and a large remainder (Q8_0: 4 x 225, 5 x 220, 3 x 217, ...; other formats keep full + partial tiles)
 ])
 def test_prefill_tails_that_ride_along_with_full_token_tiles(device, fmt, dtype, rows):
     """Row counts a few rows above a multiple of 256: the prefill kernel lets every full token tile of such an expert take up
