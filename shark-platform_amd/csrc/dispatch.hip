@@ -15,11 +15,14 @@ static constexpr int kDispatchWaves = kDispatchThreads / 64;
 // expert) and wcnt[16][E] (per-wave counts of the current chunk).
 __global__ void __launch_bounds__(kDispatchThreads)
 dispatch_build_kernel(const int32_t* __restrict__ idx, int64_t n, int E, int32_t* __restrict__ counts,
-                      int32_t* __restrict__ offsets, int32_t* __restrict__ perm, int32_t* __restrict__ inv) {
+                      int32_t* __restrict__ offsets, int32_t* __restrict__ perm, int32_t* __restrict__ inv,
+                      int32_t* __restrict__ zero_words, int n_zero) {
   extern __shared__ int32_t sm[];
   int32_t* base = sm;
   int32_t* wcnt = sm + E;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (the fused layer forward has the ticket words of the projections' split reductions cleared here: a launch it makes anyway)
+  if (tid < n_zero) zero_words[tid] = 0;
 
   for (int e = tid; e < E; e += kDispatchThreads) base[e] = 0;
   __syncthreads();
@@ -70,6 +73,82 @@ dispatch_build_kernel(const int32_t* __restrict__ idx, int64_t n, int E, int32_t
       base[ee] += s;
     }
     __syncthreads();
+  }
+}
+
+// The same result for launches of at most 8 chunks of 1024 pairs and at most 64 experts (a prefill batch of 4096 tokens
+// with top-2 routing), with three barriers in all instead of three per chunk: every thread fetches its pair of every
+// chunk at once (one memory latency instead of one per chunk and pass), the per-wavefront counts of all chunks go to
+// LDS in one sweep, one thread per expert turns its column of counts (chunk by chunk, wavefront by wavefront: the order
+// of the pairs) into running positions, and after the scan over the experts every pair knows its place.
+static constexpr int kDispatchRegChunks = 8;
+static constexpr int kDispatchRegExperts = 64;
+__global__ void __launch_bounds__(kDispatchThreads)
+dispatch_build_reg_kernel(const int32_t* __restrict__ idx, int n, int E, int32_t* __restrict__ counts,
+                          int32_t* __restrict__ offsets, int32_t* __restrict__ perm, int32_t* __restrict__ inv,
+                          int32_t* __restrict__ zero_words, int n_zero) {
+  extern __shared__ int32_t sm[];
+  int32_t* cnt = sm;  // [chunk][wavefront][E]: count, then the position of the wavefront's first pair inside its expert
+  int32_t* first = sm + kDispatchRegChunks * kDispatchWaves * E;  // [E] first row of each expert
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid < n_zero) zero_words[tid] = 0;
+  const int chunks = (n + kDispatchThreads - 1) / kDispatchThreads;
+  int e[kDispatchRegChunks], rank[kDispatchRegChunks];
+#pragma unroll
+  for (int c = 0; c < kDispatchRegChunks; ++c) {
+    const int i = c * kDispatchThreads + tid;
+    e[c] = i < n ? idx[i] : -1;
+  }
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+  for (int c = 0; c < kDispatchRegChunks; ++c) {
+    if (c < chunks) {
+      if (e[c] >= E) e[c] = E - 1;  // out-of-range ids are a caller error; clamp to stay in bounds
+      if (e[c] < 0 && c * kDispatchThreads + tid < n) e[c] = 0;
+      rank[c] = 0;
+      for (int ee = 0; ee < E; ++ee) {
+        const uint64_t mask = __ballot(e[c] == ee);
+        if (e[c] == ee) rank[c] = __popcll(mask & lt_mask);
+        if (lane == 0) cnt[(c * kDispatchWaves + wave) * E + ee] = __popcll(mask);
+      }
+    }
+  }
+  __syncthreads();
+  if (tid < E) {
+    int32_t run = 0;
+    for (int c = 0; c < chunks; ++c) {
+      int32_t v[kDispatchWaves];  // a chunk's sixteen counts are read together, not one after the other
+#pragma unroll
+      for (int w = 0; w < kDispatchWaves; ++w) v[w] = cnt[(c * kDispatchWaves + w) * E + tid];
+#pragma unroll
+      for (int w = 0; w < kDispatchWaves; ++w) {
+        cnt[(c * kDispatchWaves + w) * E + tid] = run;
+        run += v[w];
+      }
+    }
+    counts[tid] = run;
+    first[tid] = run;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int32_t run = 0;
+    for (int ee = 0; ee < E; ++ee) {
+      const int32_t c = first[ee];
+      offsets[ee] = run;
+      first[ee] = run;
+      run += c;
+    }
+    offsets[E] = run;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < kDispatchRegChunks; ++c) {
+    const int i = c * kDispatchThreads + tid;
+    if (i < n) {
+      const int32_t pos = first[e[c]] + cnt[(c * kDispatchWaves + wave) * E + e[c]] + rank[c];
+      perm[pos] = i;
+      inv[i] = pos;
+    }
   }
 }
 
@@ -153,6 +232,23 @@ scale_rows_kernel(const T* __restrict__ y, const T* __restrict__ g, int64_t K, T
     out[r * K + i] = Cvt<T>::from_f32(keep_f32(__fmul_rn(gv, Cvt<T>::to_f32(y[r * K + i]))));
 }
 
+int dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv,
+                   int32_t* zero_words, int n_zero, hipStream_t st) {
+  STMOE_REQUIRE(n_pairs >= 0 && n_pairs < 0x7fffffffLL, STMOE_ERR_SHAPE, "dispatch_build: n_pairs=%lld", (long long)n_pairs);
+  STMOE_REQUIRE(E >= 1 && E <= 1024, STMOE_ERR_SHAPE, "dispatch_build: expert count %d outside 1..1024", E);
+  STMOE_REQUIRE(counts && offsets, STMOE_ERR_NULL, "dispatch_build: counts/offsets NULL");
+  STMOE_REQUIRE(n_pairs == 0 || (idx && perm && inv), STMOE_ERR_NULL, "dispatch_build: idx/perm/inv NULL");
+  STMOE_REQUIRE(n_zero >= 0 && n_zero <= kDispatchThreads && (n_zero == 0 || zero_words), STMOE_ERR_SHAPE, "dispatch_build: %d words to clear", n_zero);
+  if (n_pairs <= kDispatchRegChunks * kDispatchThreads && E <= kDispatchRegExperts) {
+    const size_t lds = sizeof(int32_t) * (size_t)E * (kDispatchRegChunks * kDispatchWaves + 1);
+    dispatch_build_reg_kernel<<<1, kDispatchThreads, lds, st>>>(idx, (int)n_pairs, E, counts, offsets, perm, inv, zero_words, n_zero);
+    return check_launch("dispatch_build");
+  }
+  const size_t lds = sizeof(int32_t) * (size_t)E * (1 + kDispatchWaves);
+  dispatch_build_kernel<<<1, kDispatchThreads, lds, st>>>(idx, n_pairs, E, counts, offsets, perm, inv, zero_words, n_zero);
+  return check_launch("dispatch_build");
+}
+
 }  // namespace stmoe
 
 using namespace stmoe;
@@ -175,13 +271,7 @@ extern "C" int stmoe_scale_rows(const void* y, const void* g, int dtype, int64_t
 
 extern "C" int stmoe_dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets,
                                     int32_t* perm, int32_t* inv, stmoe_stream_t stream) {
-  STMOE_REQUIRE(n_pairs >= 0 && n_pairs < 0x7fffffffLL, STMOE_ERR_SHAPE, "dispatch_build: n_pairs=%lld", (long long)n_pairs);
-  STMOE_REQUIRE(E >= 1 && E <= 1024, STMOE_ERR_SHAPE, "dispatch_build: expert count %d outside 1..1024", E);
-  STMOE_REQUIRE(counts && offsets, STMOE_ERR_NULL, "dispatch_build: counts/offsets NULL");
-  STMOE_REQUIRE(n_pairs == 0 || (idx && perm && inv), STMOE_ERR_NULL, "dispatch_build: idx/perm/inv NULL");
-  const size_t lds = sizeof(int32_t) * (size_t)E * (1 + kDispatchWaves);
-  dispatch_build_kernel<<<1, kDispatchThreads, lds, as_stream(stream)>>>(idx, n_pairs, E, counts, offsets, perm, inv);
-  return check_launch("dispatch_build");
+  return dispatch_build(idx, n_pairs, E, counts, offsets, perm, inv, nullptr, 0, as_stream(stream));
 }
 
 extern "C" int stmoe_combine(const void* y_sorted, const void* gate, const int32_t* inv, int dtype, int64_t T, int k,

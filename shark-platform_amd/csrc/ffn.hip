@@ -143,7 +143,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
                             const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
                             int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
                             const float* z_scale, void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
-                            stmoe_stream_t stream, void** events) {
+                            stmoe_stream_t stream, void** events, bool tickets_zeroed = false) {
   STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1, STMOE_ERR_SHAPE, "grouped_ffn: T=%lld K=%lld N=%lld E=%d k=%d",
                 (long long)T, (long long)K, (long long)N, E, k);
   STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
@@ -191,6 +191,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   p.w0 = make_view(w_gate); p.w1 = make_view(w_up);
   p.out = z; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr; p.expert_rows_bound = T;
   p.split_scratch = ws.total > ws.split ? reinterpret_cast<float*>(base + ws.split) : nullptr;
+  p.split_tickets_zeroed = tickets_zeroed;
   mark(events, 0, st);
   if (x_scale) {
     if (mfma8_in) rc = stmoe_quantize_fp8(x, dtype, x_scale, T * K, xa, stream);
@@ -213,6 +214,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   q.w0 = make_view(w_down); q.w1 = q.w0;
   q.out = y_sorted; q.ldo = K; q.n_out = K; q.kred = N; q.act = act; q.x_scale = nullptr; q.expert_rows_bound = T;
   q.split_scratch = ws.total > ws.split ? reinterpret_cast<float*>(base + ws.split) : nullptr;
+  q.split_tickets_zeroed = tickets_zeroed;  // (a launch that uses the tickets leaves them at zero)
   mark(events, 2, st);
   if (z_scale) {
     if (mfma8_out && !mfma8_in) rc = stmoe_quantize_fp8(z, dtype, z_scale, rows * N, zq, stream);
@@ -354,10 +356,16 @@ static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int6
   if (rc) return rc;
   mark(events, 3, st);
   mark(events, 4, st);
-  if (!router_dispatches && (rc = stmoe_dispatch_build(idx, T * k, E, counts, offsets, perm, inv, stream))) return rc;
+  // the dispatch launch also clears the ticket words of the projections' split reductions (if this shape has any)
+  const FfnWs fws = carve_ffn(T, k, K, N, dtype);
+  const bool has_tickets = fws.total > fws.split && !router_dispatches;
+  int32_t* tickets = has_tickets ? reinterpret_cast<int32_t*>(base + ws.ffn + fws.split + mfma_ws_tickets_offset()) : nullptr;
+  if (!router_dispatches &&
+      (rc = dispatch_build(idx, T * k, E, counts, offsets, perm, inv, tickets, has_tickets ? mfma_ws_ticket_count() : 0, st)))
+    return rc;
   mark(events, 5, st);
   if ((rc = grouped_ffn_impl(xn, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, z_scale, y,
-                             base + ws.ffn, workspace_bytes - ws.ffn, variant, stream, events ? events + 6 : nullptr)))
+                             base + ws.ffn, workspace_bytes - ws.ffn, variant, stream, events ? events + 6 : nullptr, has_tickets)))
     return rc;
   mark(events, 10, st);
   rc = stmoe_combine(y, gate, inv, dtype, T, k, K, out_norm_w, w_dtype, eps, h, out, stream);

@@ -31,6 +31,7 @@ struct GemmParams {
   const float* out_scale; // fp8 kernel only: quantise the result with this reciprocal scale and store e4m3fn bytes
   int64_t expert_rows_bound;  // host-side bound of rows per expert (a token gives an expert at most one row)
   float* split_scratch;       // optional fp32 scratch for split reductions (mfma_ws_partial_bytes() bytes)
+  bool split_tickets_zeroed;  // the caller vouches that the scratch's ticket words (mfma_ws_tickets_offset()) are zero
 };
 
 // Row range of expert e; without offsets there is one expert with `fixed_rows` rows.
@@ -123,6 +124,8 @@ int launch_mfma_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int
 int launch_mfma_big(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_mfma_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, float* partial, hipStream_t st);
 size_t mfma_ws_partial_bytes();
+size_t mfma_ws_tickets_offset();  // byte offset of the split units' ticket words inside that scratch
+int mfma_ws_ticket_count();
 int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_fp8_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_fp8_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);

@@ -46,7 +46,51 @@ struct WsArgs {
   int n_tiles;
   int wgs_per_xcd;  // grid size / 8
   float* partial;
+  int* tickets;  // one counter per split unit, zero at launch and zero again when the launch is over
 };
+
+// A unit that is split along the reduction is finished by whichever of its chunks is done last: every chunk writes its
+// fp32 partial tile and draws a ticket (an integer atomic), and the workgroup that draws the last one adds the chunks in
+// chunk order, so the sum does not depend on which workgroup that is.  One row of the partial tile (tile rows, then the
+// absorbed tail's rows from BM on) per 8 threads.  DOWN: the sums; GATEUP: the gated product of the gate sums (columns
+// 0..127 of the partial tile) and the up sums (columns 128..255).
+static constexpr size_t kWsSlotFloats = (size_t)256 * (256 + kBigTailRows);
+static constexpr int kWsTickets = 8 * kBigChunkSlotsPerXcd;
+template <typename T, int MODE>
+__device__ __forceinline__ void ws_reduce_row(const GemmParams& p, const BigTile& t, const float* base, int chunks, int r, int c8) {
+  constexpr int BN = 256, BM = 256;
+  const int rows_here = t.row_end - t.row_begin;
+  int sorted_row;
+  if (r < rows_here) sorted_row = t.row_begin + r;
+  else if (r >= BM && r - BM < t.tail_rows) sorted_row = t.tail_begin + (r - BM);
+  else return;
+  base += (size_t)r * BN;
+  auto total = [&](int col) {
+    floatx4_t sum = *reinterpret_cast<const floatx4_t*>(base + col);
+    for (int c = 1; c < chunks; ++c) sum = sum + *reinterpret_cast<const floatx4_t*>(base + (size_t)c * kWsSlotFloats + col);
+    return sum;
+  };
+  T* orow = reinterpret_cast<T*>(p.out) + out_row(p, sorted_row) * p.ldo;
+  if (MODE == MODE_GATEUP) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = (c8 + 8 * j) * 4;
+      const floatx4_t gs = total(col), us = total(BN / 2 + col);
+      const float gq[4] = {gs[0], gs[1], gs[2], gs[3]}, uq[4] = {us[0], us[1], us[2], us[3]};
+      uint2* dst = reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * (BN / 2) + col);
+      if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq);
+      else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int col = (c8 + 8 * j) * 4;
+      const floatx4_t sum = total(col);
+      *reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * BN + col) = make_uint2(pack2<T>(sum[0], sum[1]), pack2<T>(sum[2], sum[3]));
+    }
+  }
+}
+__global__ void ws_zero_tickets_kernel(int* tickets) { tickets[threadIdx.x] = 0; }
 
 template <typename T, int WF, int MODE>
 __global__ void __launch_bounds__(768, 1)
@@ -522,53 +566,27 @@ grouped_mfma_ws_kernel(WsArgs args) {
     if (wave < 8) unit(WsInt<0>{}, WsInt<0>{});
     else unit(WsInt<1>{}, WsInt<0>{});
   }
-  }  // next item
-}
-
-// Adds the chunks of every split unit in chunk order and writes the rows: DOWN: the sums; GATEUP: the gated product of
-// the gate sums (columns 0..127 of the partial tile) and the up sums (columns 128..255).  Grid: (8 XCDs x 16 split
-// units, 8 blocks of 32 rows); the unit list is recomputed with the same plan as the main kernel.
-template <typename T, int MODE, int BALANCE>
-__global__ void __launch_bounds__(256) big_reduce_kernel(GemmParams p, int n_tiles, const float* partial) {
-  constexpr int BN = 256, BM = 256;
-  const int xcd = blockIdx.x >> 4, su = blockIdx.x & 15;
-  const int lane_off = big_lane_offsets(p);
-  const BigPlan pl = big_plan(p, lane_off, BM, n_tiles, xcd, true, true, BALANCE);
-  if (su >= pl.rest) return;
-  BigTile t;
-  if (!big_unit(p, lane_off, BM, n_tiles, pl, pl.whole + su, t, true, BALANCE)) return;
-  const int rows_here = t.row_end - t.row_begin;
-  const int r = blockIdx.y * 32 + (threadIdx.x >> 3);  // row of the partial tile: tile rows, then the absorbed tail's rows from BM on
-  int sorted_row;
-  if (r < rows_here) sorted_row = t.row_begin + r;
-  else if (r >= BM && r - BM < t.tail_rows) sorted_row = t.tail_begin + (r - BM);
-  else return;
-  constexpr size_t kSlot = (size_t)BN * (BM + kBigTailRows);
-  const float* base = partial + (size_t)(xcd * kBigChunkSlotsPerXcd + su * pl.chunks) * kSlot + r * BN;
-  auto total = [&](int col) {
-    floatx4_t sum = *reinterpret_cast<const floatx4_t*>(base + col);
-    for (int c = 1; c < pl.chunks; ++c) sum = sum + *reinterpret_cast<const floatx4_t*>(base + (size_t)c * kSlot + col);
-    return sum;
-  };
-  T* orow = reinterpret_cast<T*>(p.out) + out_row(p, sorted_row) * p.ldo;
-  if (MODE == MODE_GATEUP) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int col = ((threadIdx.x & 7) + 8 * j) * 4;
-      const floatx4_t gs = total(col), us = total(BN / 2 + col);
-      const float gq[4] = {gs[0], gs[1], gs[2], gs[3]}, uq[4] = {us[0], us[1], us[2], us[3]};
-      uint2* dst = reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * (BN / 2) + col);
-      if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq);
-      else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq);
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int col = ((threadIdx.x & 7) + 8 * j) * 4;
-      const floatx4_t sum = total(col);
-      *reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * BN + col) = make_uint2(pack2<T>(sum[0], sum[1]), pack2<T>(sum[2], sum[3]));
+  if (tile.nchunks > 1) {
+    // chunk of a split unit (every wavefront of the workgroup gets here): the workgroup that draws the unit's last ticket
+    // adds the chunks.  Each thread's partial sums are made visible device-wide before the ticket is drawn, and the
+    // drawing workgroup drops what its caches hold before it reads the other chunks.  LDS is free after the unit's last
+    // K step; the next unit's loaders start only after the last barrier below.
+    __threadfence();
+    __syncthreads();
+    int* const drawn_s = reinterpret_cast<int*>(lds);
+    int* const ticket = ka.tickets + (tile.chunk_slot - tile.chunk);
+    if (tid == 0) *drawn_s = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const int drawn = *drawn_s;
+    __syncthreads();
+    if (drawn == tile.nchunks - 1) {
+      __threadfence();
+      const float* base = partial + (size_t)(tile.chunk_slot - tile.chunk) * kWsSlotFloats;
+      for (int r = tid >> 3; r < BM + kBigTailRows; r += 96) ws_reduce_row<T, MODE>(p, tile, base, tile.nchunks, r, tid & 7);
+      if (tid == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // as the launch found it
     }
   }
+  }  // next item
 }
 
 template <typename T, int WF, int MODE>
@@ -583,11 +601,15 @@ static int launch_ws_m(const GemmParams& p, int64_t max_rows, float* partial, hi
   const int m_slots = (int)((max_rows + BM - 1) / BM) + experts;
   // one workgroup per CU (it takes all of the CU's LDS), fewer when an XCD's list cannot be longer than that
   const int per_xcd = std::min(kBigCusPerXcd, big_grid(n_tiles, m_slots, partial != nullptr) / 8);
-  kern<<<dim3((unsigned)(8 * per_xcd)), 768, lds_bytes, st>>>(WsArgs{p, n_tiles, per_xcd, partial});
-  int rc = check_launch("grouped_mfma_ws");
-  if (rc || !partial) return rc;
-  big_reduce_kernel<T, MODE, ws_balance(WF)><<<dim3(8 * 16, (BM + kBigTailRows + 31) / 32), 256, 0, st>>>(p, n_tiles, partial);
-  return check_launch("big_reduce");
+  // the tickets of the split units follow the partial tiles; a launch leaves them at zero, so only a caller that cannot
+  // vouch for the scratch's history has them cleared first
+  int* tickets = partial ? reinterpret_cast<int*>(partial + (size_t)kWsTickets * kWsSlotFloats) : nullptr;
+  if (tickets && !p.split_tickets_zeroed) {
+    ws_zero_tickets_kernel<<<1, kWsTickets, 0, st>>>(tickets);
+    if (int rc = check_launch("ws_zero_tickets")) return rc;
+  }
+  kern<<<dim3((unsigned)(8 * per_xcd)), 768, lds_bytes, st>>>(WsArgs{p, n_tiles, per_xcd, partial, tickets});
+  return check_launch("grouped_mfma_ws");
 }
 
 template <typename T, int WF>
@@ -596,7 +618,9 @@ static int launch_ws_t(int mode, const GemmParams& p, int64_t max_rows, float* p
                              : launch_ws_m<T, WF, MODE_DOWN>(p, max_rows, partial, st);
 }
 
-size_t mfma_ws_partial_bytes() { return big_partial_bytes(256, 256); }
+size_t mfma_ws_partial_bytes() { return big_partial_bytes(256, 256) + kWsTickets * sizeof(int); }
+size_t mfma_ws_tickets_offset() { return big_partial_bytes(256, 256); }
+int mfma_ws_ticket_count() { return kWsTickets; }
 
 // `partial`: optional fp32 scratch of mfma_ws_partial_bytes() bytes; with it the last units of a launch, which would
 // run on a few CUs only, are split along the reduction.

@@ -1,7 +1,7 @@
 // RMS norm and the router (logits, softmax, top-k, gate renormalisation) of MoeBlock.forward
 // (sharktank/sharktank/layers/mixture_of_experts_block.py:68-83, norm.py:34-41,
 //  sharktank/sharktank/ops/default_impls.py:328-359,402-408).
-#include "stmoe_common.h"
+#include "weights.h"
 
 namespace stmoe {
 
@@ -87,44 +87,12 @@ template <> struct Vec8<bf16_t> {
   }
 };
 
+// fp32 softmax over the E logits, top-k of the probabilities and renormalised gates of one token, computed alike by
+// every lane from the logits lg[0..E) (already rounded to T); lane 0 writes.
 template <typename T, int EP>
-__global__ void __launch_bounds__(256)
-router_topk_kernel(const T* __restrict__ x, const T* __restrict__ wr, int64_t T_tokens, int64_t K, int E, int k,
-                   T* __restrict__ logits_out, int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out,
-                   T* __restrict__ gate_out) {
-  const int lane = threadIdx.x & 63;
-  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (t >= T_tokens) return;
-  const T* xr = x + t * K;
-
-  float acc[EP];
-#pragma unroll
-  for (int e = 0; e < EP; ++e) acc[e] = 0.0f;
-
-  for (int64_t k0 = (int64_t)lane * 8; k0 < K; k0 += 512) {
-    Vec8<T> xv;
-    xv.load(xr + k0);
-#pragma unroll
-    for (int e = 0; e < EP; ++e) {
-      if (e < E) {
-        Vec8<T> wv;
-        wv.load(wr + (int64_t)e * K + k0);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[e] = __fadd_rn(acc[e], __fmul_rn(xv.v[j], wv.v[j]));
-      }
-    }
-  }
-
-  float lg[EP];
-#pragma unroll
-  for (int e = 0; e < EP; ++e) lg[e] = (e < E) ? round_to<T>(wave_xor_sum(acc[e])) : -INFINITY;
-
-  if (logits_out) {
-#pragma unroll
-    for (int e = 0; e < EP; ++e)
-      if (e < E && lane == (e & 63)) logits_out[t * E + e] = Cvt<T>::from_f32(lg[e]);
-  }
-
+__device__ __forceinline__ void softmax_topk_store(const float (&lg)[EP], int E, int k, int64_t t, int lane,
+                                                   int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out,
+                                                   T* __restrict__ gate_out) {
   // fp32 softmax over the E logits (F.softmax(dim=1, dtype=float)).
   float mx = lg[0];
 #pragma unroll
@@ -173,6 +141,47 @@ router_topk_kernel(const T* __restrict__ x, const T* __restrict__ wr, int64_t T_
   }
 }
 
+template <typename T, int EP>
+__global__ void __launch_bounds__(256)
+router_topk_kernel(const T* __restrict__ x, const T* __restrict__ wr, int64_t T_tokens, int64_t K, int E, int k,
+                   T* __restrict__ logits_out, int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out,
+                   T* __restrict__ gate_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T_tokens) return;
+  const T* xr = x + t * K;
+
+  float acc[EP];
+#pragma unroll
+  for (int e = 0; e < EP; ++e) acc[e] = 0.0f;
+
+  for (int64_t k0 = (int64_t)lane * 8; k0 < K; k0 += 512) {
+    Vec8<T> xv;
+    xv.load(xr + k0);
+#pragma unroll
+    for (int e = 0; e < EP; ++e) {
+      if (e < E) {
+        Vec8<T> wv;
+        wv.load(wr + (int64_t)e * K + k0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[e] = __fadd_rn(acc[e], __fmul_rn(xv.v[j], wv.v[j]));
+      }
+    }
+  }
+
+  float lg[EP];
+#pragma unroll
+  for (int e = 0; e < EP; ++e) lg[e] = (e < E) ? round_to<T>(wave_xor_sum(acc[e])) : -INFINITY;
+
+  if (logits_out) {
+#pragma unroll
+    for (int e = 0; e < EP; ++e)
+      if (e < E && lane == (e & 63)) logits_out[t * E + e] = Cvt<T>::from_f32(lg[e]);
+  }
+
+  softmax_topk_store<T, EP>(lg, E, k, t, lane, idx_out, idx64_out, gate_out);
+}
+
 // ---------------------------------------------------------------------------------------------------
 // router, one workgroup (8 wavefronts) per token, optionally fused with the preceding RMS norm.
 //
@@ -187,8 +196,8 @@ struct SingleTokenDispatch {
   int32_t *counts, *offsets, *perm, *inv;
 };
 
-template <typename T, typename W, bool FUSE_NORM, int PRE>
-__global__ void __launch_bounds__(512, PRE ? 4 : 8)
+template <typename T, typename W, bool FUSE_NORM, int PRE, bool LATE>
+__global__ void __launch_bounds__(512, (PRE && !LATE) ? 4 : 8)
 router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float eps, T* __restrict__ xn,
                  const T* __restrict__ wr, int64_t K, int E, int k, T* __restrict__ logits_out,
                  int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out, T* __restrict__ gate_out,
@@ -205,24 +214,29 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
   // latency runs in parallel with the norm (they do not depend on it).  PRE chunks of 512 elements are kept in registers.
   // Rows of at least NC * 512 elements (the usual case) take their first loads without a bounds test per load: loads
   // under separate conditions are waited for one by one, those of a straight line are all in flight together.
-  // PRE = 8 (a whole row of 4096) for launches of at most 64 tokens and 4 up to 512 tokens (latency); PRE = 0 for more
-  // tokens, where the 16 registers of the prefetch cost a quarter of the workgroups a CU can hold and throughput counts.
+  // PRE = 8 (a whole row of 4096) for launches of at most 64 tokens and 4 up to 512 tokens (latency).  Launches of more
+  // tokens, where throughput counts and the prefetch registers held through the norm would cost a quarter of the
+  // workgroups a CU can hold, request the same 8 chunks only after the norm's registers are free (LATE), in front of the
+  // barrier that ends the norm: all in flight together, where a loop over the chunks waits for them one by one.
   constexpr int NC = 8;
   const bool long_row = K >= (int64_t)NC * 512;
   uint4 wpre[PRE ? PRE : 1];
-  if (PRE > 0 && sizeof(T) == 2 && wave < E) {  // 16-bit rows (a chunk of 8 elements is one 16-byte load)
-    const T* wrow = wr + (int64_t)wave * K;
-    if (long_row) {
+  auto prefetch = [&]() {
+    if (PRE > 0 && sizeof(T) == 2 && wave < E) {  // 16-bit rows (a chunk of 8 elements is one 16-byte load)
+      const T* wrow = wr + (int64_t)wave * K;
+      if (long_row) {
 #pragma unroll
-      for (int j = 0; j < PRE; ++j) wpre[j] = *reinterpret_cast<const uint4*>(wrow + lane * 8 + j * 512);
-    } else {
+        for (int j = 0; j < PRE; ++j) wpre[j] = *reinterpret_cast<const uint4*>(wrow + lane * 8 + j * 512);
+      } else {
 #pragma unroll
-      for (int j = 0; j < PRE; ++j) {
-        const int64_t k0 = (int64_t)lane * 8 + (int64_t)j * 512;
-        if (k0 < K) wpre[j] = *reinterpret_cast<const uint4*>(wrow + k0);
+        for (int j = 0; j < PRE; ++j) {
+          const int64_t k0 = (int64_t)lane * 8 + (int64_t)j * 512;
+          if (k0 < K) wpre[j] = *reinterpret_cast<const uint4*>(wrow + k0);
+        }
       }
     }
-  }
+  };
+  if constexpr (!LATE) prefetch();
   if constexpr (FUSE_NORM) {
     // the row's elements tid + 512 j are read once and kept (NC of them) for the second pass; the norm weights are
     // requested before the reduction
@@ -285,6 +299,7 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
       for (int64_t i = (int64_t)tid * 8 + 4; i < K; i += 512 * 8)
         *reinterpret_cast<uint4*>(&xs[i]) = *reinterpret_cast<const uint4*>(&xr[i]);
   }
+  if constexpr (LATE) prefetch();
   __syncthreads();
 
   for (int e = wave; e < E; e += 8) {
@@ -307,7 +322,17 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
         else chunk(k0, nullptr);
       }
     }
-    for (int64_t k0 = (int64_t)lane * 8 + (int64_t)PRE * 512; k0 < K; k0 += 512) chunk(k0, nullptr);
+    int64_t k0 = (int64_t)lane * 8 + (int64_t)PRE * 512;
+    if constexpr (sizeof(T) == 2) {
+      for (; k0 + 3 * 512 < K; k0 += 4 * 512) {  // four chunks requested together, added in increasing order as before
+        uint4 wb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) wb[j] = *reinterpret_cast<const uint4*>(wrow + k0 + j * 512);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) chunk(k0 + j * 512, &wb[j]);
+      }
+    }
+    for (; k0 < K; k0 += 512) chunk(k0, nullptr);
     const float l = round_to<T>(wave_xor_sum(acc));
     if (lane == 0) {
       lg_s[e] = l;
@@ -373,6 +398,170 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// ffn_norm + router, one wavefront per token: for launches of many tokens, where the workgroup-per-token kernel above
+// holds four tokens per CU at a time and every token pays its chain of latencies (row, reduction, barrier, router rows,
+// barrier, softmax) in one of two or more rounds.  Here a CU holds a token per wavefront, all tokens of a usual prefill
+// launch are in flight at once, and nothing waits at a barrier.  Same bits as rms_norm_kernel + router_topk_kernel:
+//   * sum of squares: rms_norm_kernel's thread j adds elements j, j + 512, ...; its wavefront v is threads 64 v .. 64 v + 63.
+//     Lane l here plays thread l + 64 v of every wavefront v = 0..7 in turn: eight running sums over the elements
+//     l + 64 v + 512 c in increasing c, eight xor butterflies, and the eight wavefront sums combined in the same order;
+//   * a logit is a wavefront's sum anyway (lane-owned pieces of 8 elements per chunk of 512, then the butterfly).
+// The row is fetched once in the router's layout (16 bytes per lane and chunk); the norm reads its elements in thread
+// order through the wavefront's own piece of LDS; the normalised row is computed, stored and multiplied in the
+// router's layout again (normalisation is elementwise).  16-bit rows of NCH * 512 elements.
+//
+// fp16: a product of two fp16 numbers is exact in fp32 (22 significant bits, exponents far inside the fp32 range), so a
+// fused multiply-add rounds once exactly where the separate multiply and add round: same bits, fewer instructions.  bf16
+// products can fall into the fp32 subnormal range, where the separate multiply would round: they keep both steps.
+template <typename T> __device__ __forceinline__ float mul_add_like_separate(float acc, float a, float b) {
+  if constexpr (__is_same(T, f16_t)) return __fmaf_rn(a, b, acc);
+  else return __fadd_rn(acc, __fmul_rn(a, b));
+}
+
+template <typename T, typename W, int NCH, int EP>
+__global__ void __launch_bounds__(256)
+norm_router_wave_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float eps, T* __restrict__ xn,
+                        const T* __restrict__ wr, int64_t T_tokens, int E, int k, int32_t* __restrict__ idx_out,
+                        T* __restrict__ gate_out) {
+  static_assert(sizeof(T) == 2, "16-bit rows");
+  constexpr int K = NCH * 512;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
+  if (t >= T_tokens) return;  // (no barrier in this kernel: every wavefront works on its own piece of LDS)
+  uint4* const xs4 = reinterpret_cast<uint4*>(smem) + wave * (K / 8);
+  const T* const xs = reinterpret_cast<const T*>(xs4);
+  const uint4* const xr4 = reinterpret_cast<const uint4*>(x + t * K);
+  uint4 raw[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) raw[c] = xr4[c * 64 + lane];
+  // What does not depend on the row is requested right behind it, so that its latency runs beside the row's: the first
+  // expert's router row and the first norm weights.  Loads are issued a whole batch at a time throughout: the wavefront
+  // has nobody to hide a latency behind, and loads requested one by one are waited for one by one.
+  constexpr int NWB = 4;                 // chunks per batch of norm weights
+  constexpr bool DOUBLE = NCH <= 8;      // two router-row buffers (the next expert's row is fetched during this one's sums)
+  auto load_router_row = [&](uint4 (&dst)[NCH], int e) {
+    const uint4* const w4 = reinterpret_cast<const uint4*>(wr + (int64_t)e * K);
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) dst[c] = w4[c * 64 + lane];
+  };
+  auto load_norm_weights = [&](Vec8<W> (&dst)[NWB], int c0) {
+#pragma unroll
+    for (int i = 0; i < NWB; ++i) dst[i].load(norm_w + ((c0 + i) * 64 + lane) * 8);
+  };
+  uint4 wa[NCH], wb[DOUBLE ? NCH : 1];
+  Vec8<W> nw[NWB];
+  load_router_row(wa, 0);
+  load_norm_weights(nw, 0);
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) xs4[c * 64 + lane] = raw[c];
+  __builtin_amdgcn_wave_barrier();  // (a wavefront's LDS accesses are served in program order)
+
+  float sv[8];
+#pragma unroll
+  for (int v = 0; v < 8; ++v) sv[v] = 0.0f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c)
+#pragma unroll
+    for (int v = 0; v < 8; ++v) {
+      const float e = Cvt<T>::to_f32(xs[lane + 64 * v + 512 * c]);
+      sv[v] = mul_add_like_separate<T>(sv[v], e, e);
+    }
+#pragma unroll
+  for (int v = 0; v < 8; ++v) sv[v] = wave_xor_sum(sv[v]);
+  const float total = ((sv[0] + sv[1]) + (sv[2] + sv[3])) + ((sv[4] + sv[5]) + (sv[6] + sv[7]));
+  const float rs = rms_scale(total, K, eps);
+
+  float xf[NCH][8];  // the normalised row as the router multiplies it: values of T
+  uint4* const xn4 = reinterpret_cast<uint4*>(xn + t * K);
+#pragma unroll
+  for (int c0 = 0; c0 < NCH; c0 += NWB) {
+    if (c0 > 0) load_norm_weights(nw, c0);
+#pragma unroll
+    for (int i = 0; i < NWB; ++i) {
+      const int c = c0 + i;
+      Vec8<T> xv;
+      xv.from_raw(raw[c]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float o = round_to<W>(keep_f32(__fmul_rn(xv.v[j], rs)));
+        o = round_to<W>(keep_f32(__fmul_rn(nw[i].v[j], o)));
+        xf[c][j] = round_to<T>(o);
+      }
+      xn4[c * 64 + lane] = make_uint4(pack2<T>(xf[c][0], xf[c][1]), pack2<T>(xf[c][2], xf[c][3]), pack2<T>(xf[c][4], xf[c][5]),
+                                      pack2<T>(xf[c][6], xf[c][7]));
+    }
+  }
+
+  float lg[EP];
+  auto logit = [&](const uint4 (&w)[NCH]) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      Vec8<T> wv;
+      wv.from_raw(w[c]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc = mul_add_like_separate<T>(acc, xf[c][j], wv.v[j]);
+    }
+    return round_to<T>(wave_xor_sum(acc));
+  };
+#pragma unroll
+  for (int e = 0; e < EP; ++e) {
+    lg[e] = -INFINITY;
+    if (e < E) {
+      if constexpr (DOUBLE) {
+        // expert e sits in wa (even e) or wb (odd e); the other buffer takes expert e + 1 meanwhile
+        if (e % 2 == 0) {
+          if (e + 1 < E) load_router_row(wb, e + 1);
+          lg[e] = logit(wa);
+        } else {
+          if (e + 1 < E) load_router_row(wa, e + 1);
+          lg[e] = logit(wb);
+        }
+      } else {
+        if (e > 0) load_router_row(wa, e);
+        lg[e] = logit(wa);
+      }
+    }
+  }
+  softmax_topk_store<T, EP>(lg, E, k, t, lane, idx_out, nullptr, gate_out);
+}
+
+// Whether the wavefront-per-token kernel takes this launch (16-bit rows of 2048, 4096, 6144 or 8192 elements, at most 16
+// experts, 16-byte aligned operands); launches of fewer tokens keep the workgroup-per-token kernel, whose eight
+// wavefronts share a token's work and finish it sooner.
+static constexpr int64_t kWaveRouterMinTokens = 768;  // (measured at 4096-element rows: 14 us against 13.5 at 512 tokens, 16 against 18 at 1024, 17 against 25 at 2048)
+template <typename T, typename W>
+static bool launch_norm_router_wave(const void* x, const void* norm_w, float eps, void* xn, const void* wr, int64_t T_tokens,
+                                    int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st) {
+  if constexpr (sizeof(T) != 2) {
+    return false;
+  } else {
+    if (T_tokens < kWaveRouterMinTokens || E > 16 || K % 2048 != 0 || K > 8192) return false;
+    if (!aligned16(x) || !aligned16(norm_w) || !aligned16(xn) || !aligned16(wr)) return false;
+    const dim3 grid((unsigned)((T_tokens + 3) / 4));
+    const size_t lds = (size_t)4 * K * 2;
+#define STMOE_NRW(NCH, EP)                                                                                              \
+  norm_router_wave_kernel<T, W, NCH, EP><<<grid, 256, lds, st>>>((const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, \
+                                                                 T_tokens, E, k, idx, (T*)gate)
+#define STMOE_NRW_E(NCH)      \
+  do {                        \
+    if (E <= 8) STMOE_NRW(NCH, 8); \
+    else STMOE_NRW(NCH, 16);  \
+  } while (0)
+    switch (K / 512) {
+      case 4: STMOE_NRW_E(4); break;
+      case 8: STMOE_NRW_E(8); break;
+      case 12: STMOE_NRW_E(12); break;
+      default: STMOE_NRW_E(16); break;
+    }
+#undef STMOE_NRW_E
+#undef STMOE_NRW
+    return true;
+  }
+}
+
 template <typename T, typename W, bool FUSE_NORM>
 static int launch_router_wg(const void* x, const void* norm_w, float eps, void* xn, const void* wr, int64_t T_tokens,
                             int64_t K, int E, int k, void* logits, int32_t* idx, int64_t* idx64, void* gate, hipStream_t st,
@@ -380,13 +569,13 @@ static int launch_router_wg(const void* x, const void* norm_w, float eps, void* 
   const size_t lds = ((K * sizeof(T) + 15) / 16) * 16 + (64 + 8 + 64) * sizeof(float);
   if (lds > 64 * 1024) return set_error(STMOE_ERR_UNSUPPORTED, "router: K=%lld does not fit the per-token LDS row", (long long)K);
   if (T_tokens <= 64)
-    router_wg_kernel<T, W, FUSE_NORM, 8><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
+    router_wg_kernel<T, W, FUSE_NORM, 8, false><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
         (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
   else if (T_tokens <= 512)
-    router_wg_kernel<T, W, FUSE_NORM, 4><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
+    router_wg_kernel<T, W, FUSE_NORM, 4, false><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
         (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
   else
-    router_wg_kernel<T, W, FUSE_NORM, 0><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
+    router_wg_kernel<T, W, FUSE_NORM, 0, true><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
         (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
   return check_launch("router_wg");
 }
@@ -398,7 +587,11 @@ int norm_router(const void* h, int dtype, const void* norm_w, int w_dtype, float
                 int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv) {
   SingleTokenDispatch disp{nullptr, nullptr, nullptr, nullptr};
   if (T_tokens == 1 && counts && offsets && perm && inv) disp = SingleTokenDispatch{counts, offsets, perm, inv};
-#define STMOE_NR(TT, WW) return launch_router_wg<TT, WW, true>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, nullptr, idx, nullptr, gate, st, disp)
+#define STMOE_NR(TT, WW)                                                                                                   \
+  do {                                                                                                                     \
+    if (launch_norm_router_wave<TT, WW>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, idx, gate, st)) return check_launch("norm_router_wave"); \
+    return launch_router_wg<TT, WW, true>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, nullptr, idx, nullptr, gate, st, disp); \
+  } while (0)
   if (dtype == STMOE_F32 && w_dtype == STMOE_F32) STMOE_NR(float, float);
   if (dtype == STMOE_F16 && w_dtype == STMOE_F32) STMOE_NR(f16_t, float);
   if (dtype == STMOE_BF16 && w_dtype == STMOE_F32) STMOE_NR(bf16_t, float);

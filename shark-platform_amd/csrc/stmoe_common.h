@@ -18,6 +18,10 @@ int norm_router(const void* h, int dtype, const void* norm_w, int w_dtype, float
                 int64_t T_tokens, int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st,
                 int32_t* counts = nullptr, int32_t* offsets = nullptr, int32_t* perm = nullptr, int32_t* inv = nullptr);
 
+// stmoe_dispatch_build that also clears `n_zero` (at most 1024) 32-bit words at `zero_words` (nullable).
+int dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv,
+                   int32_t* zero_words, int n_zero, hipStream_t st);
+
 #define STMOE_REQUIRE(cond, code, ...)            \
   do {                                            \
     if (!(cond)) return ::stmoe::set_error((code), __VA_ARGS__); \

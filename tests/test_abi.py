@@ -81,3 +81,30 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_hip, "_LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="is missing"):
         _hip.load_library()
+
+
+def test_hand_scheduled_kernels_get_no_scratch_accesses_from_the_compiler():
+    """The prefill kernels issue their loads by hand and wait for them with counted `s_waitcnt vmcnt(N)`.  That count only
+    holds while the compiler adds no vector-memory instruction of its own to those wavefronts: a register spilled to scratch
+    memory would be one (and a spill of a register with a load in flight would read it too early).  The build keeps the
+    compiler's per-kernel resource report beside the library; every instance of those kernels must show no scratch and no
+    spilled vector register."""
+    from sharktank_amd import _hip
+
+    report = os.path.splitext(_hip.library_path())[0] + ".resources.txt"
+    assert os.path.exists(report), f"{report} is missing: build with the Makefile (make -C shark-platform_amd/csrc)"
+    kernels, name = {}, None
+    for line in open(report):
+        key, _, value = line.strip().partition(": ")
+        if key == "Function Name":
+            name = value
+            kernels[name] = {}
+        elif name is not None:
+            kernels[name][key] = value
+    hand = {n: r for n, r in kernels.items() if "grouped_mfma_ws_kernel" in n or "grouped_fp8_ws_kernel" in n}
+    assert len(hand) >= 12 + 2, sorted(hand)  # 2 dtypes x 3 formats x 2 modes, and the fp8 x fp8 kernel
+    for n, r in hand.items():
+        assert r["ScratchSize [bytes/lane]"] == "0", (n, r)
+        assert r["VGPRs Spill"] == "0", (n, r)
+        if "grouped_mfma_ws_kernel" in n:
+            assert int(r["VGPRs"]) <= 168, (n, r)  # 12 wavefronts per CU

@@ -371,3 +371,44 @@ def test_small_batch_forward_equals_staged_calls(device, T, E, k):
     staged = _hip.combine(y, gate, inv, T, k, residual=h)
     for got in (fused, again, third):
         assert torch.equal(staged.view(torch.int16), got.reshape(T, case.K).view(torch.int16))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("norm_in_act_dtype", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T,K,E,k", [(256, 2048, 8, 2), (301, 4096, 8, 2), (2051, 4096, 8, 2), (515, 6144, 16, 4), (260, 8192, 3, 3)])
+def test_prefill_front_end_equals_staged_calls(device, dtype, T, K, E, k, norm_in_act_dtype):
+    """Launches of many tokens run ffn_norm + router with one wavefront per token (rows of 2048 / 4096 / 6144 / 8192
+    elements).  Its normalised rows, routing indices and gates must have the bits of rms_norm + router_topk called one
+    after the other (whose own bits the oracle's ordered restatements pin), and so must the layer output."""
+    from sharktank_amd import _hip
+    from sharktank_amd import types as ST
+    from sharktank_amd.layers import MoeBlock
+    from sharktank_amd.types import unbox_tensor
+
+    case = MC.build(MC.Case(T=T, K=K, N=256, E=E, k=k, fmt="q8_0", dtype=dtype, seed=900 + T + E))
+    if T == 301 and dtype == torch.float16:
+        case.planes["h"][:7] *= 1e-4  # rows whose squares and products reach down to fp16 subnormals
+        case.planes["h"][7:9] *= 200.0
+    theta = MC.make_theta(case, device)
+    if norm_in_act_dtype:
+        flat = theta.flatten()
+        flat["ffn_norm.weight"] = ST.DefaultPrimitiveTensor(name="ffn_norm.weight", data=case.planes["ffn_norm"].to(dtype).to(device))
+        theta = ST.Theta(flat)
+    block = MoeBlock(theta, expert_count=E, expert_used_count=k, rms_epsilon=case.eps)
+    wg, wu, wd = block.experts.device_weights()
+    h = case.planes["h"].to(device)
+    fused, idx_f, gate_f = block(h.reshape(1, T, K), return_routing=True)
+
+    norm_w = unbox_tensor(block.ffn_norm.weight)
+    xn = _hip.rms_norm(h, norm_w, case.eps)
+    if not norm_in_act_dtype:  # (the oracle restates the fp32-weight form)
+        want_xn = O.rms_norm_ordered(case.planes["h"], case.planes["ffn_norm"], case.eps)
+        assert torch.equal(xn.cpu().view(torch.int16), want_xn.view(torch.int16))
+    idx, gate, _ = _hip.router_topk(xn, block._router_weight(dtype), k)
+    assert torch.equal(idx.cpu().to(torch.int64), idx_f.cpu().to(torch.int64))
+    assert torch.equal(gate.view(torch.int16), gate_f.view(torch.int16))
+    counts, offsets, perm, inv = _hip.dispatch_build(idx, E)
+    y = _hip.grouped_ffn(xn, wg, wu, wd, block.experts._act, offsets, perm, k)
+    staged = _hip.combine(y, gate, inv, T, k, residual=h)
+    assert torch.equal(staged.view(torch.int16), fused.reshape(T, K).view(torch.int16))
