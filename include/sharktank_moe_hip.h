@@ -140,7 +140,8 @@ int stmoe_dequant_tensor_scaled_per_axis(const void* qs, int qs_dtype, const voi
                                          int out_dtype, stmoe_stream_t stream);
 
 /* DynamicScaledQuantizer._quantize_raw_tensor for float8_e4m3fn (sharktank/sharktank/types/quantizers.py:368-389):
- * amax = max|x|; scale = T(448 / max(amax, eps)), eps = finfo(float8_e4m3fn).eps = 0.125; rscale = T(1 / scale);
+ * amax = max|x|; scale = T(T(1 / max(amax, eps)) * 448) (torch evaluates the reference's `finfo.max / amax.clamp(eps)`, a
+ * number over a tensor, as reciprocal times number), eps = finfo(float8_e4m3fn).eps = 0.125; rscale = T(1 / scale);
  * out = e4m3fn(clamp(T(x * scale))), every step in x's dtype T as eager torch computes it.  scale_rscale_out receives
  * {scale, rscale} (the T values, widened to fp32); `scratch` is device memory of at least
  * stmoe_dynamic_quantize_fp8_scratch_bytes() bytes.  Two launches, no synchronisation. */
@@ -220,14 +221,32 @@ size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int64_t K, int
  * (variant 7: the same arithmetic on the general 128x128 tile kernel only).
  * x itself is always given unquantised in `dtype`.
  * `perm` may be NULL when k == 1 and the rows of x are already grouped by expert (sorted row i is row i of x): with
- * E == 1 and offsets {0, T} this is the plain feed-forward network of one expert (FFNMOE,
- * sharktank/sharktank/layers/ffn_moe_block.py:77-127).
+ * E == 1 this is the plain feed-forward network of one expert (FFNMOE,
+ * sharktank/sharktank/layers/ffn_moe_block.py:77-127; FFN, sharktank/sharktank/layers/ffn_block.py:21-51), and `offsets`
+ * may then be NULL (the expert owns all T rows): no device array has to be built for the call.
  * `variant` 0 picks the kernel by shape; other values force one (see the kernel list in ffn.hip). */
 int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                       const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
                       int act, const int32_t* offsets, const int32_t* perm, const float* x_scale /*nullable*/,
                       const float* z_scale /*nullable*/, void* y_sorted, void* workspace, size_t workspace_bytes,
                       int variant, stmoe_stream_t stream);
+
+/* The two halves of stmoe_grouped_ffn as calls of their own, for callers that need the gated intermediate between them:
+ * a dynamic or per-axis quantizer of the input of `ffn_down_exps` (DynamicScaledQuantizer,
+ * sharktank/sharktank/types/quantizers.py:338-389; LinearLayer applies a q_input in front of its matmul,
+ * sharktank/sharktank/layers/linear.py:72-78) needs the whole intermediate before it can scale any of it.
+ *   stmoe_grouped_gate_up: z[i,:] = act(Wg[e] . x[t]) * (Wu[e] . x[t]) for every sorted position i; z [T*k, N] in `dtype`,
+ *                          rows in dispatch order.  x_scale as in stmoe_grouped_ffn.
+ *   stmoe_grouped_down:    y[i,:] = Wd[e] . z[i,:]; z is read as it is (the caller has quantised and dequantised it if it
+ *                          wants that; a scale it computed stays in device memory, nothing comes back to the host).
+ * Workspace: stmoe_grouped_ffn_workspace_bytes(T, k, K, N, dtype) for either.  Variants 5 and 7 are not available here. */
+int stmoe_grouped_gate_up(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                          const stmoe_weight* w_gate, const stmoe_weight* w_up, int act, const int32_t* offsets,
+                          const int32_t* perm, const float* x_scale /*nullable*/, void* z_sorted, void* workspace,
+                          size_t workspace_bytes, int variant, stmoe_stream_t stream);
+int stmoe_grouped_down(const void* z_sorted, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                       const stmoe_weight* w_down, const int32_t* offsets, void* y_sorted, void* workspace,
+                       size_t workspace_bytes, int variant, stmoe_stream_t stream);
 
 /* One gathered-expert projection over all (token, slot) pairs, without the [T,k,rows,cols] weight gather of
  * `weights[experts]` + einsum_2args (ffn_moe_block.py:37-41; sharktank/sharktank/ops/default_impls.py:72-94):
@@ -239,6 +258,19 @@ int stmoe_grouped_mmt(const void* a, int dtype, int64_t T, int k, int a_per_pair
 
 /* out[r, :] = g[r] * y[r, :] rounded to `dtype`: einsum "me,men->men" (default_impls.py:97-105) on flattened pairs. */
 int stmoe_scale_rows(const void* y, const void* g, int dtype, int64_t rows, int64_t K, void* out, stmoe_stream_t stream);
+
+/* out[r, c] = y[r, c] + bias[c]: the bias of `linear` (sharktank/sharktank/ops/default_impls.py:328-341, `result + bias`).
+ * y [rows, cols]; dtypes F32/F16/BF16; out_dtype must be torch's promotion of the two (equal dtypes stay, mixed ones
+ * give F32); operands are widened to fp32, added, rounded once.  out may alias y when the dtypes are equal. */
+int stmoe_add_bias(const void* y, int y_dtype, const void* bias, int bias_dtype, int64_t rows, int64_t cols, void* out,
+                   int out_dtype, stmoe_stream_t stream);
+
+/* softmax over the last axis of x [rows, cols] (`ops.softmax`, sharktank/sharktank/ops/signatures.py:974-993, default
+ * implementation F.softmax, default_impls.py:426-432; MoeBlock applies it to the router logits with dtype=float,
+ * mixture_of_experts_block.py:72-74): values widened to fp32, p = expf(x - max) / sum, rounded to out_dtype.  Rows of at
+ * most 64 elements are summed in index order, as the router kernel sums them: ranking these probabilities reproduces
+ * stmoe_router_topk's choice bit for bit. */
+int stmoe_softmax(const void* x, int x_dtype, int64_t rows, int64_t cols, void* out, int out_dtype, stmoe_stream_t stream);
 
 /* Weighted combine (ffn_moe_block.py:73-74) and the layer tail (mixture_of_experts_block.py:86-90):
  *   o[t,:] = sum_j round(gate[t,j] * y[inv[t*k+j],:])   (slot order, fp32 sum, rounded to `dtype`)

@@ -120,8 +120,10 @@ absmax_partial_kernel(const T* __restrict__ x, int64_t n, float* __restrict__ pa
   }
 }
 // Pass 2: every workgroup folds the partial maxima itself (a few KB from L2), derives the scale as eager torch does in
-// x's dtype T -- scale = T(448 / max(amax, eps)), rscale = T(1 / scale), eps = finfo(float8_e4m3fn).eps = 0.125 -- and
-// quantises its elements: e4m3fn(clamp(T(x * scale))).
+// x's dtype T -- scale = T(T(1 / max(amax, eps)) * 448), rscale = T(1 / scale), eps = finfo(float8_e4m3fn).eps = 0.125 -- and
+// quantises its elements: e4m3fn(clamp(T(x * scale))).  (The reference writes `finfo.max / amax.clamp(eps)`, a Python
+// number divided by a tensor, which torch evaluates as `tensor.reciprocal() * number`: two roundings in T, not one
+// division.  amax = 4.8867 in fp16 gives 91.625 that way and 91.6875 as a quotient.)
 template <typename T>
 __global__ void __launch_bounds__(256)
 dynamic_quantize_fp8_kernel(const T* __restrict__ x, int64_t n, const float* __restrict__ partial, int n_partial,
@@ -141,7 +143,7 @@ dynamic_quantize_fp8_kernel(const T* __restrict__ x, int64_t n, const float* __r
   float amax = red[0];
   for (int w = 1; w < 4; ++w) amax = (amax != amax || red[w] != red[w]) ? __uint_as_float(0x7fc00000u) : fmaxf(amax, red[w]);
   const float clamped = amax != amax ? amax : fmaxf(amax, 0.125f);
-  const float scale = round_to<T>(__fdiv_rn(448.0f, clamped));
+  const float scale = round_to<T>(keep_f32(__fmul_rn(round_to<T>(__fdiv_rn(1.0f, clamped)), 448.0f)));
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     scale_rscale[0] = scale;
     scale_rscale[1] = round_to<T>(__fdiv_rn(1.0f, scale));

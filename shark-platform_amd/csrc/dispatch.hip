@@ -249,6 +249,30 @@ int dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, 
   return check_launch("dispatch_build");
 }
 
+// out[r, c] = O(y[r, c] + bias[c]): the bias add of `linear` (sharktank/sharktank/ops/default_impls.py:328-341), each
+// operand widened to fp32 (exact), one fp32 add, one rounding to the promoted dtype O, as eager torch computes it.
+__device__ __forceinline__ float load_f32(const void* p, int dtype, int64_t i) {
+  switch (dtype) {
+    case STMOE_F16: return (float)reinterpret_cast<const f16_t*>(p)[i];
+    case STMOE_BF16: return bf16_to_f32(reinterpret_cast<const bf16_t*>(p)[i]);
+    default: return reinterpret_cast<const float*>(p)[i];
+  }
+}
+__device__ __forceinline__ void store_f32(void* p, int dtype, int64_t i, float v) {
+  switch (dtype) {
+    case STMOE_F16: reinterpret_cast<f16_t*>(p)[i] = (f16_t)v; break;
+    case STMOE_BF16: reinterpret_cast<bf16_t*>(p)[i] = f32_to_bf16(v); break;
+    default: reinterpret_cast<float*>(p)[i] = v; break;
+  }
+}
+__global__ void __launch_bounds__(256)
+add_bias_kernel(const void* __restrict__ y, int y_dtype, const void* __restrict__ bias, int b_dtype, int64_t cols,
+                void* __restrict__ out, int o_dtype) {
+  const int64_t r = blockIdx.x;
+  for (int64_t c = threadIdx.x; c < cols; c += 256)
+    store_f32(out, o_dtype, r * cols + c, __fadd_rn(load_f32(y, y_dtype, r * cols + c), load_f32(bias, b_dtype, c)));
+}
+
 }  // namespace stmoe
 
 using namespace stmoe;
@@ -267,6 +291,20 @@ extern "C" int stmoe_scale_rows(const void* y, const void* g, int dtype, int64_t
     default: return set_error(STMOE_ERR_DTYPE, "scale_rows: dtype %d is not f32/f16/bf16", dtype);
   }
   return check_launch("scale_rows");
+}
+
+extern "C" int stmoe_add_bias(const void* y, int y_dtype, const void* bias, int bias_dtype, int64_t rows, int64_t cols, void* out,
+                              int out_dtype, stmoe_stream_t stream) {
+  STMOE_REQUIRE(rows >= 0 && cols > 0 && rows < 0x7fffffffLL, STMOE_ERR_SHAPE, "add_bias: rows=%lld cols=%lld", (long long)rows, (long long)cols);
+  auto is_float = [](int d) { return d == STMOE_F32 || d == STMOE_F16 || d == STMOE_BF16; };
+  STMOE_REQUIRE(is_float(y_dtype) && is_float(bias_dtype) && is_float(out_dtype), STMOE_ERR_DTYPE, "add_bias: dtypes %d + %d -> %d", y_dtype, bias_dtype, out_dtype);
+  // torch's promotion: equal dtypes stay, everything else (f16 + bf16 included) goes to f32
+  const int promoted = y_dtype == bias_dtype ? y_dtype : STMOE_F32;
+  STMOE_REQUIRE(out_dtype == promoted, STMOE_ERR_DTYPE, "add_bias: dtypes %d + %d give %d, not %d", y_dtype, bias_dtype, promoted, out_dtype);
+  if (rows == 0) return STMOE_OK;
+  STMOE_REQUIRE(y && bias && out, STMOE_ERR_NULL, "add_bias: NULL pointer");
+  add_bias_kernel<<<dim3((unsigned)rows), 256, 0, as_stream(stream)>>>(y, y_dtype, bias, bias_dtype, cols, out, out_dtype);
+  return check_launch("add_bias");
 }
 
 extern "C" int stmoe_dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets,

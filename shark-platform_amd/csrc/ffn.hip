@@ -139,26 +139,34 @@ static inline void mark(void** events, int i, hipStream_t st) {
   if (events && events[i]) (void)hipEventRecord(reinterpret_cast<hipEvent_t>(events[i]), st);
 }
 
+// stages: 1 = gate/up projection only (the gated intermediate goes to `z_io`), 2 = down projection only (reads `z_io`),
+// 3 = both (the intermediate lives in the workspace).  offsets == NULL: one expert that owns all T * k rows.
 static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                             const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
                             int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
                             const float* z_scale, void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
-                            stmoe_stream_t stream, void** events, bool tickets_zeroed = false) {
+                            stmoe_stream_t stream, void** events, bool tickets_zeroed = false, int stages = 3,
+                            void* z_io = nullptr) {
   STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1, STMOE_ERR_SHAPE, "grouped_ffn: T=%lld K=%lld N=%lld E=%d k=%d",
                 (long long)T, (long long)K, (long long)N, E, k);
   STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
                 "grouped_ffn: activation dtype %d is not f32/f16/bf16", dtype);
   STMOE_REQUIRE(act == STMOE_ACT_SILU || act == STMOE_ACT_GELU_ERF, STMOE_ERR_UNSUPPORTED, "grouped_ffn: activation %d", act);
+  const bool do_in = (stages & 1) != 0, do_out = (stages & 2) != 0;
   int rc;
-  if ((rc = check_weight(w_gate, "grouped_ffn(ffn_gate_exps)", E, N, K))) return rc;
-  if ((rc = check_weight(w_up, "grouped_ffn(ffn_up_exps)", E, N, K))) return rc;
-  if ((rc = check_weight(w_down, "grouped_ffn(ffn_down_exps)", E, K, N))) return rc;
-  STMOE_REQUIRE(weight_tag(w_gate) == weight_tag(w_up), STMOE_ERR_UNSUPPORTED,
-                "grouped_ffn: gate and up weights must share one format");
+  if (do_in) {
+    if ((rc = check_weight(w_gate, "grouped_ffn(ffn_gate_exps)", E, N, K))) return rc;
+    if ((rc = check_weight(w_up, "grouped_ffn(ffn_up_exps)", E, N, K))) return rc;
+    STMOE_REQUIRE(weight_tag(w_gate) == weight_tag(w_up), STMOE_ERR_UNSUPPORTED,
+                  "grouped_ffn: gate and up weights must share one format");
+  }
+  if (do_out && (rc = check_weight(w_down, "grouped_ffn(ffn_down_exps)", E, K, N))) return rc;
   if (T == 0) return STMOE_OK;
-  STMOE_REQUIRE(x && offsets && (perm || k == 1) && y_sorted, STMOE_ERR_NULL, "grouped_ffn: NULL pointer");
-  STMOE_REQUIRE(aligned16(x) && aligned16(y_sorted) && aligned16(workspace), STMOE_ERR_ALIGN,
-                "grouped_ffn: x, y_sorted and workspace must be 16-byte aligned");
+  STMOE_REQUIRE(offsets || E == 1, STMOE_ERR_NULL, "grouped_ffn: offsets may only be NULL with a single expert");
+  STMOE_REQUIRE((!do_in || (x && (perm || k == 1))) && (!do_out || y_sorted) && (stages == 3 || z_io), STMOE_ERR_NULL,
+                "grouped_ffn: NULL pointer");
+  STMOE_REQUIRE((!do_in || aligned16(x)) && (!do_out || aligned16(y_sorted)) && aligned16(workspace) && aligned16(z_io),
+                STMOE_ERR_ALIGN, "grouped_ffn: x, y_sorted, the intermediate and the workspace must be 16-byte aligned");
   STMOE_REQUIRE((K * dtype_size(dtype)) % 16 == 0 && (N * dtype_size(dtype)) % 16 == 0, STMOE_ERR_SHAPE,
                 "grouped_ffn: rows of x and of the intermediate must be multiples of 16 bytes");
   const size_t need = stmoe_grouped_ffn_workspace_bytes(T, k, K, N, dtype);
@@ -168,7 +176,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   const int64_t rows = T * k;
   const FfnWs ws = carve_ffn(T, k, K, N, dtype);
   char* base = (char*)workspace;
-  void* z = base + ws.z;
+  void* z = stages == 3 ? (void*)(base + ws.z) : z_io;
   void* xa = base + ws.xa;
   void* zq = base + ws.zq;
 
@@ -177,46 +185,54 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   // unchanged: the streaming kernel is bound by the weight stream anyway, and the 16-bit prefill kernel with its
   // producer/consumer pipeline is currently faster than the fp8 matrix-core kernel.  Variant 5 sends both operands to
   // the fp8 matrix cores as bytes and scales the fp32 dot product once.
-  const bool fp8_w_in = w_gate->format == STMOE_W_FP8 || w_gate->format == STMOE_W_FP8_PACKED;
-  const bool fp8_w_out = w_down->format == STMOE_W_FP8 || w_down->format == STMOE_W_FP8_PACKED;
-  const bool want_mfma8 = variant == 5 || variant == 7;
+  const bool want_mfma8 = (variant == 5 || variant == 7) && stages == 3;
+  STMOE_REQUIRE(!(variant == 5 || variant == 7) || stages == 3, STMOE_ERR_UNSUPPORTED,
+                "grouped_ffn: variants 5 and 7 (fp8 matrix cores) run both projections in one call");
+  const bool fp8_w_in = want_mfma8 && (w_gate->format == STMOE_W_FP8 || w_gate->format == STMOE_W_FP8_PACKED);
+  const bool fp8_w_out = want_mfma8 && (w_down->format == STMOE_W_FP8 || w_down->format == STMOE_W_FP8_PACKED);
   STMOE_REQUIRE(!want_mfma8 || (x_scale && z_scale), STMOE_ERR_UNSUPPORTED, "grouped_ffn: variants 5 and 7 (fp8 matrix cores) need x_scale and z_scale");
   const bool t16 = dtype == STMOE_F16 || dtype == STMOE_BF16;
   const bool mfma8_in = t16 && x_scale && fp8_w_in && w_gate->dtype == STMOE_F32 && K % 16 == 0 && want_mfma8;
   const bool mfma8_out = t16 && z_scale && fp8_w_out && w_down->dtype == STMOE_F32 && N % 16 == 0 && want_mfma8;
-  const int v16 = want_mfma8 ? 0 : variant;
+  const int v16 = (variant == 5 || variant == 7) ? 0 : variant;
+  float* const split = ws.total > ws.split ? reinterpret_cast<float*>(base + ws.split) : nullptr;
+  const int32_t n_experts = offsets ? E : 1;
 
-  GemmParams p{};
-  p.a = x; p.lda = K; p.perm = perm; p.k_top = k; p.offsets = offsets; p.E = E; p.fixed_rows = 0;
-  p.w0 = make_view(w_gate); p.w1 = make_view(w_up);
-  p.out = z; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr; p.expert_rows_bound = T;
-  p.split_scratch = ws.total > ws.split ? reinterpret_cast<float*>(base + ws.split) : nullptr;
-  p.split_tickets_zeroed = tickets_zeroed;
-  mark(events, 0, st);
-  if (x_scale) {
-    if (mfma8_in) rc = stmoe_quantize_fp8(x, dtype, x_scale, T * K, xa, stream);
-    else rc = stmoe_fake_quant_fp8(x, dtype, x_scale, T * K, xa, stream);
+  if (do_in) {
+    GemmParams p{};
+    p.a = x; p.lda = K; p.perm = perm; p.k_top = k; p.offsets = offsets; p.E = n_experts; p.fixed_rows = offsets ? 0 : rows;
+    p.w0 = make_view(w_gate); p.w1 = make_view(w_up);
+    p.out = z; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr; p.expert_rows_bound = T;
+    p.split_scratch = split;
+    p.split_tickets_zeroed = tickets_zeroed;
+    mark(events, 0, st);
+    if (x_scale) {
+      if (mfma8_in) rc = stmoe_quantize_fp8(x, dtype, x_scale, T * K, xa, stream);
+      else rc = stmoe_fake_quant_fp8(x, dtype, x_scale, T * K, xa, stream);
+      if (rc) return rc;
+      p.a = xa;
+    }
+    if (mfma8_in) {
+      p.x_scale = x_scale;
+      if (mfma8_out) { p.out = zq; p.out_scale = z_scale; }
+      rc = run_fp8_projection(variant, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
+    } else {
+      rc = run_projection(v16, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
+    }
     if (rc) return rc;
-    p.a = xa;
+    mark(events, 1, st);
   }
-  if (mfma8_in) {
-    p.x_scale = x_scale;
-    if (mfma8_out) { p.out = zq; p.out_scale = z_scale; }
-    rc = run_fp8_projection(variant, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
-  } else {
-    rc = run_projection(v16, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
-  }
-  if (rc) return rc;
-  mark(events, 1, st);
+  if (!do_out) return STMOE_OK;
 
   GemmParams q{};
-  q.a = z; q.lda = N; q.perm = nullptr; q.k_top = 1; q.offsets = offsets; q.E = E; q.fixed_rows = 0;
+  q.a = z; q.lda = N; q.perm = nullptr; q.k_top = 1; q.offsets = offsets; q.E = n_experts; q.fixed_rows = offsets ? 0 : rows;
   q.w0 = make_view(w_down); q.w1 = q.w0;
   q.out = y_sorted; q.ldo = K; q.n_out = K; q.kred = N; q.act = act; q.x_scale = nullptr; q.expert_rows_bound = T;
-  q.split_scratch = ws.total > ws.split ? reinterpret_cast<float*>(base + ws.split) : nullptr;
+  q.split_scratch = split;
   q.split_tickets_zeroed = tickets_zeroed;  // (a launch that uses the tickets leaves them at zero)
   mark(events, 2, st);
   if (z_scale) {
+    STMOE_REQUIRE(stages == 3, STMOE_ERR_UNSUPPORTED, "grouped_ffn: the down projection on its own takes the intermediate as it is");
     if (mfma8_out && !mfma8_in) rc = stmoe_quantize_fp8(z, dtype, z_scale, rows * N, zq, stream);
     else if (!mfma8_out) rc = stmoe_fake_quant_fp8(z, dtype, z_scale, rows * N, z, stream);  // in place
     else rc = STMOE_OK;
@@ -240,6 +256,21 @@ extern "C" int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K,
                                  int variant, stmoe_stream_t stream) {
   return grouped_ffn_impl(x, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, z_scale, y_sorted,
                           workspace, workspace_bytes, variant, stream, nullptr);
+}
+
+extern "C" int stmoe_grouped_gate_up(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                                     const stmoe_weight* w_gate, const stmoe_weight* w_up, int act, const int32_t* offsets,
+                                     const int32_t* perm, const float* x_scale, void* z_sorted, void* workspace,
+                                     size_t workspace_bytes, int variant, stmoe_stream_t stream) {
+  return grouped_ffn_impl(x, dtype, T, K, N, E, k, w_gate, w_up, nullptr, act, offsets, perm, x_scale, nullptr, nullptr, workspace,
+                          workspace_bytes, variant, stream, nullptr, false, 1, z_sorted);
+}
+
+extern "C" int stmoe_grouped_down(const void* z_sorted, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
+                                  const stmoe_weight* w_down, const int32_t* offsets, void* y_sorted, void* workspace,
+                                  size_t workspace_bytes, int variant, stmoe_stream_t stream) {
+  return grouped_ffn_impl(nullptr, dtype, T, K, N, E, k, nullptr, nullptr, w_down, STMOE_ACT_SILU, offsets, nullptr, nullptr, nullptr,
+                          y_sorted, workspace, workspace_bytes, variant, stream, nullptr, false, 2, const_cast<void*>(z_sorted));
 }
 
 extern "C" int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight* w, void* out, int variant,

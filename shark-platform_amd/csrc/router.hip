@@ -616,6 +616,52 @@ static int launch_router(const void* x, const void* wr, int64_t T_tokens, int64_
   return check_launch("router_topk");
 }
 
+// ---------------------------------------------------------------------------------------------------
+// softmax over the last axis, one wavefront per row: values widened to fp32, p = expf(x - max) / sum, rounded to the
+// output dtype (torch.nn.functional.softmax(x, dim=-1, dtype=...)).  Rows of at most 64 elements (router logits over the
+// experts) are summed in index order by a serial loop over the lanes' values, the router kernels' own arithmetic, so
+// that ranking these probabilities gives the router's choice; longer rows add lane-strided partial sums and combine
+// them with the xor butterfly.
+__device__ __forceinline__ float softmax_load(const void* p, int dtype, int64_t i) {
+  switch (dtype) {
+    case STMOE_F16: return (float)reinterpret_cast<const f16_t*>(p)[i];
+    case STMOE_BF16: return bf16_to_f32(reinterpret_cast<const bf16_t*>(p)[i]);
+    default: return reinterpret_cast<const float*>(p)[i];
+  }
+}
+__device__ __forceinline__ void softmax_store(void* p, int dtype, int64_t i, float v) {
+  switch (dtype) {
+    case STMOE_F16: reinterpret_cast<f16_t*>(p)[i] = (f16_t)v; break;
+    case STMOE_BF16: reinterpret_cast<bf16_t*>(p)[i] = f32_to_bf16(v); break;
+    default: reinterpret_cast<float*>(p)[i] = v; break;
+  }
+}
+__global__ void __launch_bounds__(256)
+softmax_rows_kernel(const void* __restrict__ x, int x_dtype, int64_t rows, int64_t cols, void* __restrict__ out, int o_dtype) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int64_t base = r * cols;
+  if (cols <= 64) {
+    const float l = lane < cols ? softmax_load(x, x_dtype, base + lane) : 0.0f;
+    float mx = __shfl(l, 0);
+    for (int e = 1; e < cols; ++e) mx = fmaxf(mx, __shfl(l, e));
+    const float ex = expf(l - mx);
+    float denom = 0.0f;
+    for (int e = 0; e < cols; ++e) denom += __shfl(ex, e);
+    if (lane < cols) softmax_store(out, o_dtype, base + lane, ex / denom);
+    return;
+  }
+  float mx = -INFINITY;
+  for (int64_t c = lane; c < cols; c += 64) mx = fmaxf(mx, softmax_load(x, x_dtype, base + c));
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+  float sum = 0.0f;
+  for (int64_t c = lane; c < cols; c += 64) sum += expf(softmax_load(x, x_dtype, base + c) - mx);
+  sum = wave_xor_sum(sum);
+  for (int64_t c = lane; c < cols; c += 64) softmax_store(out, o_dtype, base + c, expf(softmax_load(x, x_dtype, base + c) - mx) / sum);
+}
+
 }  // namespace stmoe
 
 using namespace stmoe;
@@ -664,4 +710,14 @@ extern "C" int stmoe_router_topk(const void* x, const void* w_router, int dtype,
     case STMOE_BF16: return launch_router<bf16_t>(x, w_router, T, K, E, k, logits_out, idx_out, idx64_out, gate_out, st);
     default: return set_error(STMOE_ERR_DTYPE, "router_topk: dtype %d is not f32/f16/bf16", dtype);
   }
+}
+
+extern "C" int stmoe_softmax(const void* x, int x_dtype, int64_t rows, int64_t cols, void* out, int out_dtype, stmoe_stream_t stream) {
+  STMOE_REQUIRE(rows >= 0 && cols > 0 && rows < 0x7fffffffLL * 4, STMOE_ERR_SHAPE, "softmax: rows=%lld cols=%lld", (long long)rows, (long long)cols);
+  auto is_float = [](int d) { return d == STMOE_F32 || d == STMOE_F16 || d == STMOE_BF16; };
+  STMOE_REQUIRE(is_float(x_dtype) && is_float(out_dtype), STMOE_ERR_DTYPE, "softmax: dtypes %d -> %d", x_dtype, out_dtype);
+  if (rows == 0) return STMOE_OK;
+  STMOE_REQUIRE(x && out, STMOE_ERR_NULL, "softmax: NULL pointer");
+  softmax_rows_kernel<<<dim3((unsigned)((rows + 3) / 4)), 256, 0, as_stream(stream)>>>(x, x_dtype, rows, cols, out, out_dtype);
+  return check_launch("softmax");
 }

@@ -89,7 +89,13 @@ SIGNATURES = {
     "stmoe_grouped_ffn": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, POINTER(StmoeWeight), POINTER(StmoeWeight),
                                   POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int,
                                   c_void_p]),
+    "stmoe_grouped_gate_up": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, POINTER(StmoeWeight), POINTER(StmoeWeight),
+                                      c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    "stmoe_grouped_down": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, POINTER(StmoeWeight), c_void_p, c_void_p,
+                                   c_void_p, c_size_t, c_int, c_void_p]),
     "stmoe_grouped_mmt": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, POINTER(StmoeWeight), c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "stmoe_add_bias": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p]),
+    "stmoe_softmax": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p]),
     "stmoe_scale_rows": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "stmoe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int64, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p]),
     "stmoe_moe_forward": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
@@ -508,6 +514,68 @@ def grouped_ffn(x, w_gate: DeviceWeight, w_up: DeviceWeight, w_down: DeviceWeigh
                                      _ptr(offsets), _ptr(perm), _ptr(xs), _ptr(zs), _ptr(y), _ptr(workspace), workspace.numel(), variant,
                                      _stream(dev)))
     return y
+
+
+def grouped_gate_up(x, w_gate: DeviceWeight, w_up: DeviceWeight, act: int, offsets, perm, k: int, *, variant: int = VARIANT_AUTO,
+                    x_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [T,K] -> the gated intermediate z [T*k, N], rows in dispatch order (the first half of grouped_ffn)."""
+    dev = _dev(x, offsets, perm)
+    lib = load_library()
+    x_c = _contig(x)
+    T, K = x_c.shape
+    N, E = w_gate.rows, w_gate.experts
+    workspace = torch.empty(max(grouped_ffn_workspace_bytes(T, k, K, N, x_c.dtype), 1), dtype=torch.uint8, device=dev)
+    z = torch.empty((T * k, N), dtype=x_c.dtype, device=dev)
+    xs = _scale1(x_scale)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_grouped_gate_up(_ptr(x_c), dtype_enum(x_c.dtype), T, K, N, E, k, w_gate.ref, w_up.ref, act, _ptr(offsets),
+                                         _ptr(perm), _ptr(xs), _ptr(z), _ptr(workspace), workspace.numel(), variant, _stream(dev)))
+    return z
+
+
+def grouped_down(z, w_down: DeviceWeight, offsets, T: int, k: int, *, variant: int = VARIANT_AUTO) -> torch.Tensor:
+    """z [T*k, N] (dispatch order) -> y_sorted [T*k, K] (the second half of grouped_ffn; z is used as it is)."""
+    dev = _dev(z, offsets)
+    lib = load_library()
+    z_c = _contig(z)
+    N, K, E = w_down.cols, w_down.rows, w_down.experts
+    workspace = torch.empty(max(grouped_ffn_workspace_bytes(T, k, K, N, z_c.dtype), 1), dtype=torch.uint8, device=dev)
+    y = torch.empty((T * k, K), dtype=z_c.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_grouped_down(_ptr(z_c), dtype_enum(z_c.dtype), T, K, N, E, k, w_down.ref, _ptr(offsets), _ptr(y),
+                                      _ptr(workspace), workspace.numel(), variant, _stream(dev)))
+    return y
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """y [..., cols] + bias [cols] in torch's promoted dtype (the bias add of `linear`)."""
+    dev = _dev(y, bias)
+    lib = load_library()
+    y_c, b_c = _contig(y), _contig(bias)
+    cols = y_c.shape[-1]
+    if b_c.dim() != 1 or b_c.shape[0] != cols:
+        raise ValueError(f"add_bias: bias {list(bias.shape)} does not match rows of {cols} elements")
+    rows = y_c.numel() // cols if cols else 0
+    out = torch.empty(y_c.shape, dtype=torch.promote_types(y_c.dtype, b_c.dtype), device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_add_bias(_ptr(y_c), dtype_enum(y_c.dtype), _ptr(b_c), dtype_enum(b_c.dtype), rows, cols, _ptr(out),
+                                  dtype_enum(out.dtype), _stream(dev)))
+    return out
+
+
+def softmax(x: torch.Tensor, dim: int = -1, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """torch.nn.functional.softmax(x, dim, dtype) computed in fp32 by the library; the result has dtype `dtype` (x's if None)."""
+    dev = _dev(x)
+    lib = load_library()
+    out_dtype = dtype or x.dtype
+    moved = x.movedim(dim, -1)
+    x_c = _contig(moved)
+    cols = x_c.shape[-1]
+    rows = x_c.numel() // cols if cols else 0
+    out = torch.empty(x_c.shape, dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.stmoe_softmax(_ptr(x_c), dtype_enum(x_c.dtype), rows, cols, _ptr(out), dtype_enum(out_dtype), _stream(dev)))
+    return out.movedim(-1, dim)
 
 
 def grouped_mmt(a: torch.Tensor, w: "DeviceWeight", offsets, perm, T: int, k: int, *, a_per_pair: bool,

@@ -53,8 +53,7 @@ class FFN(ThetaLayer):
             T = x.shape[0]
             if T == 0:
                 return h.new_empty(*h.shape[:-1], wd.rows)
-            offsets = torch.tensor([0, T], dtype=torch.int32, device=x.device)
-            y = _hip.grouped_ffn(x, wg, wu, wd, self._act, offsets, None, 1)
+            y = _hip.grouped_ffn(x, wg, wu, wd, self._act, None, None, 1)  # one expert owns every row: no offsets array
             return y.reshape(*h.shape[:-1], y.shape[-1])
         if self.is_gated:
             ffn_gate = ops.elementwise(self.activation_fn, self.ffn_gate(h))

@@ -13,7 +13,7 @@ import torch.nn.functional as F
 
 from .. import _hip
 from .. import ops
-from ..ops import device_weight, gather_experts
+from ..ops import device_weight, expert_dispatch, gather_experts
 from ..utils import debugging
 from ..types import (DefaultPrimitiveTensor, DynamicScaledQuantizer, PlanarQuantizedTensor, QuantizedTensor,
                      StaticScaledQuantizer, Theta)
@@ -48,12 +48,14 @@ class PreGatherFFNMOE(ThetaLayer):
         for q in (self.q_input, self.q_intermediate):
             if q is not None and not isinstance(q, (StaticScaledQuantizer, DynamicScaledQuantizer)):
                 raise NotImplementedError(f"PreGatherFFNMOE: activation quantizer {type(q).__name__} has no kernel")
-        # Inside the fused kernels the intermediate exists only tile by tile, so its quantizer must be known before the
-        # launch: static and per tensor.  The input quantizer may also be per axis or dynamic (see forward).
+        # Inside the fused call the intermediate goes from one projection to the next without the host seeing it, so its
+        # quantizer must be known before the launch: static and per tensor.  A dynamic one (its scale is the maximum of the
+        # whole intermediate) or a per-axis one over the features runs between the two projections as calls of their own
+        # (see forward); the scale it computes stays on the device.
         qz = self.q_intermediate
-        if qz is not None and (not isinstance(qz, StaticScaledQuantizer) or qz.axis is not None):
-            raise NotImplementedError("PreGatherFFNMOE: the quantizer of the gated intermediate (ffn_down_exps.q_input) must be "
-                                      "static and per tensor; a dynamic or per-axis one needs the whole intermediate first")
+        if isinstance(qz, StaticScaledQuantizer) and qz.axis is not None and qz.axis not in (-1, 2):
+            raise NotImplementedError("PreGatherFFNMOE: a per-axis quantizer of the gated intermediate [tokens, slots, features] "
+                                      "(ffn_down_exps.q_input) must scale along the features (axis -1)")
         self.activation = activation
         self._act = activation_enum(activation)
         self._dw = None
@@ -72,10 +74,11 @@ class PreGatherFFNMOE(ThetaLayer):
             )
         return self._dw
 
-    def pre_matmul_gather(self, inputs, weights, experts, einstring="mk,menk->men"):
+    def pre_matmul_gather(self, inputs, weights, experts, einstring="mk,menk->men", dispatch=None):
         """`einsum_2args(inputs, weights[experts, :, :], einstring)` as in the reference
-        (sharktank/sharktank/layers/ffn_moe_block.py:37-41); the gather stays lazy and the product is grouped by expert."""
-        return ops.einsum_2args(inputs, gather_experts(weights, experts), einstring)
+        (sharktank/sharktank/layers/ffn_moe_block.py:37-41); the gather stays lazy and the product is grouped by expert.
+        `dispatch` (not in the reference): the grouping of `experts`, if the caller has it already."""
+        return ops.einsum_2args(inputs, gather_experts(weights, experts, dispatch), einstring)
 
     def forward_unfused(self, h: torch.Tensor, experts: torch.Tensor, expert_gate: torch.Tensor):
         """The reference's forward written with the same `ops` calls, one kernel per einsum (ffn_moe_block.py:60-74).
@@ -83,19 +86,25 @@ class PreGatherFFNMOE(ThetaLayer):
         act = {_hip.ACT_SILU: F.silu, _hip.ACT_GELU_ERF: F.gelu}[self._act]
         if self.q_input is not None or self.q_intermediate is not None:
             raise NotImplementedError("forward_unfused: activation quantizers are handled by forward only")
-        ffn_gate = ops.elementwise(act, self.pre_matmul_gather(h, self.ffn_gate, experts))
-        ffn_up = self.pre_matmul_gather(h, self.ffn_up, experts)
-        ffn_down = self.pre_matmul_gather(ffn_gate * ffn_up, self.ffn_down, experts, einstring="mek,menk->men")
+        dispatch = expert_dispatch(experts, self.expert_count)  # one grouping for the three products of this forward
+        ffn_gate = ops.elementwise(act, self.pre_matmul_gather(h, self.ffn_gate, experts, dispatch=dispatch))
+        ffn_up = self.pre_matmul_gather(h, self.ffn_up, experts, dispatch=dispatch)
+        ffn_down = self.pre_matmul_gather(ffn_gate * ffn_up, self.ffn_down, experts, einstring="mek,menk->men", dispatch=dispatch)
         ffn_down = ops.einsum_2args(expert_gate, ffn_down, "me,men->men")
         return torch.sum(ffn_down, dim=1)
 
     def activation_scales(self):
-        """(reciprocal scale of the input quantizer, of the intermediate quantizer) as the kernels take them: one device
-        float each; None where there is no quantizer or where `quantized_input` has to apply it before the launch."""
-        q = self.q_input
+        """(reciprocal scale of the input quantizer, of the intermediate quantizer) as the fused kernels take them: one
+        device float each; None where there is no quantizer or where the quantizer has to run as a pass of its own."""
+        q, qz = self.q_input, self.q_intermediate
         xs = q.reciprocal_scale if isinstance(q, StaticScaledQuantizer) and q.axis is None else None
-        zs = self.q_intermediate.reciprocal_scale if self.q_intermediate is not None else None
+        zs = qz.reciprocal_scale if isinstance(qz, StaticScaledQuantizer) and qz.axis is None else None
         return xs, zs
+
+    @property
+    def fusable(self) -> bool:
+        """Whether one fused call can run the whole FFN: every activation quantizer is static and per tensor (or absent)."""
+        return all(q is None or (isinstance(q, StaticScaledQuantizer) and q.axis is None) for q in (self.q_input, self.q_intermediate))
 
     def quantized_input(self, h: torch.Tensor):
         """(h', x_scale): how the input quantizer reaches the kernels.  Static per tensor: the kernels quantise themselves
@@ -114,15 +123,19 @@ class PreGatherFFNMOE(ThetaLayer):
         return int(self.ffn_gate.shape[0])
 
     def bigger_mmg(self, inputs, weights, experts):
-        """The reference keeps this alternative to the gather (one matmul against all experts, then a gather of the
-        results; ffn_moe_block.py:43-51) for experiments and never calls it from forward; it has no kernel here."""
-        raise NotImplementedError("PreGatherFFNMOE.bigger_mmg: unused by forward in the reference; not built")
+        """`einsum_2args(inputs, weights[experts, :, :], "mek,menk->men")` (ffn_moe_block.py:43-47): every (token, slot)
+        pair's own input row [T, k, cols] times its expert's matrix; pre_matmul_gather with the per-pair einsum."""
+        return ops.einsum_2args(inputs, gather_experts(weights, experts), "mek,menk->men")
 
     def one_hot_matmul(self, inputs, weights, experts):
-        """As bigger_mmg with a one-hot selection (ffn_moe_block.py:53-58): unused by the reference's forward; not built."""
+        """The reference's experiment that multiplies by every expert and mixes the results with a one-hot matrix of a
+        fixed 8 classes (ffn_moe_block.py:49-58): never called by its forward; it has no kernel here."""
         raise NotImplementedError("PreGatherFFNMOE.one_hot_matmul: unused by forward in the reference; not built")
 
-    def forward(self, h: torch.Tensor, experts: torch.Tensor, expert_gate: torch.Tensor):
+    def grouped(self, h: torch.Tensor, experts: torch.Tensor):
+        """The expert FFN of every (token, slot) pair, rows grouped by expert: (y [T*k, K] in dispatch order, inv [T*k] with
+        the row of pair t*k + j).  `forward` weights and sums these rows; MoeBlock does the same together with its output
+        norm and residual."""
         wg, wu, wd = self.device_weights()
         T, k = experts.shape
         if debugging.flags.enable_nan_checks:
@@ -131,9 +144,25 @@ class PreGatherFFNMOE(ThetaLayer):
             if bool(((experts < 0) | (experts >= wg.experts)).any()):
                 raise IndexError(f"PreGatherFFNMOE: expert index outside 0..{wg.experts - 1}")
         _, offsets, perm, inv = _hip.dispatch_build(experts, wg.experts)
-        _, zs = self.activation_scales()
+        xs, zs = self.activation_scales()
         h, xs = self.quantized_input(h)
-        y = _hip.grouped_ffn(h, wg, wu, wd, self._act, offsets, perm, k, variant=self.kernel_variant, x_scale=xs, z_scale=zs)
+        qz = self.q_intermediate
+        if qz is None or zs is not None:
+            y = _hip.grouped_ffn(h, wg, wu, wd, self._act, offsets, perm, k, variant=self.kernel_variant, x_scale=xs, z_scale=zs)
+        else:
+            # A dynamic or per-axis quantizer of the intermediate: gate/up projection, the quantizer's own quantise and
+            # dequantise on the whole intermediate (as LinearLayer applies a q_input, linear.py:72-78; the rows' order does not
+            # matter to a maximum over all of them nor to a scale per feature), down projection.
+            z = _hip.grouped_gate_up(h, wg, wu, self._act, offsets, perm, k, x_scale=xs)
+            if isinstance(qz, StaticScaledQuantizer):  # per axis, along the features: axis 1 of the [T*k, N] rows
+                qz = StaticScaledQuantizer(name=qz.name, scale=qz.scale, reciprocal_scale=qz.reciprocal_scale, dtype=qz.dtype, axis=1)
+            z = qz.quantize(z).unpack().dequant(z.dtype)
+            y = _hip.grouped_down(z, wd, offsets, T, k)
+        return y, inv
+
+    def forward(self, h: torch.Tensor, experts: torch.Tensor, expert_gate: torch.Tensor):
+        T, k = experts.shape
+        y, inv = self.grouped(h, experts)
         return _hip.combine(y, expert_gate.to(h.dtype), inv, T, k)
 
 
@@ -180,7 +209,5 @@ class FFNMOE(ThetaLayer):
                              for layer in (self.ffn_gate, self.ffn_up, self.ffn_down))
         wg, wu, wd = self._dw
         x = h.reshape(-1, h.shape[-1])
-        T = x.shape[0]
-        offsets = torch.tensor([0, T], dtype=torch.int32, device=x.device)
-        y = _hip.grouped_ffn(x, wg, wu, wd, _hip.ACT_SILU, offsets, None, 1)
+        y = _hip.grouped_ffn(x, wg, wu, wd, _hip.ACT_SILU, None, None, 1)  # one expert owns every row: no offsets array
         return y.reshape(*h.shape[:-1], y.shape[-1])

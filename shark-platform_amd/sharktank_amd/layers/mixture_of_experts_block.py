@@ -14,6 +14,7 @@ import torch
 import torch.nn.functional as F
 
 from .. import _hip
+from ..ops.hip_impls import _tensor_version
 from ..types import Theta, unbox_tensor
 from ..utils import debugging
 from .base import ThetaLayer
@@ -52,7 +53,7 @@ class MoeBlock(ThetaLayer):
         whose router tensor is replaced or resized gets a fresh copy (an in-place update of the same storage needs
         `reset_caches()`)."""
         src = unbox_tensor(self.ffn_gate_inp.weight)
-        key = (dtype, src.data_ptr(), tuple(src.shape), src.dtype, src._version)
+        key = (dtype, src.data_ptr(), tuple(src.shape), src.dtype, _tensor_version(src))
         hit = self._router_w.get(dtype)
         if hit is None or hit[0] != key:
             hit = (key, src.to(dtype).contiguous())
@@ -91,6 +92,8 @@ class MoeBlock(ThetaLayer):
         # reserve_workspace first), so that no later, larger forward replaces the buffer under the graph.
         if self._workspace is None or self._workspace.numel() < need or self._workspace.device != h.device:
             self._workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=h.device)
+        if not self.experts.fusable:
+            return self._forward_staged(h, x, ffn_norm_w, out_norm_w, return_routing)
         xs, zs = self.experts.activation_scales()
         # With tracing or golden dumps switched on, the routing is fetched as well and recorded beside the output (the
         # kernels and the results are the same either way).
@@ -105,6 +108,22 @@ class MoeBlock(ThetaLayer):
             out, idx, gate = res
         else:
             out, idx, gate = res, None, None
+        return self._finish(out, idx, gate, h.shape, return_routing)
+
+    def _forward_staged(self, h, x, ffn_norm_w, out_norm_w, return_routing: bool):
+        """The same forward as separate calls, for expert FFNs whose activation quantizers cannot ride inside the fused
+        call (a dynamic or per-axis quantizer of the input or of the intermediate): norm, router, the experts' grouped FFN
+        with its quantizer passes, then the weighted sum with the output norm and the residual."""
+        T, k = x.shape[0], self.expert_used_count
+        xn = _hip.rms_norm(x, ffn_norm_w, self.rms_epsilon)
+        idx, gate, _ = _hip.router_topk(xn, self._router_weight(h.dtype), k)
+        y, inv = self.experts.grouped(xn, idx)
+        out = _hip.combine(y, gate, inv, T, k, out_norm_w=out_norm_w, eps=self.rms_epsilon, residual=x)
+        return self._finish(out, idx, gate, h.shape, return_routing)
+
+    def _finish(self, out, idx, gate, shape, return_routing: bool):
+        batch_size, sequence_length, feature_dim = shape
+        tracing = debugging.flags.enable_tensor_trace or debugging.flags.save_goldens_path is not None
         out = out.reshape(batch_size, sequence_length, feature_dim)
         if tracing:
             record = {"top_k_experts": idx, "expert_gate": gate, "output": out}

@@ -17,7 +17,7 @@ from ..types.tensors import GatheredExpertsTensor, InferenceTensor, PrimitiveTen
 from ._registry import AllOfType
 from .signatures import *
 
-__all__ = ["device_weight", "gather_experts"]
+__all__ = ["device_weight", "expert_dispatch", "gather_experts"]
 
 _FLOAT_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
 
@@ -38,15 +38,25 @@ def device_weight(w, *, stacked: bool, prepack: bool = False) -> _hip.DeviceWeig
     return dw
 
 
+def _tensor_version(t: torch.Tensor) -> int:
+    """The tensor's in-place modification counter.  Tensors created under torch.inference_mode() do not track one (reading
+    it raises); they cannot be modified in place outside inference mode either, so they count as unchanged."""
+    try:
+        return t._version
+    except RuntimeError:
+        return -1
+
+
 def _planes_key(w):
-    """What a cached descriptor of `w` depends on: the identity, shape and version of every plane."""
+    """What a cached descriptor of `w` depends on: the identity, shape and version of every plane.  (The version counts
+    in-place changes made through torch; a plane rewritten through a raw pointer needs a fresh tensor object.)"""
     if isinstance(w, torch.Tensor):
         ts = (w,)
     elif isinstance(w, (Q8_0, Q4_1)):
         ts = (w.raw,)
     else:
         ts = tuple(w.globals.values())
-    return tuple((t.data_ptr(), tuple(t.shape), t.dtype, t._version) for t in ts)
+    return tuple((t.data_ptr(), tuple(t.shape), t.dtype, _tensor_version(t)) for t in ts)
 
 
 _TENSOR_CACHE = {}  # id(torch.Tensor) -> (weakref to it, {(stacked, prepack, dtype): (planes key, descriptor)})
@@ -180,16 +190,33 @@ def matmul_tensor_tensor(lhs, rhs, *, transpose_rhs: bool):
 
 
 def _linear(input, weight, bias, *, accum_dtype=None):
-    if bias is not None:
-        return NotImplemented
+    """matmul(input, weight^T) (+ bias), as linear_default composes it (sharktank/sharktank/ops/default_impls.py:328-341):
+    the product is rounded to the input's dtype, the bias is added in the two tensors' promoted dtype."""
     input = unbox_tensor(input)
-    if isinstance(weight, QuantizedTensor):
-        return matmul(input, weight, transpose_rhs=True)
-    return matmul(input, weight, transpose_rhs=True)  # a dense weight is cast to the input's dtype once and kept
+    result = matmul(input, weight, transpose_rhs=True)  # a dense weight is cast to the input's dtype once and kept
+    if bias is not None:
+        bias = unbox_tensor(bias)
+        if bias.dim() != 1 or bias.dtype not in _FLOAT_DTYPES:
+            return NotImplemented
+        result = _hip.add_bias(result, bias)
+    return result
 
 
 linear.override(Tensor, Tensor)(_linear)
 linear.override(Tensor, QuantizedTensor)(_linear)
+linear.override(Tensor, Tensor, Tensor)(_linear)
+linear.override(Tensor, QuantizedTensor, Tensor)(_linear)
+
+
+@softmax.override(Tensor)
+def softmax_hip(tensor, dim=None, dtype=None):
+    """F.softmax (sharktank/sharktank/ops/default_impls.py:426-432) in fp32 on the device."""
+    x = unbox_tensor(tensor)
+    if x.dtype not in _FLOAT_DTYPES or (dtype is not None and dtype not in _FLOAT_DTYPES) or x.dim() == 0:
+        return NotImplemented
+    if dim is None:  # torch's legacy default: axis 0 for 0-, 1- and 3-dimensional inputs, else 1
+        dim = 0 if x.dim() in (0, 1, 3) else 1
+    return _hip.softmax(x, dim, dtype)
 
 
 @get_index.override(AllOfType(Tensor, PrimitiveTensor))
@@ -215,8 +242,10 @@ def _is_expert_index(key):
     return first
 
 
-def gather_experts(weights, experts: torch.Tensor) -> GatheredExpertsTensor:
-    """Lazy `weights[experts, :, :]` for an expert-stacked weight [E, rows, cols] of any supported kind."""
+def gather_experts(weights, experts: torch.Tensor, dispatch=None) -> GatheredExpertsTensor:
+    """Lazy `weights[experts, :, :]` for an expert-stacked weight [E, rows, cols] of any supported kind.  `dispatch`: the
+    (offsets, perm) arrays of `experts` if the caller has built them already (the einsums of one forward index their
+    weights with the same tensor); they are never kept beyond the gathered tensor itself."""
     if len(weights.shape) != 3:
         raise ValueError(f"gather_experts: expert-stacked weight must be [E, rows, cols], got {list(weights.shape)}")
     w = weights if isinstance(weights, InferenceTensor) else None
@@ -224,7 +253,9 @@ def gather_experts(weights, experts: torch.Tensor) -> GatheredExpertsTensor:
         from ..types.tensors import DefaultPrimitiveTensor
 
         w = DefaultPrimitiveTensor(data=weights)
-    return GatheredExpertsTensor(weights=w, experts=experts)
+    g = GatheredExpertsTensor(weights=w, experts=experts)
+    g._dispatch = dispatch
+    return g
 
 
 @get_index.override(QuantizedTensor)
@@ -235,21 +266,11 @@ def get_index_quantized_experts(tensor: QuantizedTensor, key):
     return gather_experts(tensor, experts)
 
 
-_LAST_DISPATCH = None  # (weakref to the experts tensor, its planes key, expert count, (offsets, perm))
-
-
-def _dispatch_of(experts: torch.Tensor, E: int):
-    """The dispatch arrays of an index tensor.  The three einsums of one PreGatherFFNMOE forward index with the same tensor:
-    the arrays are built for the first and reused by the other two."""
-    global _LAST_DISPATCH
-    import weakref
-
-    key = _planes_key(experts)
-    last = _LAST_DISPATCH
-    if last is not None and last[0]() is experts and last[1] == key and last[2] == E:
-        return last[3]
+def expert_dispatch(experts: torch.Tensor, E: int):
+    """(offsets, perm) of an index tensor [T, k]: rows grouped by expert.  Built from the tensor's present contents on
+    every call: an index buffer may be refilled in place by a kernel (a fused forward, a graph replay) without torch
+    noticing, so nothing here is remembered from call to call."""
     _, offsets, perm, _ = _hip.dispatch_build(experts, E)
-    _LAST_DISPATCH = (weakref.ref(experts), key, E, (offsets, perm))
     return offsets, perm
 
 
@@ -257,7 +278,7 @@ def _gathered_state(g: GatheredExpertsTensor):
     if g._device_weight is None:
         g._device_weight = cached_device_weight(g.weights, stacked=True)
     if g._dispatch is None:
-        g._dispatch = _dispatch_of(g.experts, g._device_weight.experts)
+        g._dispatch = expert_dispatch(g.experts, g._device_weight.experts)
     return g._device_weight, g._dispatch
 
 

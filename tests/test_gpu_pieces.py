@@ -527,6 +527,33 @@ def test_dynamic_quantizer_bit_exact(device, dtype, n, kind):
     assert torch.equal(lay.dequant().cpu().reshape(-1), O.dequant_tensor_scaled(want_rscale, want_qs, layout_dtype=dtype).reshape(-1))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_dynamic_quantizer_scale_is_reciprocal_times_number(device, dtype):
+    """The reference's `finfo.max / amax.clamp(eps)` divides a Python number by a tensor, which torch evaluates as
+    `amax.reciprocal() * 448`: two roundings in the tensor's dtype.  A single division rounds differently for about one
+    maximum in four (amax = 4.8867 in fp16: 91.625 against 91.6875), which moves every sample that sits near a rounding
+    boundary.  Sixty maxima, among them that one."""
+    from sharktank_amd import types as ST
+
+    g = torch.Generator().manual_seed(77)
+    q = ST.DynamicScaledQuantizer(dtype=torch.float8_e4m3fn)
+    differs = 0
+    for i in range(60):
+        x = torch.randn(257, generator=g) * (0.05 + 3.0 * float(torch.rand((), generator=g)))
+        if i == 0:
+            x = x.clamp(-4.0, 4.0)
+            x[5] = 4.8867
+        x = x.to(dtype)
+        want_qs, want_rscale = O.dynamic_quantize(x, torch.float8_e4m3fn)
+        lay = q.quantize(x.to(device)).unpack()
+        assert torch.equal(lay.d.cpu().reshape(()), want_rscale.reshape(())), (i, float(x.abs().max()))
+        assert torch.equal(lay.qs.cpu().view(torch.uint8), want_qs.view(torch.uint8)), (i, float(x.abs().max()))
+        amax = x.abs().max().clamp(0.125)
+        differs += int((torch.tensor(448.0, dtype=dtype) / amax) != 448.0 / amax)
+    if dtype == torch.float16:
+        assert differs >= 5, "the sample no longer tells the two formulas apart"
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", [0, 1])
 def test_matrix_core_probe_runs(device, kind):

@@ -139,10 +139,9 @@ def test_router_with_bias_is_refused():
 
 
 def test_unused_reference_alternatives_are_named():
-    """PreGatherFFNMOE.bigger_mmg / one_hot_matmul exist in the reference and are never called by its forward."""
+    """PreGatherFFNMOE.one_hot_matmul exists in the reference (with a hard-wired 8 experts) and is never called by its forward."""
     from sharktank_amd.layers import PreGatherFFNMOE
 
     ffn = PreGatherFFNMOE(_tiny_theta())
-    for fn in (ffn.bigger_mmg, ffn.one_hot_matmul):
-        with pytest.raises(NotImplementedError, match="unused by forward"):
-            fn(None, None, None)
+    with pytest.raises(NotImplementedError, match="unused by forward"):
+        ffn.one_hot_matmul(None, None, None)
