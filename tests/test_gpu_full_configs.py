@@ -8,8 +8,8 @@ The CPU oracle cannot run these shapes in full in reasonable time, so each case 
     prefill launches is a token tile times a feature tile, and a row spans all feature tiles, so every unit of both
     launches, split along the reduction or not, has rows in the sample), rows of the expert's last, partial token tile,
     and the rows that ride along with a full tile (1-16 rows above a multiple of 256).  The MoE contribution y - h is
-    held to the tolerance on its own (the residual h ~ N(0, 1) would hide an error of the FFN kernels): 1e-3 for fp16,
-    2e-2 for fp8 weights or activations, 2e-3 for bf16 (see BF16_TOL),
+    held to the tolerance on its own (the residual h ~ N(0, 1) would hide an error of the FFN kernels): 1e-3 for fp16 and
+    for bf16, 2e-2 for fp8 weights or activations,
   * a second kernel family (the 128 x 128 tile kernel) on all rows,
   * size-independent properties on all tokens: token-permutation equivariance (routing bit-exact; outputs equal up to
     the fp32 summation grouping of the few rows whose down-projection tile is split along the reduction) and run-to-run
@@ -25,13 +25,12 @@ import moe_cases as MC
 
 pytestmark = pytest.mark.gpu
 
-# bf16 keeps 8 significant bits: rounding the output alone is a relative error of about 2^-9 / sqrt(3) = 1.1e-3 per element,
-# and the gated intermediate, the down projection and the gate-weighted slot values are each rounded again.  Where the
-# kernel and the oracle round the same fp32 value they agree exactly, so what is measured is how often a different order of
-# the fp32 sums moves a value across a bf16 rounding boundary: 4e-4 to 8e-4 on the MoE contribution at these shapes.  Two
-# formulations of the oracle itself that differ only in the order of the fp32 sums (per-token gather against per-expert
-# grouping, tests/test_oracle_golden.py) are held to 8e-3 on small layers; the kernels are held to 2e-3 here.
-BF16_TOL = 2e-3
+# bf16 keeps 8 significant bits, and the gated intermediate, the down projection and the gate-weighted slot values are each
+# rounded to it.  Where the kernel and the oracle round the same fp32 value they agree exactly, so what is measured is how
+# often a different order of the fp32 sums moves a value across a bf16 rounding boundary: 4e-4 to 8e-4 on the MoE
+# contribution at these shapes (long reductions average the flips out; layers with a hidden size of 512 measure 2e-3, see
+# tests/test_gpu_layer.py).  The limit is the north-star figure for the layer, held on the MoE contribution alone as well.
+BF16_TOL = 1e-3
 
 
 def build_device_case(device, T, K, N, fmt, dtype, act="silu", seed=0, E=8, k=2, out_norm=False, act_quant=False):
@@ -229,10 +228,10 @@ def test_config2_mixtral_q8_0_prefill_and_decode(device):
     """Mixtral-8x7B layer, Q8_0, fp16: prefill 2048 tokens and decode 32 tokens."""
     theta, pc = build_device_case(device, 2048, 4096, 14336, "q8_0", torch.float16, seed=0)
     y, idx, gate, block = run_layer(theta, pc, device)
-    rows, tiles = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2)
+    rows, tiles = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2, at_least=256)
     counts = torch.bincount(idx.cpu().reshape(-1).long(), minlength=8).tolist()
     print(f"  rows per expert {counts}: {tiles} token tiles, {len(rows)} tokens checked")
-    assert len(rows) >= 64
+    assert len(rows) >= 256
     check_against_oracle(y, idx, pc, rows)
     check_second_kernel_family(theta, pc, device, y, 1e-3)
     # PreGatherFFNMOE on its own, with the router's choices

@@ -15,10 +15,13 @@ pytestmark = pytest.mark.gpu
 TOL = {torch.float32: 1e-5, torch.float16: 1e-3, torch.bfloat16: 1e-3}
 # Limits on the MoE contribution y - h alone (the residual h ~ N(0, 1) is as large as the contribution and would hide an
 # FFN error in a check of y).  fp32 and fp16: the north-star figures.  bf16 keeps 8 significant bits and the gated
-# intermediate, the down projection and the weighted slot values are each rounded to it: two formulations of the oracle
-# itself that differ only in the order of the fp32 sums are 8e-3 apart (tests/test_oracle_golden.py), and that is the
-# figure the kernels are held to.
-MOE_TOL = {torch.float32: 1e-4, torch.float16: 1e-3, torch.bfloat16: 8e-3}
+# intermediate, the down projection and the weighted slot values are each rounded to it: a different order of the fp32
+# sums moves a value across a rounding boundary now and then, and on these small layers (hidden size 512, where few terms
+# average the flips out) the kernels measure 1.6e-3 to 2.1e-3 against the oracle; two formulations of the oracle itself
+# that differ only in that order are up to 8e-3 apart (tests/test_oracle_golden.py).  The layer output y itself is held to
+# the north-star 1e-3 (measured: under 1e-4); at the full BASELINE shapes the contribution alone is, too
+# (tests/test_gpu_full_configs.py).
+MOE_TOL = {torch.float32: 1e-4, torch.float16: 1e-3, torch.bfloat16: 3e-3}
 
 
 def run_block(case, device, variant=0):
@@ -43,6 +46,7 @@ def check_case(case, device, variant=0, tol=None, moe_tol=None):
     err_y = O.rel_l2(y, want_y)
     tol = tol or TOL[case.dtype]
     moe_tol = moe_tol or MOE_TOL[case.dtype]
+    print(f"  {case.fmt} {case.dtype} T={case.T} variant {variant}: layer rel-L2 {err_y:.2e}, MoE contribution {err:.2e} (limits {tol:.0e}, {moe_tol:.0e})")
     assert err_y < tol, f"layer output rel-L2 {err_y:.3e}"
     assert err < moe_tol, f"MoE contribution rel-L2 {err:.3e} (limit {moe_tol:.0e})"
     return err, err_y
@@ -98,8 +102,8 @@ def test_fp8_weights_and_fp8_activations(device, dtype, T):
     path quantises and dequantises the activations and multiplies in the activation dtype, which is the reference's
     own arithmetic: the MoE contribution itself (without the residual) matches the oracle to the 16-bit tolerance."""
     case = MC.Case(T=T, K=512, N=768, fmt="fp8", dtype=dtype, act_quant=True, seed=40 + T)
-    err, err_y = check_case(case, device, tol=1e-3 if dtype == torch.float16 else 8e-3)
-    assert err < (1e-3 if dtype == torch.float16 else 8e-3), f"MoE contribution rel-L2 {err:.3e}"
+    err, err_y = check_case(case, device, tol=1e-3)
+    assert err < (1e-3 if dtype == torch.float16 else 3e-3), f"MoE contribution rel-L2 {err:.3e}"
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
