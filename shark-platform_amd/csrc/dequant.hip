@@ -86,10 +86,9 @@ quantize_fp8_kernel(const T* __restrict__ x, const float* __restrict__ rscale, i
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   // eager torch divides in fp32 by the 0-dim fp32 scale and rounds the quotient to x's dtype
-  float q = round_to<T>(__fdiv_rn(Cvt<T>::to_f32(x[i]), *rscale));
-  q = fminf(fmaxf(q, -448.0f), 448.0f);
-  if (q != q) q = __uint_as_float(0x7fc00000u);
-  out[i] = f32_to_fp8_e4m3fn(q);
+  const float q = round_to<T>(__fdiv_rn(Cvt<T>::to_f32(x[i]), *rscale));
+  // (fminf / fmaxf drop a NaN operand; torch.clamp keeps it)
+  out[i] = f32_to_fp8_e4m3fn(q != q ? __uint_as_float(0x7fc00000u) : fminf(fmaxf(q, -448.0f), 448.0f));
 }
 
 // ---- dynamic per-tensor quantisation -------------------------------------------------------------------------
@@ -150,10 +149,8 @@ dynamic_quantize_fp8_kernel(const T* __restrict__ x, int64_t n, const float* __r
   }
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
-  float q = round_to<T>(__fmul_rn(Cvt<T>::to_f32(x[i]), scale));
-  q = fminf(fmaxf(q, -448.0f), 448.0f);
-  if (q != q) q = __uint_as_float(0x7fc00000u);
-  out[i] = f32_to_fp8_e4m3fn(q);
+  const float q = round_to<T>(__fmul_rn(Cvt<T>::to_f32(x[i]), scale));
+  out[i] = f32_to_fp8_e4m3fn(q != q ? __uint_as_float(0x7fc00000u) : fminf(fmaxf(q, -448.0f), 448.0f));
 }
 
 // Quantise and dequantise again in one pass: the values a fake-quantised activation tensor holds.
@@ -162,12 +159,7 @@ __global__ void __launch_bounds__(256)
 fake_quant_fp8_kernel(const T* __restrict__ x, const float* __restrict__ rscale, int64_t n, T* __restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const float rs = *rscale;
-  float q = round_to<T>(__fdiv_rn(Cvt<T>::to_f32(x[i]), rs));
-  q = fminf(fmaxf(q, -448.0f), 448.0f);
-  if (q != q) q = __uint_as_float(0x7fc00000u);
-  const float v = fp8_e4m3fn_to_f32(f32_to_fp8_e4m3fn(q));
-  out[i] = Cvt<T>::from_f32(keep_f32(__fmul_rn(v, rs)));
+  out[i] = Cvt<T>::from_f32(FakeQuant(rscale).one<T>(Cvt<T>::to_f32(x[i])));
 }
 
 template <bool I4>
@@ -307,10 +299,8 @@ quantize_fp8_per_axis_kernel(const T* __restrict__ x, const S* __restrict__ scal
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const int64_t j = (i / inner) % axis_len;
-  float q = round_to<P>(__fmul_rn(Cvt<T>::to_f32(x[i]), Cvt<S>::to_f32(scale[j])));
-  q = fminf(fmaxf(q, -448.0f), 448.0f);
-  if (q != q) q = __uint_as_float(0x7fc00000u);
-  out[i] = f32_to_fp8_e4m3fn(q);
+  const float q = round_to<P>(__fmul_rn(Cvt<T>::to_f32(x[i]), Cvt<S>::to_f32(scale[j])));
+  out[i] = f32_to_fp8_e4m3fn(q != q ? __uint_as_float(0x7fc00000u) : fminf(fmaxf(q, -448.0f), 448.0f));
 }
 
 extern "C" int stmoe_quantize_fp8_per_axis(const void* x, int x_dtype, const void* scale, int scale_dtype, int64_t axis_len,

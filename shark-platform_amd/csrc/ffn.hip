@@ -146,7 +146,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
                             int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
                             const float* z_scale, void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
                             stmoe_stream_t stream, void** events, bool tickets_zeroed = false, int stages = 3,
-                            void* z_io = nullptr) {
+                            void* z_io = nullptr, bool x_is_fake_quantized = false) {
   STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1, STMOE_ERR_SHAPE, "grouped_ffn: T=%lld K=%lld N=%lld E=%d k=%d",
                 (long long)T, (long long)K, (long long)N, E, k);
   STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
@@ -206,12 +206,15 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
     p.split_scratch = split;
     p.split_tickets_zeroed = tickets_zeroed;
     mark(events, 0, st);
-    if (x_scale) {
+    if (x_scale && !(x_is_fake_quantized && !mfma8_in)) {  // (the fused forward's norm launch may have done it already)
       if (mfma8_in) rc = stmoe_quantize_fp8(x, dtype, x_scale, T * K, xa, stream);
       else rc = stmoe_fake_quant_fp8(x, dtype, x_scale, T * K, xa, stream);
       if (rc) return rc;
       p.a = xa;
     }
+    // the quantizer of the intermediate is applied by the gate/up kernels themselves (16-bit kernels; the fp8 matrix-core
+    // kernels write real e4m3fn samples instead)
+    if (z_scale && stages == 3 && !mfma8_out && !mfma8_in) p.out_fq = z_scale;
     if (mfma8_in) {
       p.x_scale = x_scale;
       if (mfma8_out) { p.out = zq; p.out_scale = z_scale; }
@@ -234,8 +237,8 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   if (z_scale) {
     STMOE_REQUIRE(stages == 3, STMOE_ERR_UNSUPPORTED, "grouped_ffn: the down projection on its own takes the intermediate as it is");
     if (mfma8_out && !mfma8_in) rc = stmoe_quantize_fp8(z, dtype, z_scale, rows * N, zq, stream);
-    else if (!mfma8_out) rc = stmoe_fake_quant_fp8(z, dtype, z_scale, rows * N, z, stream);  // in place
-    else rc = STMOE_OK;
+    else if (!mfma8_out && mfma8_in) rc = stmoe_fake_quant_fp8(z, dtype, z_scale, rows * N, z, stream);  // in place
+    else rc = STMOE_OK;  // (done by the gate/up launch, or the fp8 kernel has written e4m3fn samples)
     if (rc) return rc;
   }
   if (mfma8_out) {
@@ -381,8 +384,11 @@ static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int6
   mark(events, 2, st);
   // a single token's dispatch is written by the router launch itself
   const bool router_dispatches = fused_front && T == 1;
+  // a static quantizer of the experts' input rides in the norm launch (which writes the rows the experts read) unless the
+  // fp8 matrix-core kernels want real e4m3fn samples
+  const float* x_fq = (fused_front && x_scale && variant != 5 && variant != 7) ? x_scale : nullptr;
   if (fused_front) rc = norm_router(h, dtype, ffn_norm_w, w_dtype, eps, xn, w_router, T, K, E, k, idx, gate, st,
-                                    router_dispatches ? counts : nullptr, offsets, perm, inv);
+                                    router_dispatches ? counts : nullptr, offsets, perm, inv, x_fq);
   else rc = stmoe_router_topk(xn, w_router, dtype, T, K, E, k, nullptr, idx, nullptr, gate, stream);
   if (rc) return rc;
   mark(events, 3, st);
@@ -396,7 +402,8 @@ static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int6
     return rc;
   mark(events, 5, st);
   if ((rc = grouped_ffn_impl(xn, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, z_scale, y,
-                             base + ws.ffn, workspace_bytes - ws.ffn, variant, stream, events ? events + 6 : nullptr, has_tickets)))
+                             base + ws.ffn, workspace_bytes - ws.ffn, variant, stream, events ? events + 6 : nullptr, has_tickets, 3,
+                             nullptr, x_fq != nullptr)))
     return rc;
   mark(events, 10, st);
   rc = stmoe_combine(y, gate, inv, dtype, T, k, K, out_norm_w, w_dtype, eps, h, out, stream);

@@ -75,7 +75,7 @@ grouped_generic_kernel(GemmParams p) {
   if (lane == 0) {
     const float scale = p.x_scale ? *p.x_scale : 1.0f;
     T* o = reinterpret_cast<T*>(p.out) + out_row(p, i) * p.ldo + n;
-    if (MODE == MODE_GATEUP) *o = Cvt<T>::from_f32(gateup_epilogue<T>(p.act, acc0, acc1, scale));
+    if (MODE == MODE_GATEUP) *o = Cvt<T>::from_f32(gateup_epilogue<T>(p.act, acc0, acc1, scale, fq_scale(p)));
     else *o = Cvt<T>::from_f32(acc0 * scale);
   }
 }

@@ -29,6 +29,7 @@ struct GemmParams {
   int32_t act;
   const float* x_scale;   // optional scale applied to the fp32 dot products (fp8 activations)
   const float* out_scale; // fp8 kernel only: quantise the result with this reciprocal scale and store e4m3fn bytes
+  const float* out_fq;    // GATEUP, 16-bit kernels: fake-quantise the gated product with this reciprocal scale (see below)
   int64_t expert_rows_bound;  // host-side bound of rows per expert (a token gives an expert at most one row)
   float* split_scratch;       // optional fp32 scratch for split reductions (mfma_ws_partial_bytes() bytes)
   bool split_tickets_zeroed;  // the caller vouches that the scratch's ticket words (mfma_ws_tickets_offset()) are zero
@@ -73,11 +74,20 @@ __device__ __forceinline__ float act_rt(int act, float v) {
 
 __device__ __forceinline__ int64_t out_row(const GemmParams& p, int i) { return p.out_perm ? (int64_t)p.out_perm[i] : (int64_t)i; }
 
+// A static quantizer of the gated intermediate (the q_input of the down projection) is applied where the intermediate is
+// produced: the value written is the quantised and dequantised one (FakeQuant) of the gated product, instead of a second
+// pass over the whole intermediate.
+__device__ __forceinline__ FakeQuant fq_scale(const GemmParams& p) { return FakeQuant(p.out_fq); }
+
 template <typename T> __device__ __forceinline__ float gateup_epilogue(int act, float g, float u, float scale) {
   const float gr = round_to<T>(g * scale);
   const float a = round_to<T>(act_rt(act, gr));
   const float ur = round_to<T>(u * scale);
   return round_to<T>(__fmul_rn(a, ur));
+}
+template <typename T> __device__ __forceinline__ float gateup_epilogue(int act, float g, float u, float scale, const FakeQuant& fq) {
+  const float v = gateup_epilogue<T>(act, g, u, scale);
+  return fq.on() ? fq.one<T>(v) : v;
 }
 
 // Epilogue of the prefill kernels for one accumulator quad (4 consecutive features of one token): the same rounding
@@ -91,6 +101,20 @@ template <int ACT> __device__ __forceinline__ float act_fast(float v) {
   else
     return act_gelu_erf(v);
 }
+template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t v);
+template <> __device__ __forceinline__ float unpack_lo<f16_t>(uint32_t v) { return (float)__builtin_bit_cast(f16_t, (uint16_t)(v & 0xffffu)); }
+template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t v) { return __uint_as_float(v << 16); }
+template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t v);
+template <> __device__ __forceinline__ float unpack_hi<f16_t>(uint32_t v) { return (float)__builtin_bit_cast(f16_t, (uint16_t)(v >> 16)); }
+template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
+// FakeQuant of four packed values of T
+template <typename T> __device__ __forceinline__ uint2 fake_quant_quad(uint2 v, const FakeQuant& fq) {
+  float a = unpack_lo<T>(v.x), b = unpack_hi<T>(v.x), c = unpack_lo<T>(v.y), d = unpack_hi<T>(v.y);
+  fq.pair<T>(a, b);
+  fq.pair<T>(c, d);
+  return make_uint2(pack2<T>(a, b), pack2<T>(c, d));
+}
+
 template <typename T, int ACT>
 __device__ __forceinline__ uint2 gateup_quad(const float (&g)[4], const float (&u)[4]) {
   if constexpr (__is_same(T, f16_t)) {
@@ -111,6 +135,11 @@ __device__ __forceinline__ uint2 gateup_quad(const float (&g)[4], const float (&
     }
     return make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
   }
+}
+template <typename T, int ACT>
+__device__ __forceinline__ uint2 gateup_quad(const float (&g)[4], const float (&u)[4], const FakeQuant& fq) {
+  const uint2 v = gateup_quad<T, ACT>(g, u);
+  return fq.on() ? fake_quant_quad<T>(v, fq) : v;
 }
 
 }  // namespace stmoe

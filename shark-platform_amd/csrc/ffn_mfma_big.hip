@@ -244,6 +244,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
   // ---- epilogue ---------------------------------------------------------------------------------------
   auto store_gateup = [&](auto act_tag) {
     constexpr int ACT = decltype(act_tag)::value;
+    const FakeQuant fq = fq_scale(p);
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
       const int r = wm * 64 + tj * 16 + n_in;
@@ -253,7 +254,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
         for (int ti = 0; ti < 4; ++ti) {
           const float gq[4] = {acc[ti][tj][0], acc[ti][tj][1], acc[ti][tj][2], acc[ti][tj][3]};
           const float uq[4] = {acc[ti + 4][tj][0], acc[ti + 4][tj][1], acc[ti + 4][tj][2], acc[ti + 4][tj][3]};
-          *reinterpret_cast<uint2*>(orow + ti * 16) = gateup_quad<T, ACT>(gq, uq);
+          *reinterpret_cast<uint2*>(orow + ti * 16) = gateup_quad<T, ACT>(gq, uq, fq);
         }
       }
     }

@@ -137,6 +137,7 @@ grouped_mfma_tile_kernel(GemmParams p) {
   }
 
   const float scale = p.x_scale ? *p.x_scale : 1.0f;
+  const FakeQuant fq = fq_scale(p);
 #pragma unroll
   for (int ti = 0; ti < 4; ++ti)
 #pragma unroll
@@ -147,7 +148,7 @@ grouped_mfma_tile_kernel(GemmParams p) {
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          if (MODE == MODE_GATEUP) v[r] = gateup_epilogue<T>(p.act, acc[0][ti][tj][r], acc[NW - 1][ti][tj][r], scale);
+          if (MODE == MODE_GATEUP) v[r] = gateup_epilogue<T>(p.act, acc[0][ti][tj][r], acc[NW - 1][ti][tj][r], scale, fq);
           else v[r] = acc[0][ti][tj][r] * scale;
         }
         uint2 pk = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));

@@ -72,14 +72,15 @@ __device__ __forceinline__ void ws_reduce_row(const GemmParams& p, const BigTile
   };
   T* orow = reinterpret_cast<T*>(p.out) + out_row(p, sorted_row) * p.ldo;
   if (MODE == MODE_GATEUP) {
+    const FakeQuant fq = fq_scale(p);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int col = (c8 + 8 * j) * 4;
       const floatx4_t gs = total(col), us = total(BN / 2 + col);
       const float gq[4] = {gs[0], gs[1], gs[2], gs[3]}, uq[4] = {us[0], us[1], us[2], us[3]};
       uint2* dst = reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * (BN / 2) + col);
-      if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq);
-      else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq);
+      if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq, fq);
+      else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq, fq);
     }
   } else {
 #pragma unroll
@@ -91,6 +92,67 @@ __device__ __forceinline__ void ws_reduce_row(const GemmParams& p, const BigTile
   }
 }
 __global__ void ws_zero_tickets_kernel(int* tickets) { tickets[threadIdx.x] = 0; }
+
+// ---- the loaders' load queue, checked at compile time --------------------------------------------------------
+// A loader's loads are issued by hand and awaited with `s_waitcnt vmcnt(N)`: "at most N of my loads may still be in
+// flight", the N youngest.  Each N in the kernel is written as a formula over the loads per step; the model below replays
+// the order in which the prologue and the K steps issue their loads (W: the weight pieces of a step, X: its direct token
+// loads, T: the operands of the ride-along rows) and derives, for each wait, the largest N that still covers everything
+// the code behind the wait reads.  The static_asserts in the kernel compare the two for every unit shape and format.
+struct WsLoadQueue {
+  static constexpr int kMax = 64;
+  int kind[kMax] = {}, step[kMax] = {}, count[kMax] = {}, n = 0;
+  constexpr void issue(int k, int s, int c) {
+    if (c == 0) return;
+    kind[n] = k; step[n] = s; count[n] = c; ++n;
+  }
+  // loads younger than the youngest entry of (kind k, step s): what may stay in flight when that entry must have landed
+  constexpr int younger_than(int k, int s) const {
+    int at = -1;
+    for (int i = 0; i < n; ++i)
+      if (kind[i] == k && step[i] == s) at = i;
+    if (at < 0) return -1;  // never issued: a modelling error
+    int y = 0;
+    for (int i = at + 1; i < n; ++i) y += count[i];
+    return y;
+  }
+};
+enum { WS_W = 0, WS_X = 1, WS_T = 2 };
+constexpr int ws_min(int a, int b) { return a < b ? a : b; }
+// the largest N for the three kinds of wait: 0 = the prologue's first (before the weights of step 0 are converted),
+// 1 = its second (before the first barrier), 2 + kt = the wait that ends K step kt
+constexpr int ws_model_wait(int which, int W, int X, int T) {
+  WsLoadQueue q;
+  q.issue(WS_T, 0, T); q.issue(WS_W, 0, W); q.issue(WS_X, 0, X);
+  q.issue(WS_T, 1, T); q.issue(WS_W, 1, W); q.issue(WS_X, 1, X);
+  q.issue(WS_W, 2, W);
+  if (which == 0) return T ? ws_min(q.younger_than(WS_W, 0), q.younger_than(WS_T, 0)) : q.younger_than(WS_W, 0);
+  q.issue(WS_T, 2, T); q.issue(WS_W, 3, W);
+  // step 0 reads the token rows of step 0 and converts the weights of step 1 (with the ride-along operands of step 1)
+  if (which == 1) {
+    int need = ws_min(q.younger_than(WS_X, 0), q.younger_than(WS_W, 1));
+    return T ? ws_min(need, q.younger_than(WS_T, 1)) : need;
+  }
+  for (int kt = 0;; ++kt) {
+    // K step kt: per piece the reload of the weights of step kt + 4 and its share of the token loads of step kt + 2, then
+    // the ride-along operands of step kt + 3 (the interleaving inside a step does not matter to a wait at its end)
+    q.issue(WS_W, kt + 4, W); q.issue(WS_X, kt + 2, X); q.issue(WS_T, kt + 3, T);
+    if (which == 2 + kt) {
+      // behind this wait: the barrier (consumers read the token rows of step kt + 1) and the next step's conversion of the
+      // weights of step kt + 2 with the ride-along operands of step kt + 2
+      int need = ws_min(q.younger_than(WS_X, kt + 1), q.younger_than(WS_W, kt + 2));
+      return T ? ws_min(need, q.younger_than(WS_T, kt + 2)) : need;
+    }
+  }
+}
+template <int W, int X, int T> struct WsWaitCheck {
+  static_assert(ws_model_wait(0, W, X, T) == 2 * W + 2 * X + T, "prologue: wait before the first conversion");
+  static_assert(ws_model_wait(1, W, X, T) == 2 * W + X + T, "prologue: wait before the first barrier");
+  // (step 0 could leave the prologue's last weight loads in flight as well; it waits like every other step)
+  static_assert(ws_model_wait(2, W, X, T) >= W + X + T && ws_model_wait(3, W, X, T) == W + X + T &&
+                ws_model_wait(4, W, X, T) == W + X + T && ws_model_wait(9, W, X, T) == W + X + T, "wait at the end of a K step");
+  static constexpr bool ok = true;
+};
 
 template <typename T, int WF, int MODE>
 __global__ void __launch_bounds__(768, 1)
@@ -322,6 +384,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
     auto run = [&](auto tail_tag) {
       constexpr bool TAIL = decltype(tail_tag)::value != 0;
       constexpr int TLOADS = TAIL ? 2 : 0;
+      static_assert(WsWaitCheck<WLOADS, XLOADS, TLOADS>::ok, "the hand-counted waits no longer match the order of the loads");
       // what step 0 waits for goes first: a unit's first requests queue behind each other for the CU's one vector-memory path
       if constexpr (TAIL) load_tx(WsInt<0>{}, 0);
       load_w(WsInt<0>{}, 0);
@@ -374,13 +437,14 @@ grouped_mfma_ws_kernel(WsArgs args) {
         for (int bi = 0; bi < 4; ++bi) *reinterpret_cast<floatx4_t*>(pt + piece_row(bi) + 4 * g) = tacc[bi];
       } else if (MODE == MODE_GATEUP) {
         T* orow = reinterpret_cast<T*>(p.out) + out_row(p, tile.tail_begin + n_in) * p.ldo + (int64_t)ntile * (BN / 2) + 4 * g;
+        const FakeQuant fq = fq_scale(p);
 #pragma unroll
         for (int bi = 0; bi < 2; ++bi) {
           const float gq[4] = {tacc[bi][0], tacc[bi][1], tacc[bi][2], tacc[bi][3]};
           const float uq[4] = {tacc[bi + 2][0], tacc[bi + 2][1], tacc[bi + 2][2], tacc[bi + 2][3]};
           uint2* dst = reinterpret_cast<uint2*>(orow + (2 * pw + bi) * 16);
-          if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq);
-          else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq);
+          if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq, fq);
+          else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq, fq);
         }
       } else {
         T* orow = reinterpret_cast<T*>(p.out) + out_row(p, tile.tail_begin + n_in) * p.ldo + (int64_t)ntile * BN + 4 * g;
@@ -492,6 +556,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
   // Rows are written in whole 128-byte lines (see lane_group_transpose4; the launcher checks their alignment).
   auto store_gateup = [&](auto act_tag) {
     constexpr int ACT = decltype(act_tag)::value;
+    const FakeQuant fq = fq_scale(p);  // (a quantizer of the intermediate is applied here, where the intermediate is made)
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
       const int r = wm * rpg + tj * 16 + n_in;
@@ -502,7 +567,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
         for (int ti = 0; ti < 4; ++ti) {
           const float gq[4] = {acc[ti][tj][0], acc[ti][tj][1], acc[ti][tj][2], acc[ti][tj][3]};
           const float uq[4] = {acc[ti + 4][tj][0], acc[ti + 4][tj][1], acc[ti + 4][tj][2], acc[ti + 4][tj][3]};
-          q[ti] = gateup_quad<T, ACT>(gq, uq);
+          q[ti] = gateup_quad<T, ACT>(gq, uq, fq);
         }
         lane_group_transpose4(q);
         if (mine)
@@ -515,7 +580,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
         for (int ti = 0; ti < 4; ++ti) {
           const float gq[4] = {acc[ti][tj][0], acc[ti][tj][1], acc[ti][tj][2], acc[ti][tj][3]};
           const float uq[4] = {acc[ti + 4][tj][0], acc[ti + 4][tj][1], acc[ti + 4][tj][2], acc[ti + 4][tj][3]};
-          *reinterpret_cast<uint2*>(orow + ti * 16) = gateup_quad<T, ACT>(gq, uq);
+          *reinterpret_cast<uint2*>(orow + ti * 16) = gateup_quad<T, ACT>(gq, uq, fq);
         }
       }
     }

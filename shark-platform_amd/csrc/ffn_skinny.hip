@@ -354,6 +354,7 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
     if (kw != 0) return;
   }
 
+  const FakeQuant fq = fq_scale(p);
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int i = r0 + mt * 16 + n_in;
@@ -362,7 +363,7 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
       if (MODE == MODE_GATEUP) {
         float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = gateup_epilogue<T>(p.act, acc[mt][0][r], acc[mt][1][r], 1.0f);
+        for (int r = 0; r < 4; ++r) v[r] = gateup_epilogue<T>(p.act, acc[mt][0][r], acc[mt][1][r], 1.0f, fq);
         *reinterpret_cast<uint2*>(orow + tile * 16 + 4 * g) = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
       } else {
 #pragma unroll
@@ -537,6 +538,7 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
       arrived(w0);
     }
   }
+  const FakeQuant fq = fq_scale(p);
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int i = r0 + mt * 16 + n_in;
@@ -545,7 +547,7 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
       if (MODE == MODE_GATEUP) {
         float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = gateup_epilogue<T>(p.act, acc[mt][0][r], acc[mt][1][r], 1.0f);
+        for (int r = 0; r < 4; ++r) v[r] = gateup_epilogue<T>(p.act, acc[mt][0][r], acc[mt][1][r], 1.0f, fq);
         *reinterpret_cast<uint2*>(orow + tile * 16 + 4 * g) = make_uint2(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]));
       } else {
 #pragma unroll

@@ -201,8 +201,12 @@ __global__ void __launch_bounds__(512, (PRE && !LATE) ? 4 : 8)
 router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float eps, T* __restrict__ xn,
                  const T* __restrict__ wr, int64_t K, int E, int k, T* __restrict__ logits_out,
                  int32_t* __restrict__ idx_out, int64_t* __restrict__ idx64_out, T* __restrict__ gate_out,
-                 SingleTokenDispatch disp) {
+                 SingleTokenDispatch disp, const float* __restrict__ x_fq) {
   extern __shared__ __align__(16) unsigned char smem[];
+  // x_fq (with FUSE_NORM): reciprocal scale of a static e4m3fn quantizer of the expert FFN's input.  The router multiplies
+  // the normalised row as it is; the copy written to `xn`, which only the expert projections read, is the quantised and
+  // dequantised one (fake_quant_fp8_value), so that no separate pass over the activations is needed.
+  const FakeQuant fq(FUSE_NORM ? x_fq : nullptr);
   T* xs = reinterpret_cast<T*>(smem);                                  // [K] the (normalised) token row
   float* lg_s = reinterpret_cast<float*>(smem + ((K * sizeof(T) + 15) / 16) * 16);  // [E] logits, then 8 partials
   float* part = lg_s + 64;
@@ -281,7 +285,7 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
         o = round_to<W>(keep_f32(__fmul_rn(nw[j], o)));
         const T r = Cvt<T>::from_f32(o);
         xs[i] = r;
-        xn[t * K + i] = r;
+        xn[t * K + i] = fq.on() ? Cvt<T>::from_f32(fq.one<T>(Cvt<T>::to_f32(r))) : r;
       }
     }
     for (int64_t i = tid + (int64_t)NC * 512; i < K; i += 512) {
@@ -289,7 +293,7 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
       o = round_to<W>(keep_f32(__fmul_rn(Cvt<W>::to_f32(norm_w[i]), o)));
       const T r = Cvt<T>::from_f32(o);
       xs[i] = r;
-      xn[t * K + i] = r;
+      xn[t * K + i] = fq.on() ? Cvt<T>::from_f32(fq.one<T>(Cvt<T>::to_f32(r))) : r;
     }
   } else {
     for (int64_t i = (int64_t)tid * 8; i < K; i += 512 * 8)
@@ -423,8 +427,9 @@ template <typename T, typename W, int NCH, int EP>
 __global__ void __launch_bounds__(256)
 norm_router_wave_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float eps, T* __restrict__ xn,
                         const T* __restrict__ wr, int64_t T_tokens, int E, int k, int32_t* __restrict__ idx_out,
-                        T* __restrict__ gate_out) {
+                        T* __restrict__ gate_out, const float* __restrict__ x_fq) {
   static_assert(sizeof(T) == 2, "16-bit rows");
+  const FakeQuant fq(x_fq);  // (as in router_wg_kernel: the copy in `xn` is the fake-quantised one)
   constexpr int K = NCH * 512;
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -489,8 +494,17 @@ norm_router_wave_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, f
         o = round_to<W>(keep_f32(__fmul_rn(nw[i].v[j], o)));
         xf[c][j] = round_to<T>(o);
       }
-      xn4[c * 64 + lane] = make_uint4(pack2<T>(xf[c][0], xf[c][1]), pack2<T>(xf[c][2], xf[c][3]), pack2<T>(xf[c][4], xf[c][5]),
-                                      pack2<T>(xf[c][6], xf[c][7]));
+      uint4 packed = make_uint4(pack2<T>(xf[c][0], xf[c][1]), pack2<T>(xf[c][2], xf[c][3]), pack2<T>(xf[c][4], xf[c][5]),
+                                pack2<T>(xf[c][6], xf[c][7]));
+      if (fq.on()) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = xf[c][j];
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) fq.pair<T>(v[j], v[j + 1]);
+        packed = make_uint4(pack2<T>(v[0], v[1]), pack2<T>(v[2], v[3]), pack2<T>(v[4], v[5]), pack2<T>(v[6], v[7]));
+      }
+      xn4[c * 64 + lane] = packed;
     }
   }
 
@@ -534,7 +548,7 @@ norm_router_wave_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, f
 static constexpr int64_t kWaveRouterMinTokens = 768;  // (measured at 4096-element rows: 14 us against 13.5 at 512 tokens, 16 against 18 at 1024, 17 against 25 at 2048)
 template <typename T, typename W>
 static bool launch_norm_router_wave(const void* x, const void* norm_w, float eps, void* xn, const void* wr, int64_t T_tokens,
-                                    int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st) {
+                                    int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st, const float* x_fq) {
   if constexpr (sizeof(T) != 2) {
     return false;
   } else {
@@ -544,7 +558,7 @@ static bool launch_norm_router_wave(const void* x, const void* norm_w, float eps
     const size_t lds = (size_t)4 * K * 2;
 #define STMOE_NRW(NCH, EP)                                                                                              \
   norm_router_wave_kernel<T, W, NCH, EP><<<grid, 256, lds, st>>>((const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, \
-                                                                 T_tokens, E, k, idx, (T*)gate)
+                                                                 T_tokens, E, k, idx, (T*)gate, x_fq)
 #define STMOE_NRW_E(NCH)      \
   do {                        \
     if (E <= 8) STMOE_NRW(NCH, 8); \
@@ -565,18 +579,19 @@ static bool launch_norm_router_wave(const void* x, const void* norm_w, float eps
 template <typename T, typename W, bool FUSE_NORM>
 static int launch_router_wg(const void* x, const void* norm_w, float eps, void* xn, const void* wr, int64_t T_tokens,
                             int64_t K, int E, int k, void* logits, int32_t* idx, int64_t* idx64, void* gate, hipStream_t st,
-                            SingleTokenDispatch disp = SingleTokenDispatch{nullptr, nullptr, nullptr, nullptr}) {
+                            SingleTokenDispatch disp = SingleTokenDispatch{nullptr, nullptr, nullptr, nullptr},
+                            const float* x_fq = nullptr) {
   const size_t lds = ((K * sizeof(T) + 15) / 16) * 16 + (64 + 8 + 64) * sizeof(float);
   if (lds > 64 * 1024) return set_error(STMOE_ERR_UNSUPPORTED, "router: K=%lld does not fit the per-token LDS row", (long long)K);
   if (T_tokens <= 64)
     router_wg_kernel<T, W, FUSE_NORM, 8, false><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
-        (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
+        (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp, x_fq);
   else if (T_tokens <= 512)
     router_wg_kernel<T, W, FUSE_NORM, 4, false><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
-        (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
+        (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp, x_fq);
   else
     router_wg_kernel<T, W, FUSE_NORM, 0, true><<<dim3((unsigned)T_tokens), 512, lds, st>>>(
-        (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp);
+        (const T*)x, (const W*)norm_w, eps, (T*)xn, (const T*)wr, K, E, k, (T*)logits, idx, idx64, (T*)gate, disp, x_fq);
   return check_launch("router_wg");
 }
 
@@ -584,13 +599,13 @@ static int launch_router_wg(const void* x, const void* norm_w, float eps, void* 
 // With all four dispatch pointers given and T_tokens == 1 the launch also writes the token's dispatch arrays.
 int norm_router(const void* h, int dtype, const void* norm_w, int w_dtype, float eps, void* xn, const void* wr,
                 int64_t T_tokens, int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st,
-                int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv) {
+                int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv, const float* x_fq) {
   SingleTokenDispatch disp{nullptr, nullptr, nullptr, nullptr};
   if (T_tokens == 1 && counts && offsets && perm && inv) disp = SingleTokenDispatch{counts, offsets, perm, inv};
 #define STMOE_NR(TT, WW)                                                                                                   \
   do {                                                                                                                     \
-    if (launch_norm_router_wave<TT, WW>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, idx, gate, st)) return check_launch("norm_router_wave"); \
-    return launch_router_wg<TT, WW, true>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, nullptr, idx, nullptr, gate, st, disp); \
+    if (launch_norm_router_wave<TT, WW>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, idx, gate, st, x_fq)) return check_launch("norm_router_wave"); \
+    return launch_router_wg<TT, WW, true>(h, norm_w, eps, xn, wr, T_tokens, K, E, k, nullptr, idx, nullptr, gate, st, disp, x_fq); \
   } while (0)
   if (dtype == STMOE_F32 && w_dtype == STMOE_F32) STMOE_NR(float, float);
   if (dtype == STMOE_F16 && w_dtype == STMOE_F32) STMOE_NR(f16_t, float);

@@ -16,7 +16,8 @@ int set_error(int code, const char* fmt, ...);
 int check_launch(const char* what);
 int norm_router(const void* h, int dtype, const void* norm_w, int w_dtype, float eps, void* xn, const void* wr,
                 int64_t T_tokens, int64_t K, int E, int k, int32_t* idx, void* gate, hipStream_t st,
-                int32_t* counts = nullptr, int32_t* offsets = nullptr, int32_t* perm = nullptr, int32_t* inv = nullptr);
+                int32_t* counts = nullptr, int32_t* offsets = nullptr, int32_t* perm = nullptr, int32_t* inv = nullptr,
+                const float* x_fq = nullptr);
 
 // stmoe_dispatch_build that also clears `n_zero` (at most 1024) 32-bit words at `zero_words` (nullable).
 int dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv,
@@ -111,6 +112,44 @@ __device__ __forceinline__ uint8_t f32_to_fp8_e4m3fn(float f) {
   if (enc > 0x7eu) return sign | 0x7f;           // rounded above 448
   return sign | (uint8_t)enc;
 }
+
+// quantize(x).unpack().dequant() of a static per-tensor e4m3fn quantizer (StaticScaledQuantizer,
+// sharktank/sharktank/types/quantizers.py:153-183; applied by LinearLayer, sharktank/sharktank/layers/linear.py:72-78) for
+// values of T given widened to fp32: T(f32(e4m3fn(clamp(T(x / rs)))) * rs).  The one definition of that arithmetic: the
+// stand-alone pass and the kernels that apply it to a value they have just computed share it.
+//   * x / rs, correctly rounded in fp32, comes from the correctly rounded reciprocal of rs (one division per kernel, kept
+//     in FakeQuant) and one residual step per value: q0 = x * inv, q = fma(fma(-q0, rs, x), inv, q0);
+//   * the e4m3fn rounding and its inverse are the hardware conversions (OCP e4m3fn, round to nearest even; the operand is
+//     clamped to +-448 first, NaN stays NaN).
+// Both are pinned by a test that runs every fp16 and every bf16 value through the stand-alone pass with many scales and
+// compares with eager torch on the host.
+struct FakeQuant {
+  float rs, inv;  // reciprocal scale of the quantizer (0: no quantizer) and its correctly rounded reciprocal
+  __device__ __forceinline__ explicit FakeQuant(const float* rscale) {
+    rs = rscale ? *rscale : 0.0f;
+    inv = rscale ? __fdiv_rn(1.0f, rs) : 0.0f;
+  }
+  __device__ __forceinline__ bool on() const { return rs != 0.0f; }
+  template <typename T> __device__ __forceinline__ float clamped_quotient(float x) const {
+    const float q0 = __fmul_rn(x, inv);
+    // (an infinite quotient stays as it is: the residual step would turn it into NaN, where torch clamps it to +-448; so
+    // does a zero: the residual step would lose the sign of -0)
+    const float q1 = (fabsf(q0) == INFINITY || x == 0.0f) ? q0 : __builtin_fmaf(__builtin_fmaf(-q0, rs, x), inv, q0);
+    const float q = round_to<T>(q1);
+    // fminf / fmaxf drop a NaN operand; torch.clamp keeps it
+    return q != q ? __uint_as_float(0x7fc00000u) : fminf(fmaxf(q, -448.0f), 448.0f);
+  }
+  template <typename T> __device__ __forceinline__ void pair(float& a, float& b) const {
+    const int bytes = __builtin_amdgcn_cvt_pk_fp8_f32(clamped_quotient<T>(a), clamped_quotient<T>(b), 0, false);
+    a = round_to<T>(keep_f32(__fmul_rn(__builtin_amdgcn_cvt_f32_fp8(bytes, 0), rs)));
+    b = round_to<T>(keep_f32(__fmul_rn(__builtin_amdgcn_cvt_f32_fp8(bytes, 1), rs)));
+  }
+  template <typename T> __device__ __forceinline__ float one(float a) const {
+    float b = 0.0f;
+    pair<T>(a, b);
+    return a;
+  }
+};
 
 // ---- activations ---------------------------------------------------------------------------------
 __device__ __forceinline__ float act_silu(float v) { return v / (1.0f + expf(-v)); }

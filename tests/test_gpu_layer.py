@@ -416,3 +416,39 @@ def test_prefill_front_end_equals_staged_calls(device, dtype, T, K, E, k, norm_i
     y = _hip.grouped_ffn(xn, wg, wu, wd, block.experts._act, offsets, perm, k)
     staged = _hip.combine(y, gate, inv, T, k, residual=h)
     assert torch.equal(staged.view(torch.int16), fused.reshape(T, K).view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("fmt,T,K,N", [("fp8", 40, 512, 768), ("fp8", 300, 512, 768), ("q8_0", 1100, 2048, 512), ("fp8", 700, 512, 256)])
+def test_fused_activation_quantizers_equal_separate_passes(device, fmt, dtype, T, K, N):
+    """Static e4m3fn quantizers of the experts' input and of the gated intermediate are applied where those tensors are
+    produced (the norm launch writes the fake-quantised rows, the gate/up kernels write the fake-quantised intermediate).
+    The result must have the bits of the same forward with each quantizer as a pass of its own over the finished tensor
+    (stmoe_fake_quant_fp8, itself bit-exact against the oracle): the streaming kernel, the prefill kernels with ride-along
+    rows and split units, and both front-end kernels are covered by the shapes."""
+    from sharktank_amd import _hip
+    from sharktank_amd.layers import MoeBlock
+    from sharktank_amd.types import unbox_tensor
+
+    case = MC.build(MC.Case(T=T, K=K, N=N, fmt=fmt, dtype=dtype, act_quant=True, seed=300 + T))
+    theta = MC.make_theta(case, device)
+    block = MoeBlock(theta, case.E, case.k, case.eps)
+    wg, wu, wd = block.experts.device_weights()
+    h = case.planes["h"].to(device)
+    fused, idx_f, gate_f = block(h.reshape(1, T, K), return_routing=True)
+    xs, zs = block.experts.activation_scales()
+    assert xs is not None and zs is not None
+
+    xn = _hip.rms_norm(h, unbox_tensor(block.ffn_norm.weight), case.eps)
+    idx, gate, _ = _hip.router_topk(xn, block._router_weight(dtype), case.k)
+    assert torch.equal(idx, idx_f) and torch.equal(gate, gate_f)
+    counts, offsets, perm, inv = _hip.dispatch_build(idx, case.E)
+    xq = _hip.fake_quant_fp8(xn, xs)
+    z = _hip.grouped_gate_up(xq, wg, wu, block.experts._act, offsets, perm, case.k)
+    zq = _hip.fake_quant_fp8(z, zs)
+    y = _hip.grouped_down(zq, wd, offsets, T, case.k)
+    staged = _hip.combine(y, gate, inv, T, case.k, residual=h)
+    assert torch.equal(staged.view(torch.int16), fused.reshape(T, K).view(torch.int16))
+    # the grouped FFN on its own takes both scales too
+    y2 = _hip.grouped_ffn(xn, wg, wu, wd, block.experts._act, offsets, perm, case.k, x_scale=xs, z_scale=zs)
+    assert torch.equal(y2.view(torch.int16), y.view(torch.int16))

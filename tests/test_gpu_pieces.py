@@ -565,3 +565,25 @@ def test_matrix_core_probe_runs(device, kind):
     for random_operands in (True, False):
         rate = _hip.probe_mfma(device, kind, random_operands, iters=2000, launches=2, warm_launches=2)
         assert 0.1 * peak < rate <= 1.02 * peak, f"kind {kind}, random {random_operands}: {rate:.0f} TFLOP/s"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fake_quant_every_16_bit_value_against_eager_torch(device, dtype):
+    """The fake-quantisation arithmetic the kernels share (the quotient from a correctly rounded reciprocal and one residual
+    step, the hardware's e4m3fn rounding) must give eager torch's bits -- `t / reciprocal_scale` in fp32 rounded to the
+    tensor's dtype, clamped, cast to float8_e4m3fn, widened and multiplied back (the oracle runs those torch operations on
+    the host) -- for every input there is: all 65536 bit patterns of the dtype, each with 150 scales (powers of two,
+    scales next to them, scales whose reciprocal is far from representable, very small and very large ones)."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(dtype)
+    g = torch.Generator().manual_seed(91)
+    scales = [2.0 ** e for e in range(-12, 5)] + [float(torch.tensor(2.0 ** e).nextafter(torch.tensor(4.0 if i else 0.0))) for e in range(-6, 2) for i in (0, 1)]
+    scales += [4.0 * 1.25 / 448.0, 8.0 * 2.0 / 448.0, 1.0 / 3.0, 0.1, 0.7, 1e-6, 300.0]
+    scales += (torch.rand(150 - len(scales), generator=g).double() * 0.2 + 1e-3).tolist()
+    xd = x.to(device)
+    for s in scales:
+        rs = torch.tensor(s, dtype=torch.float32)
+        want = O.fake_quant_per_tensor(x, rs)
+        got = _hip().fake_quant_fp8(xd, rs.to(device)).cpu()
+        same = (got.view(torch.int16) == want.view(torch.int16)) | (torch.isnan(got) & torch.isnan(want))
+        assert bool(same.all()), f"scale {s!r}: {int((~same).sum())} of 65536 values differ, first at bits {int(bits[~same][0]) & 0xffff:#06x}"
