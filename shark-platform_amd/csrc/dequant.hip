@@ -85,10 +85,40 @@ __global__ void __launch_bounds__(256)
 quantize_fp8_kernel(const T* __restrict__ x, const float* __restrict__ rscale, int64_t n, uint8_t* __restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  // eager torch divides in fp32 by the 0-dim fp32 scale and rounds the quotient to x's dtype
-  const float q = round_to<T>(__fdiv_rn(Cvt<T>::to_f32(x[i]), *rscale));
-  // (fminf / fmaxf drop a NaN operand; torch.clamp keeps it)
-  out[i] = f32_to_fp8_e4m3fn(q != q ? __uint_as_float(0x7fc00000u) : fminf(fmaxf(q, -448.0f), 448.0f));
+  // eager torch divides in fp32 by the 0-dim fp32 scale and rounds the quotient to x's dtype (FakeQuant::clamped_quotient)
+  out[i] = (uint8_t)FakeQuant(rscale).quantize2<T>(Cvt<T>::to_f32(x[i]), 0.0f);
+}
+
+// The same samples for rows gathered on the way: out row i = quantised row perm[i] / k of x (rows grouped by expert for the
+// fp8 matrix-core kernel, which then reads its token rows without a gather).  One workgroup per row, 8 elements per thread.
+template <typename T>
+__global__ void __launch_bounds__(256)
+quantize_fp8_gather_kernel(const T* __restrict__ x, const float* __restrict__ rscale, const int32_t* __restrict__ perm, int k,
+                           int64_t K, uint8_t* __restrict__ out, int64_t block_rows) {
+  const int64_t i = blockIdx.x;
+  const int64_t src = perm ? perm[i] / k : i;
+  const FakeQuant fq(rscale);
+  for (int64_t c = (int64_t)threadIdx.x * 8; c < K; c += 256 * 8) {
+    float v[8];
+    if constexpr (sizeof(T) == 2) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(x + src * K + c);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = Cvt<T>::to_f32(__builtin_bit_cast(T, (uint16_t)(w[j] & 0xffffu)));
+        v[2 * j + 1] = Cvt<T>::to_f32(__builtin_bit_cast(T, (uint16_t)(w[j] >> 16)));
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = Cvt<T>::to_f32(x[src * K + c + j]);
+    }
+    uint2 q;
+    q.x = fq.quantize2<T>(v[0], v[1]) | (fq.quantize2<T>(v[2], v[3]) << 16);
+    q.y = fq.quantize2<T>(v[4], v[5]) | (fq.quantize2<T>(v[6], v[7]) << 16);
+    // block_rows > 0: blocks of 64 reduction samples, [K / 64][block_rows][64] (the layout the 256 x 256 fp8 kernel streams)
+    const int64_t at = block_rows ? ((c >> 6) * block_rows + i) * 64 + (c & 63) : i * K + c;
+    *reinterpret_cast<uint2*>(out + at) = q;
+  }
 }
 
 // ---- dynamic per-tensor quantisation -------------------------------------------------------------------------
@@ -340,6 +370,25 @@ extern "C" int stmoe_quantize_fp8(const void* x, int x_dtype, const float* rscal
   }
   return check_launch("quantize_fp8");
 }
+
+namespace stmoe {
+// rows of x [*, K] (K a multiple of 8, rows 16-byte aligned) quantised into out [rows, K] in the order perm gives
+int quantize_fp8_gather(const void* x, int dtype, const float* rscale, const int32_t* perm, int k, int64_t rows, int64_t K, void* out,
+                        int64_t block_rows, hipStream_t st) {
+  STMOE_REQUIRE(rows >= 0 && rows < 0x7fffffffLL && K > 0 && K % 8 == 0 && k >= 1 && (block_rows == 0 || (block_rows >= rows && K % 64 == 0)),
+                STMOE_ERR_SHAPE, "quantize_fp8_gather: rows=%lld K=%lld", (long long)rows, (long long)K);
+  if (rows == 0) return STMOE_OK;
+  STMOE_REQUIRE(x && rscale && out, STMOE_ERR_NULL, "quantize_fp8_gather: NULL pointer");
+  const dim3 g((unsigned)rows);
+  switch (dtype) {
+    case STMOE_F32: quantize_fp8_gather_kernel<float><<<g, 256, 0, st>>>((const float*)x, rscale, perm, k, K, (uint8_t*)out, block_rows); break;
+    case STMOE_F16: quantize_fp8_gather_kernel<f16_t><<<g, 256, 0, st>>>((const f16_t*)x, rscale, perm, k, K, (uint8_t*)out, block_rows); break;
+    case STMOE_BF16: quantize_fp8_gather_kernel<bf16_t><<<g, 256, 0, st>>>((const bf16_t*)x, rscale, perm, k, K, (uint8_t*)out, block_rows); break;
+    default: return set_error(STMOE_ERR_DTYPE, "quantize_fp8_gather: dtype %d is not f32/f16/bf16", dtype);
+  }
+  return check_launch("quantize_fp8_gather");
+}
+}  // namespace stmoe
 
 extern "C" size_t stmoe_dynamic_quantize_fp8_scratch_bytes(void) { return 1024 * sizeof(float); }
 

@@ -68,11 +68,15 @@ static inline int64_t skinny_max_avg_rows(int E) { return E <= 4 ? 28 : 16; }
 static constexpr int64_t kSkinnyMaxRowsSingle = 48;
 // fp8 activations x fp8 weights on the fp8 matrix cores: the 256 x 256 kernel for packed weights and launches with
 // enough rows to fill its tiles (variant 5), the 128 x 128 kernel otherwise (and always with variant 7).
+// Whether the 256 x 256 kernel takes a projection (its token rows must come without a gather: see fp8_ws_takes' caller).
+static bool fp8_ws_takes(int variant, int wtag, int mode, int64_t kred, int64_t lda, int64_t ldo, int64_t n_out, bool offsets, int E,
+                         int64_t max_rows) {
+  return variant == 5 && wtag == WF_FP8_F32D_P && max_rows >= 320 && kred % 256 == 0 && lda % 16 == 0 && ldo % 4 == 0 &&
+         n_out % (mode == MODE_GATEUP ? 128 : 256) == 0 && (!offsets || E < 64) && max_rows * lda < ((int64_t)1 << 32);
+}
 static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
-  const bool ws_ok = variant == 5 && wtag == WF_FP8_F32D_P && max_rows >= 320 && p.kred % 256 == 0 && p.lda % 16 == 0 &&
-                     p.ldo % 4 == 0 && p.n_out % (mode == MODE_GATEUP ? 128 : 256) == 0 && (!p.offsets || p.E < 64) &&
-                     max_rows * p.lda < ((int64_t)1 << 32);
-  if (ws_ok) return launch_fp8_ws(dtype, wtag, mode, p, max_rows, st);
+  if (!p.perm && fp8_ws_takes(variant, wtag, mode, p.kred, p.lda, p.ldo, p.n_out, p.offsets != nullptr, p.E, max_rows))
+    return launch_fp8_ws(dtype, wtag, mode, p, max_rows, st);
   return launch_fp8_tile(dtype, wtag, mode, p, max_rows, st);
 }
 
@@ -123,7 +127,8 @@ static FfnWs carve_ffn(int64_t T, int k, int64_t K, int64_t N, int dtype) {
   const size_t es = dtype_size(dtype);
   w.z = 0;
   w.xa = align_up((size_t)T * k * N * es, 256);
-  w.zq = w.xa + align_up((size_t)T * K * es, 256);
+  // (the fp8 matrix-core path keeps one quantised row per (token, slot) pair there, grouped by expert)
+  w.zq = w.xa + align_up(std::max((size_t)T * K * es, (size_t)T * k * K), 256);
   w.split = w.zq + align_up((size_t)T * k * N, 256);
   // fp32 partial tiles of split reductions (prefill kernels only)
   w.total = w.split + (T * k > 128 ? align_up(mfma_ws_partial_bytes(), 256) : 0);  // kSkinnyMaxRows: smaller launches stream
@@ -197,6 +202,9 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   const int v16 = (variant == 5 || variant == 7) ? 0 : variant;
   float* const split = ws.total > ws.split ? reinterpret_cast<float*>(base + ws.split) : nullptr;
   const int32_t n_experts = offsets ? E : 1;
+  const bool z_blocked = mfma8_in && mfma8_out &&
+                         fp8_ws_takes(variant, weight_tag(w_gate), MODE_GATEUP, K, K, N, N, offsets != nullptr, n_experts, rows) &&
+                         fp8_ws_takes(variant, weight_tag(w_down), MODE_DOWN, N, N, K, K, offsets != nullptr, n_experts, rows);
 
   if (do_in) {
     GemmParams p{};
@@ -207,17 +215,28 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
     p.split_tickets_zeroed = tickets_zeroed;
     mark(events, 0, st);
     if (x_scale && !(x_is_fake_quantized && !mfma8_in)) {  // (the fused forward's norm launch may have done it already)
-      if (mfma8_in) rc = stmoe_quantize_fp8(x, dtype, x_scale, T * K, xa, stream);
+      // The 256 x 256 fp8 kernel streams its token rows in sorted order: the quantising pass writes them grouped by expert
+      // (one row per pair) and the projection needs no gather.  The 128 x 128 kernel gathers itself.
+      const bool sorted_rows = mfma8_in && perm &&
+                               fp8_ws_takes(variant, weight_tag(w_gate), MODE_GATEUP, K, K, N, N, offsets != nullptr, n_experts, rows);
+      if (sorted_rows) rc = quantize_fp8_gather(x, dtype, x_scale, perm, k, rows, K, xa, rows, st);
+      else if (mfma8_in) rc = stmoe_quantize_fp8(x, dtype, x_scale, T * K, xa, stream);
       else rc = stmoe_fake_quant_fp8(x, dtype, x_scale, T * K, xa, stream);
       if (rc) return rc;
       p.a = xa;
+      if (sorted_rows) { p.perm = nullptr; p.k_top = 1; p.a_block_rows = rows; }
     }
     // the quantizer of the intermediate is applied by the gate/up kernels themselves (16-bit kernels; the fp8 matrix-core
     // kernels write real e4m3fn samples instead)
     if (z_scale && stages == 3 && !mfma8_out && !mfma8_in) p.out_fq = z_scale;
     if (mfma8_in) {
       p.x_scale = x_scale;
-      if (mfma8_out) { p.out = zq; p.out_scale = z_scale; }
+      if (mfma8_out) {
+        p.out = zq;
+        p.out_scale = z_scale;
+        // the quantised intermediate goes from one 256 x 256 fp8 launch to the other in blocks of 64 reduction samples
+        if (z_blocked) p.out_block_rows = rows;
+      }
       rc = run_fp8_projection(variant, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
     } else {
       rc = run_projection(v16, dtype, weight_tag(w_gate), MODE_GATEUP, p, rows, st);
@@ -244,6 +263,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   if (mfma8_out) {
     q.a = zq;
     q.x_scale = z_scale;
+    if (z_blocked) q.a_block_rows = rows;
     rc = run_fp8_projection(variant, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);
   } else {
     rc = run_projection(v16, dtype, weight_tag(w_down), MODE_DOWN, q, rows, st);

@@ -29,6 +29,10 @@ struct GemmParams {
   int32_t act;
   const float* x_scale;   // optional scale applied to the fp32 dot products (fp8 activations)
   const float* out_scale; // fp8 kernel only: quantise the result with this reciprocal scale and store e4m3fn bytes
+  // fp8 256 x 256 kernel only: e4m3fn activations / results laid out in blocks of 64 reduction samples, [K / 64][rows][64]
+  // with `..._block_rows` rows per block (0: plain rows of lda / ldo bytes).  A wavefront's load of 16 token rows of one K
+  // stage is then one contiguous kilobyte instead of sixteen half cache lines.
+  int64_t a_block_rows, out_block_rows;
   const float* out_fq;    // GATEUP, 16-bit kernels: fake-quantise the gated product with this reciprocal scale (see below)
   int64_t expert_rows_bound;  // host-side bound of rows per expert (a token gives an expert at most one row)
   float* split_scratch;       // optional fp32 scratch for split reductions (mfma_ws_partial_bytes() bytes)

@@ -23,6 +23,9 @@ int norm_router(const void* h, int dtype, const void* norm_w, int w_dtype, float
 int dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* inv,
                    int32_t* zero_words, int n_zero, hipStream_t st);
 
+int quantize_fp8_gather(const void* x, int dtype, const float* rscale, const int32_t* perm, int k, int64_t rows, int64_t K, void* out,
+                        int64_t block_rows, hipStream_t st);
+
 #define STMOE_REQUIRE(cond, code, ...)            \
   do {                                            \
     if (!(cond)) return ::stmoe::set_error((code), __VA_ARGS__); \
@@ -138,6 +141,10 @@ struct FakeQuant {
     const float q = round_to<T>(q1);
     // fminf / fmaxf drop a NaN operand; torch.clamp keeps it
     return q != q ? __uint_as_float(0x7fc00000u) : fminf(fmaxf(q, -448.0f), 448.0f);
+  }
+  // the e4m3fn samples of two values in the two low bytes
+  template <typename T> __device__ __forceinline__ uint32_t quantize2(float a, float b) const {
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(clamped_quotient<T>(a), clamped_quotient<T>(b), 0, false) & 0xffffu;
   }
   template <typename T> __device__ __forceinline__ void pair(float& a, float& b) const {
     const int bytes = __builtin_amdgcn_cvt_pk_fp8_f32(clamped_quotient<T>(a), clamped_quotient<T>(b), 0, false);

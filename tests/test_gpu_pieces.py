@@ -587,3 +587,9 @@ def test_fake_quant_every_16_bit_value_against_eager_torch(device, dtype):
         got = _hip().fake_quant_fp8(xd, rs.to(device)).cpu()
         same = (got.view(torch.int16) == want.view(torch.int16)) | (torch.isnan(got) & torch.isnan(want))
         assert bool(same.all()), f"scale {s!r}: {int((~same).sum())} of 65536 values differ, first at bits {int(bits[~same][0]) & 0xffff:#06x}"
+        # the quantizer's samples themselves (the fp8 matrix-core path consumes them as bytes)
+        want_qs, _, _ = O.static_quantize_per_tensor(x, rs, torch.float8_e4m3fn)
+        got_qs = _hip().quantize_fp8(xd, rs.to(device)).cpu()
+        a, b = got_qs.view(torch.uint8), want_qs.view(torch.uint8)
+        same = (a == b) | ((a & 0x7f) == 0x7f) & ((b & 0x7f) == 0x7f)  # (any NaN code for NaN)
+        assert bool(same.all()), f"scale {s!r}: {int((~same).sum())} quantised samples differ, first at bits {int(bits[~same][0]) & 0xffff:#06x}"
