@@ -281,8 +281,10 @@ def config_legs(dev, steps, warmup):
     gates = torch.full((T5, TOPK), 0.5, dtype=torch.float16, device=dev)
     fl5 = 2.0 * T5 * TOPK * 3 * N_FFN * K_HID
     c5 = {"tokens": T5, "routing": "token t -> experts 2t mod 8, 2t+1 mod 8"}
-    for label, variant, peak in (("dequantise_then_f16_mfma", _hip.VARIANT_AUTO, MFMA_F16_PEAK_TFLOPS),
-                                 ("fp8_mfma", _hip.VARIANT_FP8_MFMA, 5000.0)):
+    # the default for fp16 activations is the fp8 matrix-core arithmetic; VARIANT_STEP_BY_STEP is the reference's
+    # quantise, dequantise, multiply in fp16
+    for label, variant, peak in (("dequantise_then_f16_mfma", _hip.VARIANT_STEP_BY_STEP, MFMA_F16_PEAK_TFLOPS),
+                                 ("fp8_mfma", _hip.VARIANT_AUTO, 5000.0)):
         ffn = PreGatherFFNMOE(theta)
         ffn._dw = block.experts.device_weights()
         ffn.kernel_variant = variant

@@ -216,15 +216,20 @@ size_t stmoe_moe_forward_workspace_bytes(int64_t T, int k, int E, int64_t K, int
  * per-tensor e4m3fn quantizers (StaticScaledQuantizer, quantizers.py:153-183) applied to x before the gate/up
  * projections and to the intermediate before the down projection.  The reference semantics is quantise then
  * dequantise (`quantize(x).unpack().dequant()`, sharktank/sharktank/layers/linear.py:72-78) followed by the
- * floating-point path, and that is what variant 0 computes (quantise, dequantise, 16-bit kernels).  Variant 5 with FP8
- * weights feeds both operands to the fp8 matrix cores as bytes and scales the fp32 dot product once by scale_x * d_w
- * (variant 7: the same arithmetic on the general 128x128 tile kernel only).
+ * floating-point path: quantise, dequantise, 16-bit kernels, every rounding where the reference rounds (the quantizers are
+ * applied by the kernels that produce the tensors).  With FP8 weights the other arithmetic is to feed both operands to the
+ * fp8 matrix cores as bytes and scale the fp32 dot product once by scale_x * d_w, which skips the rounding of the
+ * dequantised operands to `dtype` (variant 5; variant 7: the same on the general 128x128 tile kernel only).  Variant 0
+ * takes the matrix-core arithmetic where it is both much faster and well inside the fp8 tolerance of 2e-2 (packed FP8
+ * weights with fp32 scales, both quantizers, F16 activations, at least 320 rows, K and N multiples of 256) and the
+ * step-by-step arithmetic everywhere else (BF16 activations included); variant 8 never leaves the step-by-step arithmetic.
  * x itself is always given unquantised in `dtype`.
  * `perm` may be NULL when k == 1 and the rows of x are already grouped by expert (sorted row i is row i of x): with
  * E == 1 this is the plain feed-forward network of one expert (FFNMOE,
  * sharktank/sharktank/layers/ffn_moe_block.py:77-127; FFN, sharktank/sharktank/layers/ffn_block.py:21-51), and `offsets`
  * may then be NULL (the expert owns all T rows): no device array has to be built for the call.
- * `variant` 0 picks the kernel by shape; other values force one (see the kernel list in ffn.hip). */
+ * `variant` 0 picks the kernel by shape (8: the same, restricted to the reference's arithmetic); other values force one
+ * (see the kernel list in ffn.hip). */
 int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                       const stmoe_weight* w_gate, const stmoe_weight* w_up, const stmoe_weight* w_down,
                       int act, const int32_t* offsets, const int32_t* perm, const float* x_scale /*nullable*/,

@@ -46,7 +46,24 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 // variant: 0 auto, 1 generic (vector ALU), 2 MFMA 128x128 tile, 3 skinny streaming kernel (decode),
 //          4 MFMA 256x256 tile (prefill; packed Q8_0), 5 fp8 matrix cores (fp8 weights and quantised activations),
 //          6 MFMA 256x256 tile with specialised producer/consumer wavefronts (prefill; packed formats),
-//          7 fp8 matrix cores, 128x128 tile kernel only (5 uses the 256x256 LDS-direct kernel where it applies)
+//          7 fp8 matrix cores, 128x128 tile kernel only (5 uses the 256x256 LDS-direct kernel where it applies),
+//          8 auto among the kernels that follow the reference's arithmetic step by step (never the fp8 matrix cores)
+// Automatic choice with fp8 weights and static quantizers on both activations: a prefill-sized launch with fp16
+// activations goes to the fp8 matrix cores (variant 5: both operands as bytes, the fp32 dot product scaled once; 1.8 times
+// faster than dequantise-then-multiply, and 6e-3 from it on the layer output at the Mixtral shape, inside the 2e-2 the fp8
+// configuration is held to).  bf16 activations stay on the step-by-step path: there the two arithmetics are up to 4e-2
+// apart (the reference rounds the dequantised operands to 8 significant bits first).  Smaller launches stream the
+// weights and are bound by memory either way.
+static int effective_variant(int variant, int dtype, int64_t rows, int64_t K, int64_t N, const stmoe_weight* w_gate,
+                             const stmoe_weight* w_up, const stmoe_weight* w_down, const float* x_scale, const float* z_scale) {
+  if (variant == 8) return 0;
+  if (variant != 0) return variant;
+  const bool fp8_all = w_gate && w_up && w_down && w_gate->format == STMOE_W_FP8_PACKED && w_up->format == STMOE_W_FP8_PACKED &&
+                       w_down->format == STMOE_W_FP8_PACKED && w_gate->dtype == STMOE_F32 && w_up->dtype == STMOE_F32 &&
+                       w_down->dtype == STMOE_F32;
+  if (fp8_all && x_scale && z_scale && dtype == STMOE_F16 && rows >= 320 && K % 256 == 0 && N % 256 == 0) return 5;
+  return 0;
+}
 // Automatic choice of a grouped launch (the host knows the row total and the token count, not the rows per expert):
 // the streaming kernel when no expert can get more than 32 rows (token count <= 32), when the launch has at most 128 rows
 // in all (such launches get no scratch for split reductions, without which the prefill kernel leaves most CUs idle), or
@@ -158,6 +175,7 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
                 "grouped_ffn: activation dtype %d is not f32/f16/bf16", dtype);
   STMOE_REQUIRE(act == STMOE_ACT_SILU || act == STMOE_ACT_GELU_ERF, STMOE_ERR_UNSUPPORTED, "grouped_ffn: activation %d", act);
   const bool do_in = (stages & 1) != 0, do_out = (stages & 2) != 0;
+  if (variant == 8) variant = 0;  // (the entry points have resolved the automatic choice: effective_variant)
   int rc;
   if (do_in) {
     if ((rc = check_weight(w_gate, "grouped_ffn(ffn_gate_exps)", E, N, K))) return rc;
@@ -277,6 +295,7 @@ extern "C" int stmoe_grouped_ffn(const void* x, int dtype, int64_t T, int64_t K,
                                  int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
                                  const float* z_scale, void* y_sorted, void* workspace, size_t workspace_bytes,
                                  int variant, stmoe_stream_t stream) {
+  variant = effective_variant(variant, dtype, T * k, K, N, w_gate, w_up, w_down, x_scale, z_scale);
   return grouped_ffn_impl(x, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, z_scale, y_sorted,
                           workspace, workspace_bytes, variant, stream, nullptr);
 }
@@ -404,6 +423,7 @@ static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int6
   mark(events, 2, st);
   // a single token's dispatch is written by the router launch itself
   const bool router_dispatches = fused_front && T == 1;
+  variant = effective_variant(variant, dtype, T * k, K, N, w_gate, w_up, w_down, x_scale, z_scale);
   // a static quantizer of the experts' input rides in the norm launch (which writes the rows the experts read) unless the
   // fp8 matrix-core kernels want real e4m3fn samples
   const float* x_fq = (fused_front && x_scale && variant != 5 && variant != 7) ? x_scale : nullptr;

@@ -98,11 +98,18 @@ def test_small_quantized_layers(device, fmt, dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("T", [1, 24, 200, 700])
 def test_fp8_weights_and_fp8_activations(device, dtype, T):
-    """fp8 tensor-scaled weights with static fp8 quantizers on the FFN input and the gated intermediate.  The default
-    path quantises and dequantises the activations and multiplies in the activation dtype, which is the reference's
-    own arithmetic: the MoE contribution itself (without the residual) matches the oracle to the 16-bit tolerance."""
+    """fp8 tensor-scaled weights with static fp8 quantizers on the FFN input and the gated intermediate.  The
+    step-by-step path quantises and dequantises the activations and multiplies in the activation dtype, which is the
+    reference's own arithmetic: the MoE contribution itself (without the residual) matches the oracle to the 16-bit
+    tolerance.  (The automatic choice equals it for bf16 and for launches of fewer than 320 rows; larger fp16 launches go
+    to the fp8 matrix cores: test_fp8_matrix_core_layer.)"""
+    from sharktank_amd import _hip
+
     case = MC.Case(T=T, K=512, N=768, fmt="fp8", dtype=dtype, act_quant=True, seed=40 + T)
-    err, err_y = check_case(case, device, tol=1e-3)
+    err, err_y = check_case(case, device, variant=_hip.VARIANT_STEP_BY_STEP, tol=1e-3)
+    if dtype == torch.bfloat16 or T * 2 < 320:
+        built = MC.build(MC.Case(T=T, K=512, N=768, fmt="fp8", dtype=dtype, act_quant=True, seed=40 + T))
+        assert torch.equal(run_block(built, device, _hip.VARIANT_AUTO)[0], run_block(built, device, _hip.VARIANT_STEP_BY_STEP)[0])
     assert err < (1e-3 if dtype == torch.float16 else 3e-3), f"MoE contribution rel-L2 {err:.3e}"
 
 
@@ -120,6 +127,9 @@ def test_fp8_matrix_core_layer(device, dtype, T):
 
     case = MC.Case(T=T, K=512, N=768, fmt="fp8", dtype=dtype, act_quant=True, seed=40 + T)
     err, err_y = check_case(case, device, variant=_hip.VARIANT_FP8_MFMA, tol=2e-2, moe_tol=2e-2 if dtype == torch.float16 else 6e-2)
+    if dtype == torch.float16 and T * 2 >= 320:  # what the automatic choice takes for such a launch
+        built = MC.build(MC.Case(T=T, K=512, N=768, fmt="fp8", dtype=dtype, act_quant=True, seed=40 + T))
+        assert torch.equal(run_block(built, device, _hip.VARIANT_AUTO)[0], run_block(built, device, _hip.VARIANT_FP8_MFMA)[0])
     if dtype == torch.bfloat16:
         case = MC.build(case)
         y, _, _ = run_block(case, device, _hip.VARIANT_FP8_MFMA)
@@ -433,6 +443,7 @@ def test_fused_activation_quantizers_equal_separate_passes(device, fmt, dtype, T
     case = MC.build(MC.Case(T=T, K=K, N=N, fmt=fmt, dtype=dtype, act_quant=True, seed=300 + T))
     theta = MC.make_theta(case, device)
     block = MoeBlock(theta, case.E, case.k, case.eps)
+    block.experts.kernel_variant = _hip.VARIANT_STEP_BY_STEP  # (the fp8 matrix cores take real samples, not these values)
     wg, wu, wd = block.experts.device_weights()
     h = case.planes["h"].to(device)
     fused, idx_f, gate_f = block(h.reshape(1, T, K), return_routing=True)
@@ -450,5 +461,6 @@ def test_fused_activation_quantizers_equal_separate_passes(device, fmt, dtype, T
     staged = _hip.combine(y, gate, inv, T, case.k, residual=h)
     assert torch.equal(staged.view(torch.int16), fused.reshape(T, K).view(torch.int16))
     # the grouped FFN on its own takes both scales too
-    y2 = _hip.grouped_ffn(xn, wg, wu, wd, block.experts._act, offsets, perm, case.k, x_scale=xs, z_scale=zs)
+    y2 = _hip.grouped_ffn(xn, wg, wu, wd, block.experts._act, offsets, perm, case.k, x_scale=xs, z_scale=zs,
+                          variant=_hip.VARIANT_STEP_BY_STEP)
     assert torch.equal(y2.view(torch.int16), y.view(torch.int16))
