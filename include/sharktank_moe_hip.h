@@ -337,9 +337,17 @@ int stmoe_probe_mfma(int kind, int random_operands, int iters, float* sink, doub
  * `mmt_block_scaled_q8(a,d,qs)` (sharktank/sharktank/kernels/mmt_block_scaled_q8.py:30) and
  * `mmt_block_scaled_offset_q4_unsigned(a,d,qs,m)` (mmt_block_scaled_offset_q4.py:31), reached from
  * ops.matmul(Tensor, QuantizedTensor, transpose_rhs=True) (sharktank/sharktank/ops/custom_impls.py:66-103).
- * a [M,K], out [M,rows], both `dtype`; fp32 accumulation. */
-int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight* w, void* out, int variant,
-              stmoe_stream_t stream);
+ * a [M,K], out [M,rows], both `dtype`; fp32 accumulation.
+ * `workspace` (nullable; stmoe_mmt_workspace_bytes(M) bytes, 16-byte aligned): scratch for reductions split over several
+ * workgroups, which lets a launch of a few hundred rows (too few 256 x 256 units for 256 CUs) use the whole chip; without
+ * it the result is the same up to the grouping of the fp32 sums, the launch only slower.  The workspace ends in a few
+ * counters that elect the workgroup which adds a split unit's chunks; every call leaves them at zero.
+ * `workspace_ready` != 0: the caller vouches that the workspace was zero-filled before its first use and has since been
+ * written only by calls of this function (on one stream at a time); 0: the counters are cleared first, one small launch
+ * more (5 us). */
+size_t stmoe_mmt_workspace_bytes(int64_t M);
+int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight* w, void* out, void* workspace /*nullable*/,
+              size_t workspace_bytes, int workspace_ready, int variant, stmoe_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -81,8 +81,11 @@ static constexpr int64_t kSkinnyMaxRows = 128;  // == the largest T * k without 
 static inline int64_t skinny_max_avg_rows(int E) { return E <= 4 ? 28 : 16; }
 // A single matrix (no grouping): the streaming kernel re-reads the weights once per 32 rows and wins up to 48 rows
 // (24 / 38 / 45 / 58 us at 32 / 48 / 64 / 80 rows of a [14336, 4096] Q8_0 matrix, against 37 / 38 / 40 / 48 us for the
-// 256 x 256 kernel, which takes 50 us at 96-128 rows and 74-82 us from 129 to 512).
+// 256 x 256 kernel, which takes 50 us at 96-128 rows and 74-82 us from 129 to 512).  With scratch for split reductions
+// the 256 x 256 kernel cuts its 56 units into 224 chunks and takes 30 / 39 / 58 / 77 us at 64 / 128 / 256 / 512 rows
+// (Q4_1: 33 / 43 / 60 / 79): it then wins from 33 rows on.
 static constexpr int64_t kSkinnyMaxRowsSingle = 48;
+static constexpr int64_t kSkinnyMaxRowsSingleSplit = 32;
 // fp8 activations x fp8 weights on the fp8 matrix cores: the 256 x 256 kernel for packed weights and launches with
 // enough rows to fill its tiles (variant 5), the 128 x 128 kernel otherwise (and always with variant 7).
 // Whether the 256 x 256 kernel takes a projection (its token rows must come without a gather: see fp8_ws_takes' caller).
@@ -100,7 +103,7 @@ static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const 
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
-    else if (!p.offsets && p.E == 1) variant = max_rows <= kSkinnyMaxRowsSingle ? 3 : 6;
+    else if (!p.offsets && p.E == 1) variant = max_rows <= (p.split_scratch ? kSkinnyMaxRowsSingleSplit : kSkinnyMaxRowsSingle) ? 3 : 6;
     else if (p.offsets && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
                            max_rows <= kSkinnyMaxRows || max_rows <= skinny_max_avg_rows(p.E) * p.E)) variant = 3;
     // Everything else goes to the 256 x 256 kernel (which hands shapes it does not take down to the 128 x 128 one).
@@ -315,8 +318,14 @@ extern "C" int stmoe_grouped_down(const void* z_sorted, int dtype, int64_t T, in
                           y_sorted, workspace, workspace_bytes, variant, stream, nullptr, false, 2, const_cast<void*>(z_sorted));
 }
 
-extern "C" int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight* w, void* out, int variant,
-                         stmoe_stream_t stream) {
+extern "C" size_t stmoe_mmt_workspace_bytes(int64_t M) {
+  // fp32 partial tiles of split reductions: only launches between the streaming kernel's window and a chip-filling number
+  // of units can use them (see stmoe_mmt)
+  return M > kSkinnyMaxRowsSingleSplit ? align_up(mfma_ws_partial_bytes(), 256) : 0;
+}
+
+extern "C" int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight* w, void* out, void* workspace,
+                         size_t workspace_bytes, int workspace_ready, int variant, stmoe_stream_t stream) {
   STMOE_REQUIRE(w, STMOE_ERR_NULL, "mmt: weight descriptor is NULL");
   STMOE_REQUIRE(M >= 0, STMOE_ERR_SHAPE, "mmt: M=%lld", (long long)M);
   STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
@@ -332,6 +341,13 @@ extern "C" int stmoe_mmt(const void* a, int dtype, int64_t M, const stmoe_weight
   p.a = a; p.lda = w->cols; p.perm = nullptr; p.k_top = 1; p.offsets = nullptr; p.E = 1; p.fixed_rows = M;
   p.w0 = make_view(w); p.w1 = p.w0;
   p.out = out; p.ldo = w->rows; p.n_out = w->rows; p.kred = w->cols; p.act = 0; p.x_scale = nullptr;
+  // With a workspace the prefill kernel cuts the units that do not fill a round over the CUs along the reduction (256 rows
+  // of a [14336, 4096] matrix are 56 units for 256 CUs: four chunks each make 224 workgroups).
+  if (workspace && workspace_bytes >= stmoe_mmt_workspace_bytes(M) && stmoe_mmt_workspace_bytes(M) > 0) {
+    STMOE_REQUIRE(aligned16(workspace), STMOE_ERR_ALIGN, "mmt: workspace must be 16-byte aligned");
+    p.split_scratch = reinterpret_cast<float*>(workspace);
+    p.split_tickets_zeroed = workspace_ready != 0;
+  }
   return run_projection(variant, dtype, weight_tag(w), MODE_DOWN, p, M, as_stream(stream));
 }
 

@@ -56,8 +56,12 @@ struct WsArgs {
 // 0..127 of the partial tile) and the up sums (columns 128..255).
 static constexpr size_t kWsSlotFloats = (size_t)256 * (256 + kBigTailRows);
 static constexpr int kWsTickets = 8 * kBigChunkSlotsPerXcd;
-template <typename T, int MODE>
-__device__ __forceinline__ void ws_reduce_row(const GemmParams& p, const BigTile& t, const float* base, int chunks, int r, int c8) {
+// The adding workgroup is the tail of its unit and works alone, so its loads must overlap: the chunk count is a template
+// argument and a thread first issues the loads of all chunks for 64 of its row's columns (up to 16 loads of 16 bytes in
+// flight per thread), then adds them.  (With the chunk count a run-time value every load waited for the one before: the
+// sum of one 256-row unit took 45 us, as long as its reduction steps.)
+template <typename T, int MODE, int CHUNKS>
+__device__ __forceinline__ void ws_reduce_row(const GemmParams& p, const BigTile& t, const float* base, int r, int c8) {
   constexpr int BN = 256, BM = 256;
   const int rows_here = t.row_end - t.row_begin;
   int sorted_row;
@@ -65,30 +69,49 @@ __device__ __forceinline__ void ws_reduce_row(const GemmParams& p, const BigTile
   else if (r >= BM && r - BM < t.tail_rows) sorted_row = t.tail_begin + (r - BM);
   else return;
   base += (size_t)r * BN;
-  auto total = [&](int col) {
-    floatx4_t sum = *reinterpret_cast<const floatx4_t*>(base + col);
-    for (int c = 1; c < chunks; ++c) sum = sum + *reinterpret_cast<const floatx4_t*>(base + (size_t)c * kWsSlotFloats + col);
-    return sum;
-  };
+  // columns of this thread: (c8 + 8 j) * 4 for j = 0..7 (DOWN), or that gate column and its up column for j = 0..3
+  auto col_of = [&](int i) { return MODE == MODE_GATEUP ? (i >> 2) * (BN / 2) + (c8 + 8 * (i & 3)) * 4 : (c8 + 8 * i) * 4; };
   T* orow = reinterpret_cast<T*>(p.out) + out_row(p, sorted_row) * p.ldo;
-  if (MODE == MODE_GATEUP) {
-    const FakeQuant fq = fq_scale(p);
+  const FakeQuant fq = fq_scale(p);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int col = (c8 + 8 * j) * 4;
-      const floatx4_t gs = total(col), us = total(BN / 2 + col);
-      const float gq[4] = {gs[0], gs[1], gs[2], gs[3]}, uq[4] = {us[0], us[1], us[2], us[3]};
-      uint2* dst = reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * (BN / 2) + col);
-      if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq, fq);
-      else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq, fq);
-    }
-  } else {
+  for (int half = 0; half < 2; ++half) {
+    // GATEUP: j = 2 half, 2 half + 1 (i = j and 4 + j); DOWN: j = 4 half .. 4 half + 3
+    floatx4_t v[4][CHUNKS];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int col = (c8 + 8 * j) * 4;
-      const floatx4_t sum = total(col);
-      *reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * BN + col) = make_uint2(pack2<T>(sum[0], sum[1]), pack2<T>(sum[2], sum[3]));
+    for (int q = 0; q < 4; ++q) {
+      const int i = MODE == MODE_GATEUP ? (q >> 1) * 4 + 2 * half + (q & 1) : 4 * half + q;
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) v[q][c] = *reinterpret_cast<const floatx4_t*>(base + (size_t)c * kWsSlotFloats + col_of(i));
     }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int c = 1; c < CHUNKS; ++c) v[q][0] = v[q][0] + v[q][c];
+    if (MODE == MODE_GATEUP) {
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const floatx4_t gs = v[q][0], us = v[2 + q][0];
+        const float gq[4] = {gs[0], gs[1], gs[2], gs[3]}, uq[4] = {us[0], us[1], us[2], us[3]};
+        uint2* dst = reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * (BN / 2) + col_of(2 * half + q));
+        if (p.act == STMOE_ACT_SILU) *dst = gateup_quad<T, STMOE_ACT_SILU>(gq, uq, fq);
+        else *dst = gateup_quad<T, STMOE_ACT_GELU_ERF>(gq, uq, fq);
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const floatx4_t sum = v[q][0];
+        *reinterpret_cast<uint2*>(orow + (int64_t)t.ntile * BN + col_of(4 * half + q)) = make_uint2(pack2<T>(sum[0], sum[1]), pack2<T>(sum[2], sum[3]));
+      }
+    }
+  }
+}
+template <typename T, int MODE>
+__device__ __forceinline__ void ws_reduce_unit(const GemmParams& p, const BigTile& t, const float* base, int tid) {
+  constexpr int BM = 256;
+  for (int r = tid >> 3; r < BM + kBigTailRows; r += 96) {
+    if (t.nchunks == 2) ws_reduce_row<T, MODE, 2>(p, t, base, r, tid & 7);
+    else if (t.nchunks == 3) ws_reduce_row<T, MODE, 3>(p, t, base, r, tid & 7);
+    else ws_reduce_row<T, MODE, 4>(p, t, base, r, tid & 7);
   }
 }
 __global__ void ws_zero_tickets_kernel(int* tickets) { tickets[threadIdx.x] = 0; }
@@ -586,7 +609,7 @@ grouped_mfma_ws_kernel(WsArgs args) {
     }
   };
   if (tile.nchunks > 1) {
-    // chunk of a split unit: fp32 partial tile [BM][BN], added to the other chunks by big_reduce_kernel
+    // chunk of a split unit: fp32 partial tile [BM][BN], added to the other chunks by the workgroup that finishes last (below)
     float* pt = partial + (size_t)tile.chunk_slot * (BN * (BM + kBigTailRows));
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
@@ -633,10 +656,12 @@ grouped_mfma_ws_kernel(WsArgs args) {
   }
   if (tile.nchunks > 1) {
     // chunk of a split unit (every wavefront of the workgroup gets here): the workgroup that draws the unit's last ticket
-    // adds the chunks.  Each thread's partial sums are made visible device-wide before the ticket is drawn, and the
-    // drawing workgroup drops what its caches hold before it reads the other chunks.  LDS is free after the unit's last
+    // adds the chunks.  One thread speaks for the workgroup: the barrier orders every thread's partial sums before its
+    // draw, whose release makes them visible device-wide (a write-back of the XCD's L2, which all of the workgroup's stores
+    // have reached by then) and whose acquire drops what this CU's caches hold of the other chunks before anyone here
+    // reads them.  A fence per thread would do the same write-back and invalidation twelve times per workgroup: with a few
+    // hundred split units in a launch those took longer than the units themselves.  LDS is free after the unit's last
     // K step; the next unit's loaders start only after the last barrier below.
-    __threadfence();
     __syncthreads();
     int* const drawn_s = reinterpret_cast<int*>(lds);
     int* const ticket = ka.tickets + (tile.chunk_slot - tile.chunk);
@@ -645,9 +670,8 @@ grouped_mfma_ws_kernel(WsArgs args) {
     const int drawn = *drawn_s;
     __syncthreads();
     if (drawn == tile.nchunks - 1) {
-      __threadfence();
       const float* base = partial + (size_t)(tile.chunk_slot - tile.chunk) * kWsSlotFloats;
-      for (int r = tid >> 3; r < BM + kBigTailRows; r += 96) ws_reduce_row<T, MODE>(p, tile, base, tile.nchunks, r, tid & 7);
+      ws_reduce_unit<T, MODE>(p, tile, base, tid);
       if (tid == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // as the launch found it
     }
   }

@@ -108,7 +108,8 @@ SIGNATURES = {
     "stmoe_moe_forward_static": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p,
                                          POINTER(StmoeWeight), POINTER(StmoeWeight), POINTER(StmoeWeight), c_int, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_int, c_void_p]),
-    "stmoe_mmt": (c_int, [c_void_p, c_int, c_int64, POINTER(StmoeWeight), c_void_p, c_int, c_void_p]),
+    "stmoe_mmt_workspace_bytes": (c_size_t, [c_int64]),
+    "stmoe_mmt": (c_int, [c_void_p, c_int, c_int64, POINTER(StmoeWeight), c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p]),
     "stmoe_probe_mfma": (c_int, [c_int, c_int, c_int, c_void_p, POINTER(ctypes.c_double), c_void_p]),
 }
 STATIC_SCRATCH_BYTES = 16 << 20  # STMOE_STATIC_SCRATCH_BYTES
@@ -675,8 +676,25 @@ def moe_forward_static(h, ffn_norm_w, out_norm_w, eps: float, w_router, w_gate: 
     return out
 
 
-def mmt(a: torch.Tensor, w: DeviceWeight, *, variant: int = VARIANT_AUTO) -> torch.Tensor:
-    """a [..., K] @ W[rows, K]^T -> [..., rows] in a's dtype."""
+_MMT_WORKSPACE = {}  # (device, stream) -> scratch of split reductions, allocated on the first product that can use it
+
+
+def _mmt_workspace(dev: torch.device, stream: int, need: int) -> Optional[torch.Tensor]:
+    """One scratch buffer per device and stream (launches on one stream run one after the other, so they can share it),
+    zero-filled once: only stmoe_mmt writes to it afterwards, which lets every call skip the clearing of its counters."""
+    if need == 0:
+        return None
+    key = (dev, stream)
+    ws = _MMT_WORKSPACE.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(need, dtype=torch.uint8, device=dev)
+        _MMT_WORKSPACE[key] = ws
+    return ws
+
+
+def mmt(a: torch.Tensor, w: DeviceWeight, *, variant: int = VARIANT_AUTO, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a [..., K] @ W[rows, K]^T -> [..., rows] in a's dtype.  `workspace`: scratch of stmoe_mmt_workspace_bytes(M) bytes;
+    by default a buffer kept per device and stream (pass one of your own under HIP graph capture)."""
     dev = _dev(a)
     lib = load_library()
     a_c = _contig(a)
@@ -684,7 +702,12 @@ def mmt(a: torch.Tensor, w: DeviceWeight, *, variant: int = VARIANT_AUTO) -> tor
     M = a_c.numel() // K if K else 0
     out = torch.empty(tuple(a_c.shape[:-1]) + (w.rows,), dtype=a_c.dtype, device=dev)
     with torch.cuda.device(dev):
-        _check(lib.stmoe_mmt(_ptr(a_c), dtype_enum(a_c.dtype), M, w.ref, _ptr(out), variant, _stream(dev)))
+        stream = _stream(dev)
+        ready = workspace is None  # a caller's buffer has an unknown history
+        if workspace is None:
+            workspace = _mmt_workspace(dev, stream, int(lib.stmoe_mmt_workspace_bytes(M)))
+        _check(lib.stmoe_mmt(_ptr(a_c), dtype_enum(a_c.dtype), M, w.ref, _ptr(out), _ptr(workspace),
+                             workspace.numel() if workspace is not None else 0, int(ready), variant, stream))
     return out
 
 

@@ -71,7 +71,7 @@ def test_linear_and_dense_matmul(device):
 @pytest.mark.parametrize("M,N", [(1, 96), (7, 96), (16, 256), (17, 96), (32, 256), (33, 96), (40, 256), (64, 256), (80, 96), (81, 256)])
 def test_quantized_linear_few_rows(device, fmt, dtype, M, N):
     """One quantized matrix times a handful of rows (a Llama-style projection at decode): the streaming kernel runs
-    without an expert offsets array (up to 48 rows by itself, beyond that on request), from planar and from packed
+    without an expert offsets array (up to 32 rows by itself, beyond that on request), from planar and from packed
     planes, with the same bits from both."""
     import moe_cases as MC
     from sharktank_amd import _hip
@@ -89,12 +89,46 @@ def test_quantized_linear_few_rows(device, fmt, dtype, M, N):
         auto = _hip.mmt(x.to(device), dw)
         assert O.rel_l2(auto.cpu(), ref) < (1e-3 if dtype == torch.float16 else 8e-3)
         forced = _hip.mmt(x.to(device), dw, variant=_hip.VARIANT_SKINNY)
-        if M <= 48:  # the automatic choice for so few rows is the streaming kernel (N = 256: its LDS-sharing form)
+        if M <= 32:  # the automatic choice for so few rows is the streaming kernel (N = 256: its LDS-sharing form)
             assert torch.equal(auto.view(torch.int16), forced.view(torch.int16))
         else:
             assert O.rel_l2(forced.cpu(), ref) < (1e-3 if dtype == torch.float16 else 8e-3)
         outs.append(forced.cpu())
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [33, 48, 129, 200, 256, 300, 512])
+def test_quantized_linear_few_hundred_rows_splits_the_reduction(device, fmt, dtype, M):
+    """A few hundred rows of one matrix make too few 256 x 256 units for the chip: with a workspace the units are cut along
+    the reduction and the chunk that finishes last adds the fp32 partial tiles.  Checked against the oracle's dense product
+    and against the launch without a workspace (one fp32 sum per output instead of four: equal to the rounding of the
+    output), twice in a row (the tickets that elect the adding workgroup must be back at zero)."""
+    import moe_cases as MC
+    from sharktank_amd import _hip
+    from sharktank_amd.ops import device_weight
+
+    K, N = 2048, 1792  # 7 column units: every one of them is split
+    case = MC.build(MC.Case(T=4, K=K, N=N, E=1, k=1, fmt=fmt, dtype=dtype, seed=300 + M))
+    it = MC.to_inference_tensor(fmt, case.planes["gate"], [1, N, K], "w", device)
+    x = (torch.randn(M, K, generator=torch.Generator().manual_seed(M)) * 0.5).to(dtype)
+    ref = O.mmt(x, MC.dense_weights(case)[0][0].to(dtype))
+    dw = device_weight(it, stacked=True, prepack=True)
+    lib = _hip.load_library()
+    need = int(lib.stmoe_mmt_workspace_bytes(M))
+    assert need > 0 and int(lib.stmoe_mmt_workspace_bytes(32)) == 0
+    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device=device)  # stale contents must not matter
+    tol = 1e-3 if dtype == torch.float16 else 8e-3
+    plain = _hip.mmt(x.to(device), dw, workspace=torch.empty(0, dtype=torch.uint8, device=device))
+    assert O.rel_l2(plain.cpu(), ref) < tol
+    first = _hip.mmt(x.to(device), dw, workspace=ws)
+    second = _hip.mmt(x.to(device), dw, workspace=ws)
+    default = _hip.mmt(x.to(device), dw)
+    assert O.rel_l2(first.cpu(), ref) < tol
+    assert torch.equal(first.view(torch.int16), second.view(torch.int16))
+    assert torch.equal(first.view(torch.int16), default.view(torch.int16))
+    assert O.rel_l2(first.float().cpu(), plain.float().cpu()) < (5e-4 if dtype == torch.float16 else 4e-3)
 
 
 def test_layout_classes_dequant_on_device(device):
