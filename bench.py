@@ -372,6 +372,15 @@ def measured_traffic(key):
         return None
 
 
+def traffic_measured_at():
+    """Which sources the counter runs behind profiles/traffic.json were made with (the file's own stamp), or None."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get("measured_at")
+    except (OSError, ValueError):
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -407,8 +416,8 @@ def main():
     roofline = {
         "kernel": "grouped gate/up projection (prefill)", "bound": "mfma", "achieved": round(achieved, 2),
         "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4),
-        "traffic": measured_traffic("prefill_gate_up") if T == 2048 else None, "avg_kernel_ms": round(gu_ms, 4),
-        "algorithmic": gateup_flops, "algorithmic_unit": "flop per launch",
+        "traffic": measured_traffic("prefill_gate_up") if T == 2048 else None, "traffic_measured_at": traffic_measured_at(),
+        "avg_kernel_ms": round(gu_ms, 4), "algorithmic": gateup_flops, "algorithmic_unit": "flop per launch",
     }
 
     dms, dgu_ms, dst, _, _, de2e_ms = run_leg(block, h_dec.to(dev), max(args.steps, 50), args.warmup, e2e=True)
@@ -469,8 +478,8 @@ def main():
         "metric": "MoE-layer tokens/s (Mixtral Q8_0 prefill)", "value": round(T / (ms * 1e-3), 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "Mixtral-8x7B MoE layer, Q8_0 expert weights, fp16 activations, hidden 4096, FFN 14336, "
-                               f"8 experts, top-2, SiLU; prefill {T} tokens", "parallelism": "1 GPU"},
+        "config": {"workload": f"Mixtral-8x7B MoE layer, prefill {T} tokens, Q8_0 weights, fp16, 8 experts top-2, 4096 x 14336, SiLU",
+                   "parallelism": "1 GPU"},
         "layer_tflops": round(layer_flops / (ms * 1e-3) / 1e12, 2),
         "e2e_ms_per_step": round(e2e_ms, 4),
         "stage_ms": {k: round(v, 4) for k, v in st.items()},
