@@ -563,11 +563,14 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
 template <int WF> struct SkinnyLdsOcc { static constexpr int value = 2; };
 
 // A workgroup takes groups of four neighbouring items (tiles 4q .. 4q+3 of one expert), strided by the grid size.
-template <typename T, int WF, int MODE>
+// MAXMT: the most 16-row token tiles a pass takes (2 or 4).  Launches in which no expert can have more than 32 rows get the
+// instance without four-tile passes: its registers and LDS are what the one- and two-tile passes need, and it is the
+// kernel of a 32-token decode step (the instance with four-tile passes runs those 0.4 % slower).
+template <typename T, int WF, int MODE, int MAXMT>
 __global__ void __launch_bounds__(256, SkinnyLdsOcc<WF>::value)
 grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
   constexpr int G = 1;                                     // chunks per pipeline step (the host checks K % (256 G) == 0)
-  __shared__ __align__(16) uint16_t xs[2 * G * 32 * 256];  // two stages of up to 32 token rows x 256 G reduction elements
+  __shared__ __align__(16) uint16_t xs[2 * G * 16 * MAXMT * 256];  // two stages of up to 16 MAXMT token rows x 256 G reduction elements
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n_in = lane & 15;
   const int64_t nch = p.kred >> 8;
@@ -606,10 +609,14 @@ grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
       wrow[0] = (int64_t)e * p.w0.rows + tile * 32 + n_in;
       wrow[1] = wrow[0] + 16;
     }
-    if (re - rb <= 16) {
-      skinny_lds_pass<T, WF, MODE, 1, G>(p, wrow, tile, rb, re, nch, lane, wave, xs, xs_addr);
-    } else {
-      for (int r0 = rb; r0 < re; r0 += 32) skinny_lds_pass<T, WF, MODE, 2, G>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
+    // Passes of up to 64 rows (four 16-row token tiles against the same weight registers): every pass streams the item's
+    // weights once, so an expert with 33..64 rows costs one pass, not two.  The token tiles only cost MFMAs, of which the
+    // kernel has plenty to spare (the matrix cores are busy in 0.07 of the cycles with one or two tiles).
+    for (int r0 = rb; r0 < re; r0 += 16 * MAXMT) {
+      const int left = re - r0;
+      if (left <= 16) skinny_lds_pass<T, WF, MODE, 1, G>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
+      else if (MAXMT == 2 || left <= 32) skinny_lds_pass<T, WF, MODE, 2, G>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
+      else skinny_lds_pass<T, WF, MODE, MAXMT, G>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
     }
   }
 }
@@ -647,8 +654,15 @@ static int launch_skinny_t(int mode, const GemmParams& p, int64_t max_rows, hipS
       const int64_t groups = (int64_t)(tiles / 4) * p.E, capacity = 256 * SkinnyLdsOcc<WF>::value;
       const int64_t per_wg = (groups + capacity - 1) / capacity;
       dim3 grid((unsigned)((groups + per_wg - 1) / per_wg));
-      if (mode == MODE_GATEUP) grouped_skinny_lds_kernel<T, WF, MODE_GATEUP><<<grid, 256, 0, st>>>(p, tiles);
-      else grouped_skinny_lds_kernel<T, WF, MODE_DOWN><<<grid, 256, 0, st>>>(p, tiles);
+      // the most rows one expert can have: one per token (when the caller says how many tokens there are), else all of them
+      const int64_t rows_bound = p.expert_rows_bound > 0 && p.expert_rows_bound < max_rows ? p.expert_rows_bound : max_rows;
+      if (rows_bound <= 32) {
+        if (mode == MODE_GATEUP) grouped_skinny_lds_kernel<T, WF, MODE_GATEUP, 2><<<grid, 256, 0, st>>>(p, tiles);
+        else grouped_skinny_lds_kernel<T, WF, MODE_DOWN, 2><<<grid, 256, 0, st>>>(p, tiles);
+      } else {
+        if (mode == MODE_GATEUP) grouped_skinny_lds_kernel<T, WF, MODE_GATEUP, 4><<<grid, 256, 0, st>>>(p, tiles);
+        else grouped_skinny_lds_kernel<T, WF, MODE_DOWN, 4><<<grid, 256, 0, st>>>(p, tiles);
+      }
       return check_launch("grouped_skinny_lds");
     }
   }

@@ -68,12 +68,13 @@ def test_every_expert_selected(device):
 
 @pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_streaming_kernel_packed_rows_per_expert(device, fmt, dtype):
-    """The packed streaming kernels (token rows shared through LDS) with 3, 16, 17, 40 and 70 rows on the experts: one
-    token tile, two tiles, and several passes over an expert's weights."""
-    E, T, k = 8, 73, 2
+@pytest.mark.parametrize("T,rows", [(73, {0: 3, 1: 16, 2: 17, 3: 40, 4: 70}), (122, {0: 33, 1: 48, 2: 64, 3: 65, 4: 32, 5: 2})])
+def test_streaming_kernel_packed_rows_per_expert(device, fmt, dtype, T, rows):
+    """The packed streaming kernels (token rows shared through LDS) with 2 ... 70 rows on the experts: passes of one, two
+    and four 16-row token tiles against one set of weight registers (up to 16, 32 and 64 rows), both sides of each limit,
+    and experts that need a second pass over their weights (65 = 64 + 1, 70 = 64 + 6)."""
+    E, k = 8, 2
     case = MC.build(MC.Case(T=T, K=512, N=1024, E=E, k=k, fmt=fmt, dtype=dtype, seed=74))
-    rows = {0: 3, 1: 16, 2: 17, 3: 40, 4: 70}
     pairs = [e for e, n in rows.items() for _ in range(n)]  # 146 = T * k pairs
     assert len(pairs) == T * k
     # deal the pairs so that a token never gets the same expert twice
