@@ -87,6 +87,17 @@ template <> struct Vec8<bf16_t> {
   }
 };
 
+// exp(d) for d = logit - max <= 0 as the softmax needs it.  Below -87 the result is a subnormal fp32 number (or zero);
+// the fp32 exponential returns zero there, which would turn distinct tiny probabilities into ties (resolved toward the
+// lower expert index) where the reference still tells them apart.  Such values are rare; they are computed as
+// exp(d + 32) * exp(-32), whose product is rounded into the subnormal range by the multiplication (d + 32 is exact for
+// logits that were rounded to a 16-bit type).
+__device__ __forceinline__ float softmax_exp(float d) {
+  float r = expf(d);
+  if (d < -87.0f) r = expf(d + 32.0f) * 1.2664165549094176e-14f;
+  return r;
+}
+
 // fp32 softmax over the E logits, top-k of the probabilities and renormalised gates of one token, computed alike by
 // every lane from the logits lg[0..E) (already rounded to T); lane 0 writes.
 template <typename T, int EP>
@@ -97,16 +108,19 @@ __device__ __forceinline__ void softmax_topk_store(const float (&lg)[EP], int E,
   float mx = lg[0];
 #pragma unroll
   for (int e = 1; e < EP; ++e) mx = fmaxf(mx, lg[e]);
+  float ex[EP];
   float denom = 0.0f;
 #pragma unroll
-  for (int e = 0; e < EP; ++e)
-    if (e < E) denom += expf(lg[e] - mx);
+  for (int e = 0; e < EP; ++e) {
+    ex[e] = e < E ? softmax_exp(lg[e] - mx) : 0.0f;
+    if (e < E) denom += ex[e];
+  }
   // The reference ranks the fp32 probabilities (F.softmax, then torch.topk): so does this kernel, with equal
   // probabilities ordered by increasing expert index.  Distinct logits whose probabilities round to the same fp32 number
   // (logits one ulp apart next to the maximum, say) therefore count as a tie, as they do for the reference.
   float pr[EP];
 #pragma unroll
-  for (int e = 0; e < EP; ++e) pr[e] = (e < E) ? expf(lg[e] - mx) / denom : 0.0f;
+  for (int e = 0; e < EP; ++e) pr[e] = (e < E) ? ex[e] / denom : 0.0f;
   uint64_t taken = 0;
   float vsum = 0.0f;
   float pv[EP];  // selected probabilities in slot order (only the first k are used)
@@ -354,7 +368,7 @@ router_wg_kernel(const T* __restrict__ x, const W* __restrict__ norm_w, float ep
   const float l = lane < E ? lg_s[lane] : 0.0f;
   float mx = __shfl(l, 0);
   for (int e = 1; e < E; ++e) mx = fmaxf(mx, __shfl(l, e));
-  const float ex = expf(l - mx);
+  const float ex = softmax_exp(l - mx);
   float denom = 0.0f;
   for (int e = 0; e < E; ++e) denom += __shfl(ex, e);
   const float pr = ex / denom;
@@ -661,7 +675,7 @@ softmax_rows_kernel(const void* __restrict__ x, int x_dtype, int64_t rows, int64
     const float l = lane < cols ? softmax_load(x, x_dtype, base + lane) : 0.0f;
     float mx = __shfl(l, 0);
     for (int e = 1; e < cols; ++e) mx = fmaxf(mx, __shfl(l, e));
-    const float ex = expf(l - mx);
+    const float ex = softmax_exp(l - mx);
     float denom = 0.0f;
     for (int e = 0; e < cols; ++e) denom += __shfl(ex, e);
     if (lane < cols) softmax_store(out, o_dtype, base + lane, ex / denom);
@@ -672,9 +686,9 @@ softmax_rows_kernel(const void* __restrict__ x, int x_dtype, int64_t rows, int64
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
   float sum = 0.0f;
-  for (int64_t c = lane; c < cols; c += 64) sum += expf(softmax_load(x, x_dtype, base + c) - mx);
+  for (int64_t c = lane; c < cols; c += 64) sum += softmax_exp(softmax_load(x, x_dtype, base + c) - mx);
   sum = wave_xor_sum(sum);
-  for (int64_t c = lane; c < cols; c += 64) softmax_store(out, o_dtype, base + c, expf(softmax_load(x, x_dtype, base + c) - mx) / sum);
+  for (int64_t c = lane; c < cols; c += 64) softmax_store(out, o_dtype, base + c, softmax_exp(softmax_load(x, x_dtype, base + c) - mx) / sum);
 }
 
 }  // namespace stmoe

@@ -152,8 +152,17 @@ def test_router_fp16_subnormal_and_large_operands(device, T):
     want_logits = O.router_logits_ordered(x, wr.float())
     assert bool(torch.isfinite(want_logits.float()).all())
     assert torch.equal(logits.cpu().view(torch.int16), want_logits.view(torch.int16))
-    # (no index check here: logits of this size put many probabilities within an ulp of each other, where the exponential
-    # of the device and the host's may order them differently; test_router_distinct_logits_with_equal_probabilities covers that)
+    # Indices: logits of this size put some probabilities within an ulp of each other, where the exponential of the device
+    # and the host's may order them differently (test_router_distinct_logits_with_equal_probabilities covers exact ties).
+    # Every row whose k + 1 largest probabilities are at least 8 ulp apart from each other must route exactly as the oracle.
+    want_idx, want_gate, probs = O.route(want_logits, k)
+    top = torch.sort(probs, dim=1, descending=True).values[:, : k + 1]
+    clear = ((top[:, :-1] - top[:, 1:]) > 8 * torch.finfo(torch.float32).eps * top[:, :-1]).all(dim=1)
+    # (logits this large saturate the softmax of many rows: their lower probabilities are zero or equal)
+    print(f"{int(clear.sum())} of {T} rows have separated probabilities")
+    assert int(clear.sum()) >= max(1, T // 10), f"only {int(clear.sum())} of {T} rows have separated probabilities"
+    assert torch.equal(idx.cpu()[clear], want_idx[clear])
+    assert O.rel_l2(gate.cpu()[clear], want_gate[clear]) < 2e-3
 
 
 def test_router_ties_lower_index_first(device):
