@@ -103,7 +103,8 @@ static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const 
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
-    else if (!p.offsets && p.E == 1) variant = max_rows <= (p.split_scratch ? kSkinnyMaxRowsSingleSplit : kSkinnyMaxRowsSingle) ? 3 : 6;
+    // (one matrix, with or without an offsets array around its rows)
+    else if (p.E == 1) variant = max_rows <= (p.split_scratch ? kSkinnyMaxRowsSingleSplit : kSkinnyMaxRowsSingle) ? 3 : 6;
     else if (p.offsets && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
                            max_rows <= kSkinnyMaxRows || max_rows <= skinny_max_avg_rows(p.E) * p.E)) variant = 3;
     // Everything else goes to the 256 x 256 kernel (which hands shapes it does not take down to the 128 x 128 one).
@@ -221,7 +222,12 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
   const bool mfma8_in = t16 && x_scale && fp8_w_in && w_gate->dtype == STMOE_F32 && K % 16 == 0 && want_mfma8;
   const bool mfma8_out = t16 && z_scale && fp8_w_out && w_down->dtype == STMOE_F32 && N % 16 == 0 && want_mfma8;
   const int v16 = (variant == 5 || variant == 7) ? 0 : variant;
-  float* const split = ws.total > ws.split ? reinterpret_cast<float*>(base + ws.split) : nullptr;
+  // Scratch of the split reductions: part of the workspace for launches of more than 128 rows.  Smaller grouped launches
+  // stream and need none; a single matrix of 33..128 rows runs the prefill kernel and is up to 1.5 times faster with it, so
+  // a caller may append it (a workspace of the queried size plus stmoe_mmt_workspace_bytes(rows)).
+  const size_t split_bytes = align_up(mfma_ws_partial_bytes(), 256);
+  const bool appended = E == 1 && rows > kSkinnyMaxRowsSingleSplit && workspace_bytes >= ws.split + split_bytes;
+  float* const split = ws.total > ws.split || appended ? reinterpret_cast<float*>(base + ws.split) : nullptr;
   const int32_t n_experts = offsets ? E : 1;
   const bool z_blocked = mfma8_in && mfma8_out &&
                          fp8_ws_takes(variant, weight_tag(w_gate), MODE_GATEUP, K, K, N, N, offsets != nullptr, n_experts, rows) &&

@@ -508,6 +508,8 @@ def grouped_ffn(x, w_gate: DeviceWeight, w_up: DeviceWeight, w_down: DeviceWeigh
     N, E = w_gate.rows, w_gate.experts
     need = grouped_ffn_workspace_bytes(T, k, K, N, x_c.dtype)
     if workspace is None:
+        if E == 1 and T * k <= 128:  # a single matrix of 33..128 rows: room for the split reductions of the prefill kernel
+            need += int(lib.stmoe_mmt_workspace_bytes(T * k))
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
     y = torch.empty((T * k, K), dtype=x_c.dtype, device=dev)
     xs, zs = _scale1(x_scale), _scale1(z_scale)
