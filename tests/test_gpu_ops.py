@@ -314,7 +314,7 @@ def test_quantized_matmul_descriptor_is_built_once_and_packed(device):
 
 
 @pytest.mark.parametrize("fmt", ["q8_0", "q4_1"])
-@pytest.mark.parametrize("M", [1, 32, 2048])
+@pytest.mark.parametrize("M", [1, 32, 33, 100, 2048])  # 33, 100: the prefill kernel with its reductions split (scratch appended to the workspace)
 def test_ffn_layer_llama_shape(device, fmt, M):
     """FFN (sharktank/sharktank/layers/ffn_block.py:21-51) at a Llama-8B shape, hidden 4096, FFN 14336, quantized weights:
     the gated form on the fused kernels against the closed form down(silu(gate x) * up x) of the oracle, row by row."""
@@ -334,7 +334,7 @@ def test_ffn_layer_llama_shape(device, fmt, M):
     ffn = FFN(ST.Theta(tensors))
     x = torch.randn(M, K, generator=torch.Generator().manual_seed(21)).to(torch.float16)
     got = ffn(x.reshape(1, M, K).to(device)).reshape(M, K).cpu()
-    rows = list(range(M)) if M <= 32 else [0, 1, 255, 256, 257, 1023, 1024, 2047]
+    rows = list(range(M)) if M <= 32 else [r for r in (0, 1, 31, 32, 63, 64, 99, 255, 256, 257, 1023, 1024, 2047) if r < M]
     xs = x[rows]
     dense = {n: MC.dense_from_planes(fmt, planes[n], [N, K] if n != "ffn_down" else [K, N], torch.float16) for n in planes}
     z = torch.nn.functional.silu(O._mm_rt(xs, dense["ffn_gate"])) * O._mm_rt(xs, dense["ffn_up"])
