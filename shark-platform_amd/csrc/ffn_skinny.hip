@@ -219,6 +219,37 @@ template <int WF> struct SkinnyX {
   }
 };
 
+// The experts' row ranges, fetched once per wavefront with two vector loads (lane l holds expert l's first and end
+// row) instead of a scalar load per expert and step of the search: walking the offsets with dependent scalar loads cost a
+// workgroup of a one-token launch about 2 us of its 13.  At most 64 experts (checked by the launcher).
+struct SkinnyExperts {
+  int begin, end;    // of expert `lane`
+  uint64_t active;   // experts that received rows
+  int n_active;
+  __device__ __forceinline__ void init(const GemmParams& p, int lane) {
+    begin = 0;
+    end = 0;
+    if (p.offsets) {
+      if (lane < p.E) {
+        begin = p.offsets[lane];
+        end = p.offsets[lane + 1];
+      }
+    } else if (lane == 0) {
+      end = (int)p.fixed_rows;
+    }
+    active = __ballot(end > begin);
+    n_active = __builtin_popcountll(active);
+  }
+  // the a-th expert with rows (a < n_active, the same for every lane of the wavefront)
+  __device__ __forceinline__ void find(int a, int& e, int& rb, int& re) const {
+    uint64_t m = active;
+    for (int i = 0; i < a; ++i) m &= m - 1;
+    e = __builtin_ctzll(m);
+    rb = __builtin_amdgcn_readlane(begin, e);
+    re = __builtin_amdgcn_readlane(end, e);
+  }
+};
+
 // One pass of one work item: rows [r0, min(r0 + 16*MT, re)) of expert rows against the item's two weight tiles.
 // KS > 1: the KS wavefronts of a workgroup share the item, each takes a contiguous 1/KS of the chunks, and the partial
 // sums are added through LDS in a fixed order ((w0 + w1) + (w2 + w3)) by wavefront 0, which then writes the result.
@@ -392,31 +423,14 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves, bool 
   const int64_t nch = p.kred >> 8;
 
   // experts that received rows, in increasing id
-  int n_active = 0;
-  uint64_t active_mask = 0;
-  for (int e = 0; e < p.E; ++e) {
-    int b, en;
-    expert_range(p, e, b, en);
-    if (en > b) {
-      active_mask |= 1ull << e;
-      ++n_active;
-    }
-  }
-  const int n_items = n_active * tiles_per_expert;
+  SkinnyExperts experts;
+  experts.init(p, lane);
+  const int n_items = experts.n_active * tiles_per_expert;
 
   for (int item = wave_global; item < n_items; item += total_waves) {
     const int a_idx = item / tiles_per_expert, tile = item - a_idx * tiles_per_expert;
-    int e = 0;
-    {
-      int seen = 0;
-      for (int ee = 0; ee < p.E; ++ee)
-        if ((active_mask >> ee) & 1ull) {
-          if (seen == a_idx) { e = ee; break; }
-          ++seen;
-        }
-    }
-    int rb, re;
-    expert_range(p, e, rb, re);
+    int e, rb, re;
+    experts.find(__builtin_amdgcn_readfirstlane(a_idx), e, rb, re);
 
     // the two weight tiles of this item
     int64_t wrow[2];
@@ -576,31 +590,14 @@ grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
   const int64_t nch = p.kred >> 8;
   const uint32_t xs_addr = __builtin_amdgcn_readfirstlane(
       (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)xs));
-  int n_active = 0;
-  uint64_t active_mask = 0;
-  for (int e = 0; e < p.E; ++e) {
-    int b, en;
-    expert_range(p, e, b, en);
-    if (en > b) {
-      active_mask |= 1ull << e;
-      ++n_active;
-    }
-  }
+  SkinnyExperts experts;
+  experts.init(p, lane);
   const int groups_per_expert = tiles_per_expert >> 2;
-  const int n_groups = n_active * groups_per_expert;
+  const int n_groups = experts.n_active * groups_per_expert;
   for (int grp = blockIdx.x; grp < n_groups; grp += gridDim.x) {
     const int a_idx = grp / groups_per_expert, tile = (grp - a_idx * groups_per_expert) * 4 + wave;
-    int e = 0;
-    {
-      int seen = 0;
-      for (int ee = 0; ee < p.E; ++ee)
-        if ((active_mask >> ee) & 1ull) {
-          if (seen == a_idx) { e = ee; break; }
-          ++seen;
-        }
-    }
-    int rb, re;
-    expert_range(p, e, rb, re);
+    int e, rb, re;
+    experts.find(a_idx, e, rb, re);
     int64_t wrow[2];
     if (MODE == MODE_GATEUP) {
       wrow[0] = (int64_t)e * p.w0.rows + tile * 16 + n_in;
