@@ -467,6 +467,25 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
   constexpr int XROWS = 16 * MT, XCHUNK = XROWS * 256, XSTAGE = G * XCHUNK;  // elements
   constexpr int XL = XROWS / 8;                                             // direct loads (2 rows each) per wavefront per chunk
   const int g = lane >> 4, n_in = lane & 15;
+  // The pass's first weight chunk is requested before anything else: the look-ups of the token rows' addresses (the
+  // dispatch permutation) and the token loads that depend on them then run while it is on its way from memory.
+  SkinnyW<WF> w0[G][NT], w1[G][NT];
+#pragma unroll
+  for (int q = 0; q < G; ++q) {
+    w0[q][0].init(p.w0, wrow[0]);
+    w1[q][0].init(p.w0, wrow[0]);
+    w0[q][1].init(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1]);
+    w1[q][1].init(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1]);
+  }
+  auto load_w = [&](SkinnyW<WF> (*w)[NT], int64_t c) {
+#pragma unroll
+    for (int q = 0; q < G; ++q) {
+      w[q][0].load(p.w0, wrow[0], c + q, g);
+      w[q][1].load(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1], c + q, g);
+    }
+  };
+  load_w(w0, 0);
+  __builtin_amdgcn_sched_barrier(0);  // (left alone the compiler sinks the requests below the look-ups to save registers)
   uint32_t xoff[XL];  // byte offsets from p.a (the host checks that the activations span less than 4 GB)
 #pragma unroll
   for (int j = 0; j < XL; ++j) {
@@ -488,21 +507,6 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[mt][t] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
-  SkinnyW<WF> w0[G][NT], w1[G][NT];
-#pragma unroll
-  for (int q = 0; q < G; ++q) {
-    w0[q][0].init(p.w0, wrow[0]);
-    w1[q][0].init(p.w0, wrow[0]);
-    w0[q][1].init(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1]);
-    w1[q][1].init(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1]);
-  }
-  auto load_w = [&](SkinnyW<WF> (*w)[NT], int64_t c) {
-#pragma unroll
-    for (int q = 0; q < G; ++q) {
-      w[q][0].load(p.w0, wrow[0], c + q, g);
-      w[q][1].load(MODE == MODE_GATEUP ? p.w1 : p.w0, wrow[1], c + q, g);
-    }
-  };
   auto compute = [&](const SkinnyW<WF> (*w)[NT], int stage) {
 #pragma unroll
     for (int q = 0; q < G; ++q) {
@@ -534,7 +538,6 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
     __syncthreads();
   };
   load_x(0, 0);
-  load_w(w0, 0);
   arrived(w0);
   for (int64_t c = 0; c < nch; c += 2 * G) {
     if (c + G < nch) {
