@@ -707,7 +707,13 @@ def mmt(a: torch.Tensor, w: DeviceWeight, *, variant: int = VARIANT_AUTO, worksp
         stream = _stream(dev)
         ready = workspace is None  # a caller's buffer has an unknown history
         if workspace is None:
-            workspace = _mmt_workspace(dev, stream, int(lib.stmoe_mmt_workspace_bytes(M)))
+            need = int(lib.stmoe_mmt_workspace_bytes(M))
+            if need and (dev, stream) not in _MMT_WORKSPACE and torch.cuda.is_current_stream_capturing():
+                # the kept buffer is zero-filled by a launch of its own, which must not become part of somebody's graph
+                # (it would run at replay time only): a buffer of this call's own, cleared by the library inside the graph
+                workspace, ready = torch.empty(need, dtype=torch.uint8, device=dev), False
+            else:
+                workspace = _mmt_workspace(dev, stream, need)
         _check(lib.stmoe_mmt(_ptr(a_c), dtype_enum(a_c.dtype), M, w.ref, _ptr(out), _ptr(workspace),
                              workspace.numel() if workspace is not None else 0, int(ready), variant, stream))
     return out

@@ -131,6 +131,43 @@ def test_quantized_linear_few_hundred_rows_splits_the_reduction(device, fmt, dty
     assert O.rel_l2(first.float().cpu(), plain.float().cpu()) < (5e-4 if dtype == torch.float16 else 4e-3)
 
 
+def test_quantized_linear_split_reduction_under_hip_graph_capture(device):
+    """A product of a few dozen rows cuts its reduction over several workgroups, which elect the adding one through counters
+    in the workspace.  Captured in a HIP graph (the capture brings its own buffer, cleared inside the graph by a kernel: no
+    memset node) every replay must give the eager result bit for bit, with eager products, which use the kept buffer,
+    between the replays."""
+    import moe_cases as MC
+    from sharktank_amd import _hip
+    from sharktank_amd.ops import device_weight
+
+    K, N, M = 2048, 1792, 64
+    case = MC.build(MC.Case(T=4, K=K, N=N, E=1, k=1, fmt="q8_0", dtype=torch.float16, seed=77))
+    it = MC.to_inference_tensor("q8_0", case.planes["gate"], [1, N, K], "w", device)
+    dw = device_weight(it, stacked=True, prepack=True)
+    g = torch.Generator().manual_seed(78)
+    inputs = [(torch.randn(M, K, generator=g) * 0.5).to(torch.float16).to(device) for _ in range(3)]
+    eager = [_hip.mmt(x, dw) for x in inputs]  # (also the warm-up that capture needs)
+    torch.cuda.synchronize()
+    static_in = torch.empty_like(inputs[0])
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        static_in.copy_(inputs[0])
+        with torch.cuda.graph(graph, stream=side):
+            static_out = _hip.mmt(static_in, dw)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(2):
+        for x, want in zip(inputs, eager):
+            static_in.copy_(x)
+            graph.replay()
+            got = static_out.clone()
+            torch.cuda.synchronize()
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+            again = _hip.mmt(x, dw)  # eager work between the replays
+            assert torch.equal(again.view(torch.int16), want.view(torch.int16))
+
+
 def test_layout_classes_dequant_on_device(device):
     from sharktank_amd import types as ST
 
