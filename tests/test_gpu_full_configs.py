@@ -2,7 +2,7 @@
 
 The CPU oracle cannot run these shapes in full in reasonable time, so each case checks
   * routing indices of every token against the oracle (bit-exact; the router is cheap on the CPU),
-  * the layer output of at least 64 tokens against the oracle (tokens are independent given their own routing, so the oracle
+  * the layer output of at least 256 tokens (every token of the decode sweep) against the oracle (tokens are independent given their own routing, so the oracle
     on a subset of rows is the full oracle restricted to those rows).  The tokens are chosen from the dispatch arrays, not
     at random: for every expert the first and the last row of every token tile of 256 sorted rows (every unit of the two
     prefill launches is a token tile times a feature tile, and a row spans all feature tiles, so every unit of both
@@ -262,7 +262,7 @@ def test_config2_prefill_with_split_reductions(device):
     units, so the last ones are cut along the reduction and summed by the reduce kernel; rows of every token tile."""
     theta, pc = build_device_case(device, 1900, 4096, 14336, "q8_0", torch.float16, seed=7)
     y, idx, gate, block = run_layer(theta, pc, device)
-    rows, tiles = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2)
+    rows, tiles = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2, at_least=256)
     check_against_oracle(y, idx, pc, rows)
     check_second_kernel_family(theta, pc, device, y, 1e-3)
 
@@ -271,7 +271,7 @@ def test_config2_prefill_with_split_reductions(device):
 def test_config3_mixtral_q4_1_bf16_decode_sweep(device, T):
     theta, pc = build_device_case(device, T, 4096, 14336, "q4_1", torch.bfloat16, seed=3)
     y, idx, gate, block = run_layer(theta, pc, device)
-    rows = list(range(T)) if T <= 64 else tokens_that_cover_every_unit(idx.cpu().long(), 8, 2)[0]
+    rows = list(range(T))  # every token
     check_against_oracle(y, idx, pc, rows)
     # the 128 x 128 tile kernel gives the same answer as the kernel the dispatcher picked
     check_second_kernel_family(theta, pc, device, y, BF16_TOL)
@@ -303,8 +303,8 @@ def test_config4_grok_q4_1_gelu_skewed_routing(device, dtype):
     top2 = counts.sort(descending=True).values[:2].sum().item() / counts.sum().item()
     print(f"  (token, slot) pairs per expert {counts.tolist()}: the two busiest experts take {top2:.3f}")
     assert 0.55 <= top2 <= 0.65, f"routing skew off the stated 60 %: {counts.tolist()}"
-    rows, tiles = tokens_that_cover_every_unit(idx.cpu().long(), E, 2)
-    assert len(rows) >= 64
+    rows, tiles = tokens_that_cover_every_unit(idx.cpu().long(), E, 2, at_least=256)
+    assert len(rows) >= 256
     check_against_oracle(y, idx, pc, rows)
     check_second_kernel_family(theta, pc, device, y, moe_tolerance(pc))
     x, idx_o, gate_o = oracle_route(pc)
@@ -328,15 +328,15 @@ def test_config5_mixtral_fp8_weights(device):
     gg = torch.rand(T, 2, generator=torch.Generator().manual_seed(50)) + 0.25
     gates = (gg / gg.sum(dim=1, keepdim=True)).to(torch.float16)
     assert torch.bincount(experts.reshape(-1), minlength=8).tolist() == [1024] * 8
-    rows, tiles = tokens_that_cover_every_unit(experts, 8, 2)
-    assert tiles == 32 and len(rows) >= 64
+    rows, tiles = tokens_that_cover_every_unit(experts, 8, 2, at_least=256)
+    assert tiles == 32 and len(rows) >= 256
     check_pre_gather_ffn_moe(theta, pc, device, x, experts, gates, rows, 2e-2)
     got1 = pre_gather_block(theta, pc)(x[:1].to(device), experts[:1].to(device), gates[:1].to(device)).cpu()
     want1 = torch.sum(gates[:1].unsqueeze(-1) * oracle_pair_outputs(pc, x, experts, [0]), dim=1)
     assert O.rel_l2(got1, want1) < 2e-2
     # the whole block
     y, idx, gate, block = run_layer(theta, pc, device)
-    rows, _ = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2)
+    rows, _ = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2, at_least=256)
     check_against_oracle(y, idx, pc, rows)
     check_second_kernel_family(theta, pc, device, y, 2e-2)
     y1, idx1, _ = block(pc["h"][:1].reshape(1, 1, 4096).to(device), return_routing=True)
@@ -357,7 +357,7 @@ def test_config5_mixtral_fp8_weights_and_activations(device):
     x = O.rms_norm_ordered(pc["h"], pc["ffn_norm"], 1e-5)
     experts = uniform_routing(T)
     gates = torch.full((T, 2), 0.5, dtype=torch.float16)
-    rows, _ = tokens_that_cover_every_unit(experts, 8, 2)
+    rows, _ = tokens_that_cover_every_unit(experts, 8, 2, at_least=256)
     tok = torch.tensor(rows, dtype=torch.long)
     want = torch.sum(gates[tok].unsqueeze(-1) * oracle_pair_outputs(pc, x, experts, rows), dim=1)
     outs = {}
@@ -372,7 +372,7 @@ def test_config5_mixtral_fp8_weights_and_activations(device):
     # the automatic choice for fp16 activations at this size is the matrix-core arithmetic
     assert torch.equal(outs[_hip.VARIANT_AUTO], outs[_hip.VARIANT_FP8_MFMA])
     y, idx, gate, block = run_layer(theta, pc, device, variant=_hip.VARIANT_STEP_BY_STEP)
-    rows, _ = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2)
+    rows, _ = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2, at_least=256)
     check_against_oracle(y, idx, pc, rows, 1e-3)  # the reference's arithmetic step by step: 16-bit tolerance
     y0, idx0, _, _ = run_layer(theta, pc, device)
     check_against_oracle(y0, idx0, pc, rows, 2e-2)  # the default: fp8 matrix cores
