@@ -152,6 +152,42 @@ dispatch_build_reg_kernel(const int32_t* __restrict__ idx, int n, int E, int32_t
   }
 }
 
+// The same result for at most 64 pairs and 64 experts (a decode step of 32 tokens with top-2 routing): one wavefront, lane i
+// owns pair i, no LDS and no barrier.  For every expert a ballot gives its count (kept by lane `expert`) and the rank of
+// each of its pairs; the scan over the experts runs on values read from the lanes.
+__global__ void __launch_bounds__(64)
+dispatch_build_wave_kernel(const int32_t* __restrict__ idx, int n, int E, int32_t* __restrict__ counts,
+                           int32_t* __restrict__ offsets, int32_t* __restrict__ perm, int32_t* __restrict__ inv,
+                           int32_t* __restrict__ zero_words, int n_zero) {
+  const int lane = threadIdx.x;
+  for (int i = lane; i < n_zero; i += 64) zero_words[i] = 0;
+  int e = lane < n ? idx[lane] : -1;
+  if (lane < n) e = e < 0 ? 0 : (e >= E ? E - 1 : e);  // out-of-range ids are a caller error; clamp to stay in bounds
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  int rank = 0, count = 0;  // of pair `lane` inside its expert; of expert `lane`
+  for (int ee = 0; ee < E; ++ee) {
+    const uint64_t mask = __ballot(e == ee);
+    if (e == ee) rank = __popcll(mask & lt_mask);
+    if (lane == ee) count = __popcll(mask);
+  }
+  int first = 0, run = 0;  // first row of expert `lane`
+  for (int ee = 0; ee < E; ++ee) {
+    if (lane == ee) first = run;
+    run += __builtin_amdgcn_readlane(count, ee);
+  }
+  if (lane < E) {
+    counts[lane] = count;
+    offsets[lane] = first;
+  }
+  if (lane == 0) offsets[E] = run;
+  const int first_of_mine = __shfl(first, e < 0 ? 0 : e, 64);
+  if (lane < n) {
+    const int pos = first_of_mine + rank;
+    perm[pos] = lane;
+    inv[lane] = pos;
+  }
+}
+
 // One workgroup per token; every thread owns 8 consecutive features (16-byte loads for 16-bit types).
 // o = sum over slots of round(gate * y) (fp32 sum in slot order, rounded to T); optional RMS norm of o;
 // optional residual add.
@@ -239,6 +275,10 @@ int dispatch_build(const int32_t* idx, int64_t n_pairs, int E, int32_t* counts, 
   STMOE_REQUIRE(counts && offsets, STMOE_ERR_NULL, "dispatch_build: counts/offsets NULL");
   STMOE_REQUIRE(n_pairs == 0 || (idx && perm && inv), STMOE_ERR_NULL, "dispatch_build: idx/perm/inv NULL");
   STMOE_REQUIRE(n_zero >= 0 && n_zero <= kDispatchThreads && (n_zero == 0 || zero_words), STMOE_ERR_SHAPE, "dispatch_build: %d words to clear", n_zero);
+  if (n_pairs <= 64 && E <= 64) {
+    dispatch_build_wave_kernel<<<1, 64, 0, st>>>(idx, (int)n_pairs, E, counts, offsets, perm, inv, zero_words, n_zero);
+    return check_launch("dispatch_build");
+  }
   if (n_pairs <= kDispatchRegChunks * kDispatchThreads && E <= kDispatchRegExperts) {
     const size_t lds = sizeof(int32_t) * (size_t)E * (kDispatchRegChunks * kDispatchWaves + 1);
     dispatch_build_reg_kernel<<<1, kDispatchThreads, lds, st>>>(idx, (int)n_pairs, E, counts, offsets, perm, inv, zero_words, n_zero);

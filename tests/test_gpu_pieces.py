@@ -209,7 +209,9 @@ def test_router_distinct_logits_with_equal_probabilities(device, K):
 @pytest.mark.parametrize("T,k,E", [(1, 2, 8), (32, 2, 8), (2048, 2, 8), (3000, 4, 64), (7, 1, 1),
                                    # either side of the limits of the kernel that keeps a launch's pairs in registers
                                    # (8192 pairs, 64 experts), partial last chunks, one pair per token
-                                   (4096, 2, 8), (4097, 2, 8), (1023, 3, 64), (600, 2, 65), (8192, 1, 16), (513, 2, 3)])
+                                   (4096, 2, 8), (4097, 2, 8), (1023, 3, 64), (600, 2, 65), (8192, 1, 16), (513, 2, 3),
+                                   # either side of the one-wavefront kernel's limits (64 pairs, 64 experts)
+                                   (32, 2, 64), (16, 4, 64), (33, 2, 8), (8, 8, 8), (21, 3, 5), (64, 1, 65)])
 def test_dispatch_bit_exact(device, T, k, E):
     g = torch.Generator().manual_seed(8)
     idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
