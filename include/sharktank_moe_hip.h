@@ -275,7 +275,8 @@ int stmoe_add_bias(const void* y, int y_dtype, const void* bias, int bias_dtype,
 
 /* softmax over the last axis of x [rows, cols] (`ops.softmax`, sharktank/sharktank/ops/signatures.py:974-993, default
  * implementation F.softmax, default_impls.py:426-432; MoeBlock applies it to the router logits with dtype=float,
- * mixture_of_experts_block.py:72-74): values widened to fp32, p = expf(x - max) / sum, rounded to out_dtype.  Rows of at
+ * mixture_of_experts_block.py:72-74): values widened to fp32, p = exp(x - max) / sum (results below the smallest normal
+ * fp32 number are kept, not flushed to zero), rounded to out_dtype.  Rows of at
  * most 64 elements are summed in index order, as the router kernel sums them: ranking these probabilities reproduces
  * stmoe_router_topk's choice bit for bit. */
 int stmoe_softmax(const void* x, int x_dtype, int64_t rows, int64_t cols, void* out, int out_dtype, stmoe_stream_t stream);
