@@ -1,15 +1,13 @@
 """BASELINE.json configurations 2-5 at their full shapes on the GPU.
 
-The CPU oracle cannot run these shapes in full in reasonable time, so each case checks
-  * routing indices of every token against the oracle (bit-exact; the router is cheap on the CPU),
-  * the layer output of at least 256 tokens (every token of the decode sweep) against the oracle (tokens are independent given their own routing, so the oracle
-    on a subset of rows is the full oracle restricted to those rows).  The tokens are chosen from the dispatch arrays, not
-    at random: for every expert the first and the last row of every token tile of 256 sorted rows (every unit of the two
-    prefill launches is a token tile times a feature tile, and a row spans all feature tiles, so every unit of both
-    launches, split along the reduction or not, has rows in the sample), rows of the expert's last, partial token tile,
-    and the rows that ride along with a full tile (1-16 rows above a multiple of 256).  The MoE contribution y - h is
-    held to the tolerance on its own (the residual h ~ N(0, 1) would hide an error of the FFN kernels): 1e-3 for fp16 and
-    for bf16, 2e-2 for fp8 weights or activations,
+The reference's own formulation (a gathered weight stack per token) cannot run these shapes on the CPU in reasonable time,
+but tokens are independent given their routing, so the oracle is evaluated expert by expert on the rows routed to each
+(one dense FFN per expert: seconds per configuration) and EVERY token of every configuration is compared:
+  * routing indices of every token against the oracle (bit-exact),
+  * the layer output of every token against the oracle.  The MoE contribution y - h is held to the tolerance on its own
+    (the residual h ~ N(0, 1) would hide an error of the FFN kernels): 1e-3 for fp16 and for bf16, 2e-2 for fp8 weights
+    or activations; the worst single token is held to a multiple of it (a wrong row or a wrong run of features in one row
+    cannot hide in the average over thousands of rows),
   * a second kernel family (the 128 x 128 tile kernel) on all rows,
   * size-independent properties on all tokens: token-permutation equivariance (routing bit-exact; outputs equal up to
     the fp32 summation grouping of the few rows whose down-projection tile is split along the reduction) and run-to-run
@@ -135,32 +133,10 @@ def oracle_rows(pc, rows, eps=1e-5):
     return pc["h"][tok] + o, idx, gate
 
 
-def tokens_that_cover_every_unit(idx, E, k, at_least=64, seed=0):
-    """Tokens chosen from the dispatch order (stable sort of the pairs by expert): per expert and per token tile of 256
-    sorted rows the first and last row; from the expert's last, partial tile also the middle row; every row (up to 3) of a
-    tail of 1..16*c rows above c full tiles, which rides along with the full tiles; then seeded random ones up to
-    `at_least`.  Returns (sorted token list, number of (expert, token tile) pairs covered)."""
-    counts, offsets, perm, _ = O.dispatch_permutation(idx, E)
-    picked, tiles = set(), 0
-    for e in range(E):
-        a, n = int(offsets[e]), int(counts[e])
-        rows = []
-        for t0 in range(0, n, 256):
-            t1 = min(t0 + 256, n)
-            rows += [t0, t1 - 1]
-            tiles += 1
-        c, tail = n // 256, n % 256
-        if tail:
-            rows += [c * 256 + tail // 2]
-            if c >= 1 and tail <= 16 * c:
-                rows += [c * 256 + i for i in range(min(tail, 3))]
-        for r in rows:
-            picked.add(int(perm[a + r]) // k)
-    g = torch.Generator().manual_seed(seed)
-    T = idx.shape[0]
-    while len(picked) < min(at_least, T):
-        picked.add(int(torch.randint(0, T, (1,), generator=g)))
-    return sorted(picked), tiles
+def token_tiles(idx, E):
+    """Number of (expert, token tile of 256 sorted rows) pairs of a routing: the units of a prefill launch per feature tile."""
+    counts = torch.bincount(idx.reshape(-1).long(), minlength=E)
+    return int(((counts + 255) // 256).sum())
 
 
 def run_layer(theta, pc, device, variant=0, h=None):
@@ -179,20 +155,38 @@ def moe_tolerance(pc):
     return BF16_TOL if pc["dtype"] == torch.bfloat16 else 1e-3
 
 
-def check_against_oracle(y, idx, pc, rows, tol=None):
-    """Routing of every token bit-exact; on `rows` the layer output within 1e-3 (the north-star figure for the layer) and
-    the MoE contribution y - h on its own within `tol`."""
+# The worst single token against the tolerance of the whole: rows differ in how much of their contribution cancels, so one
+# row's relative error scatters around the average; measured maxima are 1.3 to 2.2 times the average at these shapes.
+WORST_ROW_FACTOR = 4.0
+
+
+def row_rel_l2(got, want):
+    d = (got.double() - want.double()).norm(dim=-1)
+    return d / want.double().norm(dim=-1).clamp_min(1e-30)
+
+
+def check_against_oracle(y, idx, pc, rows=None, tol=None, want=None, worst_tol=None):
+    """Routing of every token bit-exact; on `rows` (default: every token) the layer output within 1e-3 (the north-star
+    figure for the layer), the MoE contribution y - h on its own within `tol`, and the MoE contribution of the worst
+    single token within `worst_tol` (default WORST_ROW_FACTOR * tol).  `want`: the result of oracle_rows(pc, rows) when
+    the caller has it."""
     tol = tol or moe_tolerance(pc)
-    want, want_idx, _ = oracle_rows(pc, rows)
+    worst_tol = worst_tol or WORST_ROW_FACTOR * tol
+    rows = list(range(pc["h"].shape[0])) if rows is None else rows
+    want, want_idx, _ = want if want is not None else oracle_rows(pc, rows)
     assert torch.equal(idx.cpu().long(), want_idx), "routing indices differ"
     got = y[rows].cpu()
     h = pc["h"][rows].float()
     err = O.rel_l2(got, want)
     moe = O.rel_l2(got.float() - h, want.float() - h)
-    print(f"  {len(rows)} rows: layer rel-L2 {err:.2e}, MoE contribution rel-L2 {moe:.2e} (limit {tol:.0e})")
+    per_row = row_rel_l2(got.float() - h, want.float() - h)
+    worst = float(per_row.max())
+    print(f"  {len(rows)} rows: layer rel-L2 {err:.2e}, MoE contribution rel-L2 {moe:.2e} (limit {tol:.0e}), "
+          f"worst token {worst:.2e} (row {rows[int(per_row.argmax())]})")
     assert torch.isfinite(got.float()).all()
     assert err < tol, f"layer output rel-L2 {err:.3e}"
     assert moe < tol, f"MoE contribution rel-L2 {moe:.3e}"
+    assert worst < worst_tol, f"MoE contribution of token {rows[int(per_row.argmax())]}: rel-L2 {worst:.3e}"
     return moe
 
 
@@ -218,9 +212,11 @@ def check_pre_gather_ffn_moe(theta, pc, device, x, idx, gate, tokens, tol):
     tok = torch.tensor(tokens, dtype=torch.long)
     want = torch.sum(gate[tok].unsqueeze(-1) * oracle_pair_outputs(pc, x, idx, tokens), dim=1)
     err = O.rel_l2(got[tok], want)
-    print(f"  PreGatherFFNMOE.forward, {len(tokens)} rows: rel-L2 {err:.2e} (limit {tol:.0e})")
+    worst = float(row_rel_l2(got[tok], want).max())
+    print(f"  PreGatherFFNMOE.forward, {len(tokens)} rows: rel-L2 {err:.2e} (limit {tol:.0e}), worst token {worst:.2e}")
     assert torch.isfinite(got.float()).all()
     assert err < tol, f"PreGatherFFNMOE output rel-L2 {err:.3e}"
+    assert worst < WORST_ROW_FACTOR * tol, f"PreGatherFFNMOE output, worst token: rel-L2 {worst:.3e}"
     return got
 
 
@@ -228,10 +224,9 @@ def test_config2_mixtral_q8_0_prefill_and_decode(device):
     """Mixtral-8x7B layer, Q8_0, fp16: prefill 2048 tokens and decode 32 tokens."""
     theta, pc = build_device_case(device, 2048, 4096, 14336, "q8_0", torch.float16, seed=0)
     y, idx, gate, block = run_layer(theta, pc, device)
-    rows, tiles = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2, at_least=256)
+    rows = list(range(2048))  # every token
     counts = torch.bincount(idx.cpu().reshape(-1).long(), minlength=8).tolist()
-    print(f"  rows per expert {counts}: {tiles} token tiles, {len(rows)} tokens checked")
-    assert len(rows) >= 256
+    print(f"  rows per expert {counts}: {token_tiles(idx.cpu(), 8)} token tiles")
     check_against_oracle(y, idx, pc, rows)
     check_second_kernel_family(theta, pc, device, y, 1e-3)
     # PreGatherFFNMOE on its own, with the router's choices
@@ -259,11 +254,10 @@ def test_config2_mixtral_q8_0_prefill_and_decode(device):
 
 def test_config2_prefill_with_split_reductions(device):
     """The same layer at 1900 tokens: the units of the two prefill launches no longer fill whole rounds over the compute
-    units, so the last ones are cut along the reduction and summed by the reduce kernel; rows of every token tile."""
+    units, so the last ones are cut along the reduction and their chunks added by the workgroup that finishes last."""
     theta, pc = build_device_case(device, 1900, 4096, 14336, "q8_0", torch.float16, seed=7)
     y, idx, gate, block = run_layer(theta, pc, device)
-    rows, tiles = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2, at_least=256)
-    check_against_oracle(y, idx, pc, rows)
+    check_against_oracle(y, idx, pc)  # every token
     check_second_kernel_family(theta, pc, device, y, 1e-3)
 
 
@@ -303,8 +297,7 @@ def test_config4_grok_q4_1_gelu_skewed_routing(device, dtype):
     top2 = counts.sort(descending=True).values[:2].sum().item() / counts.sum().item()
     print(f"  (token, slot) pairs per expert {counts.tolist()}: the two busiest experts take {top2:.3f}")
     assert 0.55 <= top2 <= 0.65, f"routing skew off the stated 60 %: {counts.tolist()}"
-    rows, tiles = tokens_that_cover_every_unit(idx.cpu().long(), E, 2, at_least=256)
-    assert len(rows) >= 256
+    rows = list(range(1024))  # every token
     check_against_oracle(y, idx, pc, rows)
     check_second_kernel_family(theta, pc, device, y, moe_tolerance(pc))
     x, idx_o, gate_o = oracle_route(pc)
@@ -328,15 +321,14 @@ def test_config5_mixtral_fp8_weights(device):
     gg = torch.rand(T, 2, generator=torch.Generator().manual_seed(50)) + 0.25
     gates = (gg / gg.sum(dim=1, keepdim=True)).to(torch.float16)
     assert torch.bincount(experts.reshape(-1), minlength=8).tolist() == [1024] * 8
-    rows, tiles = tokens_that_cover_every_unit(experts, 8, 2, at_least=256)
-    assert tiles == 32 and len(rows) >= 256
+    rows = list(range(T))  # every token
+    assert token_tiles(experts, 8) == 32
     check_pre_gather_ffn_moe(theta, pc, device, x, experts, gates, rows, 2e-2)
     got1 = pre_gather_block(theta, pc)(x[:1].to(device), experts[:1].to(device), gates[:1].to(device)).cpu()
     want1 = torch.sum(gates[:1].unsqueeze(-1) * oracle_pair_outputs(pc, x, experts, [0]), dim=1)
     assert O.rel_l2(got1, want1) < 2e-2
     # the whole block
     y, idx, gate, block = run_layer(theta, pc, device)
-    rows, _ = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2, at_least=256)
     check_against_oracle(y, idx, pc, rows)
     check_second_kernel_family(theta, pc, device, y, 2e-2)
     y1, idx1, _ = block(pc["h"][:1].reshape(1, 1, 4096).to(device), return_routing=True)
@@ -357,7 +349,7 @@ def test_config5_mixtral_fp8_weights_and_activations(device):
     x = O.rms_norm_ordered(pc["h"], pc["ffn_norm"], 1e-5)
     experts = uniform_routing(T)
     gates = torch.full((T, 2), 0.5, dtype=torch.float16)
-    rows, _ = tokens_that_cover_every_unit(experts, 8, 2, at_least=256)
+    rows = list(range(T))  # every token
     tok = torch.tensor(rows, dtype=torch.long)
     want = torch.sum(gates[tok].unsqueeze(-1) * oracle_pair_outputs(pc, x, experts, rows), dim=1)
     outs = {}
@@ -372,19 +364,22 @@ def test_config5_mixtral_fp8_weights_and_activations(device):
     # the automatic choice for fp16 activations at this size is the matrix-core arithmetic
     assert torch.equal(outs[_hip.VARIANT_AUTO], outs[_hip.VARIANT_FP8_MFMA])
     y, idx, gate, block = run_layer(theta, pc, device, variant=_hip.VARIANT_STEP_BY_STEP)
-    rows, _ = tokens_that_cover_every_unit(idx.cpu().long(), 8, 2, at_least=256)
-    check_against_oracle(y, idx, pc, rows, 1e-3)  # the reference's arithmetic step by step: 16-bit tolerance
+    want_all = oracle_rows(pc, rows)
+    # the reference's arithmetic step by step: 16-bit tolerance on the whole.  A single token is held to the fp8 tolerance:
+    # where the two sides' fp32 sums differ in the last bit, an element of the intermediate can land on the other side of
+    # an e4m3 rounding boundary, a step of 1/16 of that element, and a few such elements among a token's largest move
+    # that token by several 1e-3 (measured worst token 4.6e-3 at an average of 3.2e-4)
+    check_against_oracle(y, idx, pc, rows, 1e-3, want=want_all, worst_tol=2e-2)
     y0, idx0, _, _ = run_layer(theta, pc, device)
-    check_against_oracle(y0, idx0, pc, rows, 2e-2)  # the default: fp8 matrix cores
+    check_against_oracle(y0, idx0, pc, rows, 2e-2, want=want_all)  # the default: fp8 matrix cores
     y1, idx1, _ = block(pc["h"][:1].reshape(1, 1, 4096).to(device), return_routing=True)
     assert torch.equal(idx1.cpu(), idx.cpu()[:1])
-    want1, _, _ = oracle_rows(pc, [0])
-    assert O.rel_l2(y1.reshape(1, 4096).cpu(), want1) < 1e-3  # the decode path follows the reference's arithmetic
+    assert O.rel_l2(y1.reshape(1, 4096).cpu(), want_all[0][:1]) < 1e-3  # the decode path follows the reference's arithmetic
     # run-to-run bit identity
     y2, _, _, _ = run_layer(theta, pc, device, variant=_hip.VARIANT_STEP_BY_STEP)
     assert torch.equal(y2, y)
     # fp8 matrix cores
     y8, idx8, _, _ = run_layer(theta, pc, device, variant=_hip.VARIANT_FP8_MFMA)
-    check_against_oracle(y8, idx8, pc, rows, 2e-2)
+    check_against_oracle(y8, idx8, pc, rows, 2e-2, want=want_all)
     y8b, _, _, _ = run_layer(theta, pc, device, variant=_hip.VARIANT_FP8_MFMA)
     assert torch.equal(y8b, y8) and torch.equal(y0, y8)
