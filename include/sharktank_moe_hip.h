@@ -292,7 +292,10 @@ int stmoe_combine(const void* y_sorted, const void* gate, const int32_t* inv, in
 /* Whole MoeBlock.forward (mixture_of_experts_block.py:64-90) on h [T,K] -> out [T,K]:
  * ffn_norm -> router -> dispatch -> grouped FFN -> combine (+ layer_output_norm) + residual.
  * ffn_norm_w / out_norm_w are of w_dtype; out_norm_w may be NULL.  idx_out/gate_out ([T,k]) may be NULL.
- * x_scale / z_scale: activation quantizers of the expert FFN as in stmoe_grouped_ffn (NULL: none). */
+ * x_scale / z_scale: activation quantizers of the expert FFN as in stmoe_grouped_ffn (NULL: none).
+ * The stages are not always launches of their own: ffn_norm rides in the router launch when a token row fits its LDS
+ * row; the dispatch of a single token is written by the router launch and that of at most 64 (token, slot) pairs is
+ * built inside a streamed gate/up launch (the same stable counting sort as stmoe_dispatch_build, bit for bit). */
 int stmoe_moe_forward(const void* h, int dtype, int64_t T, int64_t K, int64_t N, int E, int k,
                       const void* ffn_norm_w, const void* out_norm_w, int w_dtype, float eps,
                       const void* w_router, const stmoe_weight* w_gate, const stmoe_weight* w_up,

@@ -101,6 +101,11 @@ static int run_fp8_projection(int variant, int dtype, int wtag, int mode, const 
 }
 
 static int run_projection(int variant, int dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
+  if (p.choices) {
+    // (only the streaming kernel builds its own dispatch; the caller has checked that it takes the launch)
+    const int rc = launch_skinny(dtype, wtag, mode, p, max_rows, st);
+    return rc != STMOE_ERR_UNSUPPORTED ? rc : set_error(STMOE_ERR_UNSUPPORTED, "grouped_ffn: no streaming kernel for a launch that builds its own dispatch");
+  }
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
     // (one matrix, with or without an offsets array around its rows)
@@ -172,7 +177,8 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
                             int act, const int32_t* offsets, const int32_t* perm, const float* x_scale,
                             const float* z_scale, void* y_sorted, void* workspace, size_t workspace_bytes, int variant,
                             stmoe_stream_t stream, void** events, bool tickets_zeroed = false, int stages = 3,
-                            void* z_io = nullptr, bool x_is_fake_quantized = false) {
+                            void* z_io = nullptr, bool x_is_fake_quantized = false, const int32_t* choices = nullptr,
+                            int32_t* dispatch_counts = nullptr, int32_t* dispatch_inv = nullptr) {
   STMOE_REQUIRE(T >= 0 && K > 0 && N > 0 && E >= 1 && k >= 1, STMOE_ERR_SHAPE, "grouped_ffn: T=%lld K=%lld N=%lld E=%d k=%d",
                 (long long)T, (long long)K, (long long)N, E, k);
   STMOE_REQUIRE(dtype == STMOE_F32 || dtype == STMOE_F16 || dtype == STMOE_BF16, STMOE_ERR_DTYPE,
@@ -240,6 +246,9 @@ static int grouped_ffn_impl(const void* x, int dtype, int64_t T, int64_t K, int6
     p.out = z; p.ldo = N; p.n_out = N; p.kred = K; p.act = act; p.x_scale = nullptr; p.expert_rows_bound = T;
     p.split_scratch = split;
     p.split_tickets_zeroed = tickets_zeroed;
+    if (choices) {  // `offsets` and `perm` are filled by the gate/up launch itself (see GemmParams::choices)
+      p.choices = choices; p.n_choices = (int32_t)rows; p.dispatch_counts = dispatch_counts; p.dispatch_inv = dispatch_inv;
+    }
     mark(events, 0, st);
     if (x_scale && !(x_is_fake_quantized && !mfma8_in)) {  // (the fused forward's norm launch may have done it already)
       // The 256 x 256 fp8 kernel streams its token rows in sorted order: the quantising pass writes them grouped by expert
@@ -455,17 +464,24 @@ static int moe_forward_impl(const void* h, int dtype, int64_t T, int64_t K, int6
   if (rc) return rc;
   mark(events, 3, st);
   mark(events, 4, st);
+  // A forward of at most 64 (token, slot) pairs that streams its weights has no dispatch launch either: every wavefront of
+  // the gate/up launch sorts the router's choices itself (a few ballots) and the first one leaves the arrays for the down
+  // and combine launches.
+  const bool gate_up_dispatches =
+      fused_front && T > 1 && T * k <= 64 && E >= 2 && (variant == 0 || variant == 3) && (dtype == STMOE_F16 || dtype == STMOE_BF16) &&
+      w_gate && w_up && weight_tag(w_gate) == weight_tag(w_up) && !(x_scale && !x_fq) &&
+      skinny_takes_grouped(dtype, weight_tag(w_gate), E, K, N, K, N);
   // the dispatch launch also clears the ticket words of the projections' split reductions (if this shape has any)
   const FfnWs fws = carve_ffn(T, k, K, N, dtype);
   const bool has_tickets = fws.total > fws.split && !router_dispatches;
   int32_t* tickets = has_tickets ? reinterpret_cast<int32_t*>(base + ws.ffn + fws.split + mfma_ws_tickets_offset()) : nullptr;
-  if (!router_dispatches &&
+  if (!router_dispatches && !gate_up_dispatches &&
       (rc = dispatch_build(idx, T * k, E, counts, offsets, perm, inv, tickets, has_tickets ? mfma_ws_ticket_count() : 0, st)))
     return rc;
   mark(events, 5, st);
   if ((rc = grouped_ffn_impl(xn, dtype, T, K, N, E, k, w_gate, w_up, w_down, act, offsets, perm, x_scale, z_scale, y,
                              base + ws.ffn, workspace_bytes - ws.ffn, variant, stream, events ? events + 6 : nullptr, has_tickets, 3,
-                             nullptr, x_fq != nullptr)))
+                             nullptr, x_fq != nullptr, gate_up_dispatches ? idx : nullptr, counts, inv)))
     return rc;
   mark(events, 10, st);
   rc = stmoe_combine(y, gate, inv, dtype, T, k, K, out_norm_w, w_dtype, eps, h, out, stream);

@@ -37,6 +37,13 @@ struct GemmParams {
   int64_t expert_rows_bound;  // host-side bound of rows per expert (a token gives an expert at most one row)
   float* split_scratch;       // optional fp32 scratch for split reductions (mfma_ws_partial_bytes() bytes)
   bool split_tickets_zeroed;  // the caller vouches that the scratch's ticket words (mfma_ws_tickets_offset()) are zero
+  // Streaming GATEUP launches of at most 64 (token, slot) pairs only: the router's expert choice per pair.  When set, every
+  // wavefront builds the dispatch itself from these (counting sort by expert, stable in the pair id) and reads neither
+  // `offsets` nor `perm`; the first wavefront of the grid also writes the four dispatch arrays (`offsets` and `perm` at the
+  // addresses above, counts and inv at the ones below) for the launches that follow, so the forward needs no dispatch launch.
+  const int32_t* choices;
+  int32_t n_choices;
+  int32_t *dispatch_counts, *dispatch_inv;
 };
 
 // Row range of expert e; without offsets there is one expert with `fixed_rows` rows.
@@ -160,6 +167,7 @@ size_t mfma_ws_partial_bytes();
 size_t mfma_ws_tickets_offset();  // byte offset of the split units' ticket words inside that scratch
 int mfma_ws_ticket_count();
 int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
+bool skinny_takes_grouped(int act_dtype, int wtag, int E, int64_t kred, int64_t n_out, int64_t lda, int64_t ldo);
 int launch_fp8_tile(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 int launch_fp8_ws(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st);
 }  // namespace stmoe

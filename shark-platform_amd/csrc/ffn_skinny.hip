@@ -222,14 +222,56 @@ template <int WF> struct SkinnyX {
 // The experts' row ranges, fetched once per wavefront with two vector loads (lane l holds expert l's first and end
 // row) instead of a scalar load per expert and step of the search: walking the offsets with dependent scalar loads cost a
 // workgroup of a one-token launch about 2 us of its 13.  At most 64 experts (checked by the launcher).
+// With p.choices (GATEUP launches of at most 64 pairs) the wavefront builds the dispatch from the router's choices instead:
+// lane i owns pair i; per expert that occurs a ballot gives its count (kept by lane `expert`) and the rank of each of its
+// pairs, a scan over the lanes gives the experts' first rows, and a lane-to-lane scatter leaves the pair id of sorted
+// position l in lane l.  The result is the stable counting sort the dispatch launch computes.
 struct SkinnyExperts {
   int begin, end;    // of expert `lane`
   uint64_t active;   // experts that received rows
   int n_active;
-  __device__ __forceinline__ void init(const GemmParams& p, int lane) {
+  int pair_at_lane;  // with p.choices: the pair at sorted position `lane`
+  template <int MODE> __device__ __forceinline__ void init(const GemmParams& p, int lane, bool write_out) {
     begin = 0;
     end = 0;
-    if (p.offsets) {
+    pair_at_lane = 0;
+    if (MODE == MODE_GATEUP && p.choices) {
+      const int n = p.n_choices;
+      int e = -1;
+      if (lane < n) {
+        e = p.choices[lane];
+        e = e < 0 ? 0 : (e >= p.E ? p.E - 1 : e);  // (out-of-range ids are a caller error; clamped to stay in bounds)
+      }
+      int rank = 0, count = 0;  // of pair `lane` inside its expert; of expert `lane`
+      uint64_t todo = __ballot(lane < n);
+      while (todo) {
+        const int ee = __builtin_amdgcn_readlane(e, (int)__builtin_ctzll(todo));
+        const uint64_t m = __ballot(e == ee);
+        if (e == ee) rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        if (lane == ee) count = __builtin_popcountll(m);
+        todo &= ~m;
+      }
+      int run = 0;
+      for (int ee = 0; ee < p.E; ++ee) {
+        if (lane == ee) begin = run;
+        run += __builtin_amdgcn_readlane(count, ee);
+      }
+      end = begin + count;
+      const int first_of_mine = __builtin_amdgcn_ds_bpermute((e < 0 ? 0 : e) << 2, begin);
+      const int pos = lane < n ? first_of_mine + rank : lane;  // (lanes without a pair send to themselves)
+      pair_at_lane = __builtin_amdgcn_ds_permute(pos << 2, lane);
+      if (write_out) {
+        if (lane < p.E) {
+          p.dispatch_counts[lane] = count;
+          const_cast<int32_t*>(p.offsets)[lane] = begin;
+        }
+        if (lane == 0) const_cast<int32_t*>(p.offsets)[p.E] = n;
+        if (lane < n) {
+          const_cast<int32_t*>(p.perm)[lane] = pair_at_lane;
+          p.dispatch_inv[lane] = pos;
+        }
+      }
+    } else if (p.offsets) {
       if (lane < p.E) {
         begin = p.offsets[lane];
         end = p.offsets[lane + 1];
@@ -248,14 +290,19 @@ struct SkinnyExperts {
     rb = __builtin_amdgcn_readlane(begin, e);
     re = __builtin_amdgcn_readlane(end, e);
   }
+  // Source row of sorted position i (every lane of the wavefront calls this together).
+  template <int MODE> __device__ __forceinline__ int64_t source_row(const GemmParams& p, int i) const {
+    if (MODE == MODE_GATEUP && p.choices) return (int64_t)(__builtin_amdgcn_ds_bpermute(i << 2, pair_at_lane) / p.k_top);
+    return p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
+  }
 };
 
 // One pass of one work item: rows [r0, min(r0 + 16*MT, re)) of expert rows against the item's two weight tiles.
 // KS > 1: the KS wavefronts of a workgroup share the item, each takes a contiguous 1/KS of the chunks, and the partial
 // sums are added through LDS in a fixed order ((w0 + w1) + (w2 + w3)) by wavefront 0, which then writes the result.
 template <typename T, int WF, int MODE, int MT, int KS>
-__device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (&wrow)[2], int tile, int r0, int re,
-                                            int64_t nch_total, int lane, bool pin_prefetch) {
+__device__ __forceinline__ void skinny_pass(const GemmParams& p, const SkinnyExperts& experts, const int64_t (&wrow)[2], int tile,
+                                            int r0, int re, int64_t nch_total, int lane, bool pin_prefetch) {
   constexpr int NT = 2;
   const int kw = KS > 1 ? (int)(threadIdx.x >> 6) : 0;
   const int64_t c_begin = KS > 1 ? nch_total * kw / KS : 0;
@@ -271,8 +318,7 @@ __device__ __forceinline__ void skinny_pass(const GemmParams& p, const int64_t (
     int i = r0 + mt * 16 + n_in;
     xok[mt] = MT == 1 || i < re;
     i = min(i, re - 1);
-    const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
-    xrow[mt] = reinterpret_cast<const uint16_t*>(p.a) + src * p.lda;
+    xrow[mt] = reinterpret_cast<const uint16_t*>(p.a) + experts.template source_row<MODE>(p, i) * p.lda;
   }
   floatx4_t acc[MT][NT];
 #pragma unroll
@@ -424,7 +470,7 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves, bool 
 
   // experts that received rows, in increasing id
   SkinnyExperts experts;
-  experts.init(p, lane);
+  experts.template init<MODE>(p, lane, blockIdx.x == 0 && threadIdx.x < 64);
   const int n_items = experts.n_active * tiles_per_expert;
 
   for (int item = wave_global; item < n_items; item += total_waves) {
@@ -443,9 +489,9 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves, bool 
     }
     // up to 16 rows: one 16-row token tile; otherwise passes of two tiles (one pass up to 32 rows)
     if (re - rb <= 16) {
-      skinny_pass<T, WF, MODE, 1, KS>(p, wrow, tile, rb, re, nch, lane, pin_prefetch);
+      skinny_pass<T, WF, MODE, 1, KS>(p, experts, wrow, tile, rb, re, nch, lane, pin_prefetch);
     } else {
-      for (int r0 = rb; r0 < re; r0 += 32) skinny_pass<T, WF, MODE, 2, KS>(p, wrow, tile, r0, re, nch, lane, false);
+      for (int r0 = rb; r0 < re; r0 += 32) skinny_pass<T, WF, MODE, 2, KS>(p, experts, wrow, tile, r0, re, nch, lane, false);
     }
   }
 }
@@ -459,8 +505,8 @@ grouped_skinny_kernel(GemmParams p, int tiles_per_expert, int total_waves, bool 
 // the 16-byte unit u of row r lives at unit u ^ (r & 15), which makes the operand reads of 16 rows conflict-free and
 // is applied on the source side of the direct loads.  Weights are handled as above (registers, one chunk ahead).
 template <typename T, int WF, int MODE, int MT, int G>
-__device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64_t (&wrow)[2], int tile, int r0, int re,
-                                                int64_t nch, int lane, int wave, uint16_t* xs, uint32_t xs_addr) {
+__device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const SkinnyExperts& experts, const int64_t (&wrow)[2], int tile,
+                                                int r0, int re, int64_t nch, int lane, int wave, uint16_t* xs, uint32_t xs_addr) {
   // G chunks of 256 reduction elements form one pipeline step (G = 2 for the 4-bit format, whose chunks are half
   // as many bytes, so that as many bytes are in flight per wavefront as for the 8-bit formats)
   constexpr int NT = 2;
@@ -491,7 +537,7 @@ __device__ __forceinline__ void skinny_lds_pass(const GemmParams& p, const int64
   for (int j = 0; j < XL; ++j) {
     const int lr = 2 * (wave * XL + j) + (lane >> 5);  // LDS row; rows past the end re-read the last row (never stored)
     const int i = min(r0 + lr, re - 1);
-    const int64_t src = p.perm ? (int64_t)(p.perm[i] / p.k_top) : (int64_t)i;
+    const int64_t src = experts.template source_row<MODE>(p, i);
     xoff[j] = (uint32_t)((src * p.lda + (((lane & 31) ^ (lr & 15)) << 3)) * 2);
   }
   auto load_x = [&](int stage, int64_t c) {  // chunks c .. c + G - 1
@@ -594,7 +640,7 @@ grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
   const uint32_t xs_addr = __builtin_amdgcn_readfirstlane(
       (uint32_t)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint16_t*)xs));
   SkinnyExperts experts;
-  experts.init(p, lane);
+  experts.template init<MODE>(p, lane, blockIdx.x == 0 && wave == 0);
   const int groups_per_expert = tiles_per_expert >> 2;
   const int n_groups = experts.n_active * groups_per_expert;
   for (int grp = blockIdx.x; grp < n_groups; grp += gridDim.x) {
@@ -614,9 +660,9 @@ grouped_skinny_lds_kernel(GemmParams p, int tiles_per_expert) {
     // kernel has plenty to spare (the matrix cores are busy in 0.07 of the cycles with one or two tiles).
     for (int r0 = rb; r0 < re; r0 += 16 * MAXMT) {
       const int left = re - r0;
-      if (left <= 16) skinny_lds_pass<T, WF, MODE, 1, G>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
-      else if (MAXMT == 2 || left <= 32) skinny_lds_pass<T, WF, MODE, 2, G>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
-      else skinny_lds_pass<T, WF, MODE, MAXMT, G>(p, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
+      if (left <= 16) skinny_lds_pass<T, WF, MODE, 1, G>(p, experts, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
+      else if (MAXMT == 2 || left <= 32) skinny_lds_pass<T, WF, MODE, 2, G>(p, experts, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
+      else skinny_lds_pass<T, WF, MODE, MAXMT, G>(p, experts, wrow, tile, r0, re, nch, lane, wave, xs, xs_addr);
     }
   }
 }
@@ -673,11 +719,26 @@ static int launch_skinny_t(int mode, const GemmParams& p, int64_t max_rows, hipS
   return check_launch("grouped_skinny");
 }
 
+// Whether launch_skinny has a kernel for a grouped launch of this shape (the tests it applies itself).
+bool skinny_takes_grouped(int act_dtype, int wtag, int E, int64_t kred, int64_t n_out, int64_t lda, int64_t ldo) {
+  if (E > 64 || kred % 256 != 0 || n_out % 32 != 0 || lda % 8 != 0 || ldo % 4 != 0) return false;
+  switch (wtag) {
+    case WF_Q8_0: case WF_Q4_1: case WF_FP8_F32D: case WF_Q8_0_P: case WF_Q4_1_P: case WF_FP8_F32D_P:
+      return act_dtype == STMOE_F16 || act_dtype == STMOE_BF16;
+    case WF_DENSE_F16: return act_dtype == STMOE_F16;
+    case WF_DENSE_BF16: return act_dtype == STMOE_BF16;
+    default: return false;
+  }
+}
+
 int launch_skinny(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
   if ((!p.offsets && p.E != 1) || p.E > 64 || (!p.offsets && p.fixed_rows >= ((int64_t)1 << 31)))
     return set_error(STMOE_ERR_UNSUPPORTED, "skinny kernel: needs per-expert offsets (or a single matrix) and at most 64 experts");
   if (p.kred % 256 != 0 || p.n_out % 32 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0)
     return set_error(STMOE_ERR_UNSUPPORTED, "skinny kernel: needs K %% 256 == 0 and N %% 32 == 0");
+  if (p.choices && (mode != MODE_GATEUP || p.n_choices < 1 || p.n_choices > 64 || p.n_choices != max_rows || !p.offsets || !p.perm ||
+                    !p.dispatch_counts || !p.dispatch_inv))
+    return set_error(STMOE_ERR_SHAPE, "skinny kernel: a dispatch inside the launch takes 1..64 pairs of a gate/up launch and four arrays to fill");
   if (max_rows == 0) return STMOE_OK;
     if (act_dtype == STMOE_F16) {
     switch (wtag) {
