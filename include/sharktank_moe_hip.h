@@ -347,7 +347,8 @@ int stmoe_probe_mfma(int kind, int random_operands, int iters, float* sink, doub
  * a [M,K], out [M,rows], both `dtype`; fp32 accumulation.
  * `workspace` (nullable; stmoe_mmt_workspace_bytes(M) bytes, 16-byte aligned): scratch for reductions split over several
  * workgroups, which lets a launch of a few hundred rows (too few 256 x 256 units for 256 CUs) use the whole chip; without
- * it the result is the same up to the grouping of the fp32 sums, the launch only slower.  The workspace ends in a few
+ * it the result is the same up to the grouping of the fp32 sums, the launch only slower.  (Launches of 129 rows and more
+ * whose tiles of 64 output features x 256 rows fit the 256 CUs run on such tiles instead and use no workspace.)  The workspace ends in a few
  * counters that elect the workgroup which adds a split unit's chunks; every call leaves them at zero.
  * `workspace_ready` != 0: the caller vouches that the workspace was zero-filled before its first use and has since been
  * written only by calls of this function (on one stream at a time); 0: the counters are cleared first, one small launch

@@ -48,6 +48,7 @@ static int check_weight(const stmoe_weight* w, const char* who, int64_t E, int64
 //          6 MFMA 256x256 tile with specialised producer/consumer wavefronts (prefill; packed formats),
 //          7 fp8 matrix cores, 128x128 tile kernel only (5 uses the 256x256 LDS-direct kernel where it applies),
 //          8 auto among the kernels that follow the reference's arithmetic step by step (never the fp8 matrix cores)
+//          9 MFMA 64 x 256 tile, the narrow form of 4 (a single matrix with a few hundred rows; packed formats)
 // Automatic choice with fp8 weights and static quantizers on both activations: a prefill-sized launch with fp16
 // activations goes to the fp8 matrix cores (variant 5: both operands as bytes, the fp32 dot product scaled once; 1.8 times
 // faster than dequantise-then-multiply, and 6e-3 from it on the layer output at the Mixtral shape, inside the 2e-2 the fp8
@@ -86,6 +87,20 @@ static inline int64_t skinny_max_avg_rows(int E) { return E <= 4 ? 28 : 16; }
 // (Q4_1: 33 / 43 / 60 / 79): it then wins from 33 rows on.
 static constexpr int64_t kSkinnyMaxRowsSingle = 48;
 static constexpr int64_t kSkinnyMaxRowsSingleSplit = 32;
+// A single matrix with 129 rows or more and few output features: tiles of 64 output features x 256 rows (the narrow form of
+// the 256 x 256 kernel, variant 9) fill the CUs where 256 x 256 units cannot, without cutting the reduction.  It pays while
+// its tiles fit one round over the 256 CUs and, against the split reduction, while the reduction is short: a narrow tile
+// takes 0.6 us per K step of 64, a quarter of a split unit's reduction 0.25 us per step of the whole plus 40-45 us for the
+// fp32 partial tiles and their sum.  Measured ([out, in] Q8_0 fp16, narrow / split, us): [14336, 4096] 192 rows 42 / 58,
+// 256 rows 45 / 64 (0.67 PFLOP/s), 384 rows 81 / 73; [4096, 4096] 192 ... 1024 rows 33 ... 47 / 42 ... 67; [8192, 8192] 256
+// rows 75 / 69; [4096, 14336] 256 rows 123 / 86.  Without scratch the 256 x 256 kernel takes 1.15 us per step unsplit.
+static bool narrow_pays(int mode, const GemmParams& p, int64_t rows) {
+  if (rows <= 128) return false;
+  const int64_t features = mode == MODE_GATEUP ? 32 : 64;
+  if (p.n_out % features != 0) return false;
+  if (p.n_out / features * ((rows + 255) / 256) > 256) return false;
+  return p.split_scratch == nullptr || p.kred <= 6144;
+}
 // fp8 activations x fp8 weights on the fp8 matrix cores: the 256 x 256 kernel for packed weights and launches with
 // enough rows to fill its tiles (variant 5), the 128 x 128 kernel otherwise (and always with variant 7).
 // Whether the 256 x 256 kernel takes a projection (its token rows must come without a gather: see fp8_ws_takes' caller).
@@ -109,11 +124,17 @@ static int run_projection(int variant, int dtype, int wtag, int mode, const Gemm
   if (variant == 0) {
     if (dtype == STMOE_F32) variant = 1;
     // (one matrix, with or without an offsets array around its rows)
-    else if (p.E == 1) variant = max_rows <= (p.split_scratch ? kSkinnyMaxRowsSingleSplit : kSkinnyMaxRowsSingle) ? 3 : 6;
+    else if (p.E == 1) variant = max_rows <= (p.split_scratch ? kSkinnyMaxRowsSingleSplit : kSkinnyMaxRowsSingle) ? 3
+                                 : narrow_pays(mode, p, max_rows) ? 9 : 6;
     else if (p.offsets && ((p.expert_rows_bound > 0 && p.expert_rows_bound <= kSkinnyMaxRowsPerExpert) ||
                            max_rows <= kSkinnyMaxRows || max_rows <= skinny_max_avg_rows(p.E) * p.E)) variant = 3;
     // Everything else goes to the 256 x 256 kernel (which hands shapes it does not take down to the 128 x 128 one).
     else variant = 6;
+  }
+  if (variant == 9) {
+    int rc = launch_mfma_narrow(dtype, wtag, mode, p, max_rows, st);
+    if (rc != STMOE_ERR_UNSUPPORTED) return rc;
+    variant = 6;
   }
   if (variant == 6) {
     int rc = launch_mfma_ws(dtype, wtag, mode, p, max_rows, p.split_scratch, st);

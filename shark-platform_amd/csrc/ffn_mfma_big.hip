@@ -32,18 +32,28 @@ struct BigTagOff { static constexpr bool value = false; };
 // WN x WM wavefronts; each owns 128 weight rows x 64 token rows (32 accumulator tiles = 128 registers, which
 // leaves the register allocator room: a 128 x 128 wavefront tile fills all 256 accumulation registers and made
 // the compiler shuffle accumulators between register files around every MFMA).
-template <typename T, int WF, int MODE, int WN, int WM, int STAGES>
+//
+// TI: 16-row weight fragments per wavefront (8: the 128 x 64 wavefront tile above).  The narrow form (TI = 2, 2 x 4
+// wavefronts: 64 weight rows x 256 token rows per workgroup, 32 x 64 per wavefront) is for a single matrix with a few
+// hundred rows: 256 rows of a [14336, 4096] matrix are 56 tiles of 256 x 256 but 224 of 64 x 256, which fill the CUs
+// without cutting the reduction (no fp32 partial tiles, no workspace).  A K step then has only four weight pieces: the
+// first four wavefronts load and convert one each, the others only send token rows.
+template <typename T, int WF, int MODE, int WN, int WM, int STAGES, int TI>
 __global__ void __launch_bounds__(64 * WN * WM, 1)
 grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
   constexpr int NTHR = 64 * WN * WM;
-  constexpr int BN = 128 * WN;           // weight rows per workgroup tile (GATEUP: BN/2 gate + BN/2 up)
+  constexpr int WROWS = 16 * TI;         // weight rows per wavefront (GATEUP: half gate, half up)
+  constexpr int BN = WROWS * WN;         // weight rows per workgroup tile (GATEUP: BN/2 gate + BN/2 up)
   constexpr int BM = 64 * WM;            // token rows per workgroup tile
   static_assert(STAGES == 2, "two weight stages and three token stages");
+  static_assert(TI % 2 == 0, "gate and up fragments come in pairs");
   constexpr int WSTAGE = BN * BIG_LS, XSTAGE = BM * BIG_LS;  // elements
-  constexpr int WPIECES = (BN / 16) / (WN * WM);  // packed weight pieces per wavefront per K step
+  constexpr int NPIECES = BN / 16;                                      // packed weight pieces per K step
+  constexpr int WPIECES = NPIECES >= WN * WM ? NPIECES / (WN * WM) : 1;  // per wavefront that loads weights
+  constexpr int WLOADERS = NPIECES / WPIECES;                           // wavefronts 0 .. WLOADERS - 1 load weights
   constexpr int XPIECES = BM * 8 / NTHR;          // 16-byte token pieces per thread per K step
   constexpr int XROWS_PER_PASS = NTHR / 8;
-  static_assert(WPIECES >= 1 && XPIECES >= 1, "tile too small for the thread count");
+  static_assert(WPIECES >= 1 && XPIECES >= 1 && WPIECES * WLOADERS == NPIECES && WLOADERS <= WN * WM, "tile too small for the thread count");
   extern __shared__ __align__(16) uint16_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wn = wave / WM, wm = wave % WM;
@@ -58,7 +68,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
   BigAddr<WF> waddr[WPIECES];
 #pragma unroll
   for (int j = 0; j < WPIECES; ++j) {
-    const int rtl = wave * WPIECES + j;  // row tile (16 rows) inside the workgroup tile
+    const int rtl = (wave < WLOADERS ? wave : 0) * WPIECES + j;  // row tile (16 rows) inside the workgroup tile
     int64_t row0;                         // first global row of the row tile (expert-stacked)
     const WeightView* wv;
     if (MODE == MODE_GATEUP) {
@@ -102,7 +112,7 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) {
     const int u = ((ks * 4 + g) ^ sw) << 3;
-    a_rd[ks] = Wbase + ((MODE == MODE_GATEUP ? wn * 64 : wn * 128) + n_in) * BIG_LS + u;
+    a_rd[ks] = Wbase + ((MODE == MODE_GATEUP ? wn * (WROWS / 2) : wn * WROWS) + n_in) * BIG_LS + u;
     b_rd[ks] = Xbase + (wm * 64 + n_in) * BIG_LS + u;
   }
 
@@ -137,9 +147,9 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
   // ---- consumer -----------------------------------------------------------------------------------------
   // wavefront tile: GATEUP gate rows wn*64..+63 (LDS rows wn*64..) and the same up rows (LDS rows BN/2 + wn*64..);
   //                 DOWN rows wn*128..+127.  Token rows wm*64..+63.
-  floatx4_t acc[8][4];
+  floatx4_t acc[TI][4];
 #pragma unroll
-  for (int a = 0; a < 8; ++a)
+  for (int a = 0; a < TI; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[a][b] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
   const bool active = rows_here > wm * 64;  // wavefronts whose token rows are all past the end skip their MFMAs
@@ -151,8 +161,8 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) bf[tj] = *reinterpret_cast<const u32x4_t*>(bp + tj * 16 * BIG_LS);
 #pragma unroll
-    for (int ti = 0; ti < 8; ++ti) {
-      const int row_off = MODE == MODE_GATEUP ? (ti < 4 ? 0 : BN / 2) + (ti & 3) * 16 : ti * 16;
+    for (int ti = 0; ti < TI; ++ti) {
+      const int row_off = MODE == MODE_GATEUP ? (ti < TI / 2 ? 0 : BN / 2) + (ti % (TI / 2)) * 16 : ti * 16;
       const u32x4_t af = *reinterpret_cast<const u32x4_t*>(a_rd[ks] + PAR * WSTAGE + row_off * BIG_LS);
 #pragma unroll
       for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = mfma16b<T>(af, bf[tj], acc[ti][tj]);
@@ -168,64 +178,70 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
   // one straight-line block; LATE wavefronts produce before their MFMAs, the others after.
   // STEADY steps (kt + 3 < nkt) contain no branch, so two of them form one basic block and the compiler's waits for
   // the weight registers stay exact; the last steps run the same code with the loads guarded.
-  auto k_step = [&](auto active_tag, auto late_tag, auto parity_tag, auto steady_tag, int64_t kt, int xs) {
+  auto k_step = [&](auto active_tag, auto late_tag, auto wload_tag, auto parity_tag, auto steady_tag, int64_t kt, int xs) {
     constexpr bool ACTIVE = decltype(active_tag)::value;
     constexpr bool LATE = decltype(late_tag)::value;
+    constexpr bool WLOAD = decltype(wload_tag)::value;  // this wavefront is one of those that load weight pieces
     constexpr int PAR = decltype(parity_tag)::value;  // kt % 2
     constexpr bool STEADY = decltype(steady_tag)::value;
     using Next = BigSet<PAR ^ 1>;
     auto produce = [&]() {
       // the compiler's wait for the registers of step kt + 1 also covers the older token loads of that step
-      if (STEADY || kt + 1 < nkt) store_w(Next{});
+      if (WLOAD && (STEADY || kt + 1 < nkt)) store_w(Next{});
       if (STEADY || kt + 2 < nkt) load_x(xs >= 1 ? xs - 1 : 2, kt + 2);
-      if (STEADY || kt + 3 < nkt) load_w(Next{}, kt + 3);
+      if (WLOAD && (STEADY || kt + 3 < nkt)) load_w(Next{}, kt + 3);
     };
     // scheduling fences: without them the compiler hoists the LDS reads of both K halves and the next step's
     // conversions across the whole block and runs out of registers
+    // (the narrow form has registers to spare: there the compiler may read the second K half's operands under the first
+    // half's MFMAs)
+    constexpr bool FENCED = TI >= 8;
     if constexpr (LATE) {
       produce();
-      __builtin_amdgcn_sched_barrier(0);
+      if (FENCED) __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (ACTIVE) {
       compute(parity_tag, xs, 0);
-      __builtin_amdgcn_sched_barrier(0);
+      if (FENCED) __builtin_amdgcn_sched_barrier(0);
       compute(parity_tag, xs, 1);
-      __builtin_amdgcn_sched_barrier(0);
+      if (FENCED) __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (!LATE) {
       produce();
-      __builtin_amdgcn_sched_barrier(0);
+      if (FENCED) __builtin_amdgcn_sched_barrier(0);
     }
     // the token loads of step kt + 1 were issued during step kt - 1, before that step's weight loads; in steady state
     // exactly those weight loads and this step's token and weight loads are younger
-    if constexpr (STEADY) vm_wait<2 * WLOADS + XPIECES>();
+    // (a wavefront without weight pieces has only this step's token loads behind them)
+    if constexpr (STEADY) vm_wait<(WLOAD ? 2 * WLOADS : 0) + XPIECES>();
     else vm_wait<0>();
     __syncthreads();
   };
-  auto main_loop = [&](auto active_tag, auto late_tag) {
-    load_w(BigSet<0>{}, 0);
+  auto main_loop = [&](auto active_tag, auto late_tag, auto wload_tag) {
+    constexpr bool WLOAD = decltype(wload_tag)::value;
+    if (WLOAD) load_w(BigSet<0>{}, 0);
     load_x(0, 0);
     if (nkt > 1) {
-      load_w(BigSet<1>{}, 1);
+      if (WLOAD) load_w(BigSet<1>{}, 1);
       load_x(1, 1);
     }
     vm_wait<0>();
-    store_w(BigSet<0>{});
-    if (nkt > 2) load_w(BigSet<0>{}, 2);
+    if (WLOAD) store_w(BigSet<0>{});
+    if (WLOAD && nkt > 2) load_w(BigSet<0>{}, 2);
     __syncthreads();  // everything but the last weight loads has arrived
     int xs = 0;       // kt % 3
     int64_t kt = 0;
     for (; kt + 4 < nkt; kt += 2) {
-      k_step(active_tag, late_tag, BigSet<0>{}, BigTagOn{}, kt, xs);
+      k_step(active_tag, late_tag, wload_tag, BigSet<0>{}, BigTagOn{}, kt, xs);
       xs = xs == 2 ? 0 : xs + 1;
-      k_step(active_tag, late_tag, BigSet<1>{}, BigTagOn{}, kt + 1, xs);
+      k_step(active_tag, late_tag, wload_tag, BigSet<1>{}, BigTagOn{}, kt + 1, xs);
       xs = xs == 2 ? 0 : xs + 1;
     }
     for (; kt < nkt; kt += 2) {
-      k_step(active_tag, late_tag, BigSet<0>{}, BigTagOff{}, kt, xs);
+      k_step(active_tag, late_tag, wload_tag, BigSet<0>{}, BigTagOff{}, kt, xs);
       xs = xs == 2 ? 0 : xs + 1;
       if (kt + 1 < nkt) {
-        k_step(active_tag, late_tag, BigSet<1>{}, BigTagOff{}, kt + 1, xs);
+        k_step(active_tag, late_tag, wload_tag, BigSet<1>{}, BigTagOff{}, kt + 1, xs);
         xs = xs == 2 ? 0 : xs + 1;
       }
     }
@@ -234,11 +250,23 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
   // the next stage while the other feeds the matrix pipe, then they swap, so the vector-ALU and LDS-write work of
   // the producer overlaps MFMAs instead of leaving the matrix pipe idle between barriers.
   const bool late = (wave & 4) != 0;
-  if (active) {
-    if (late) main_loop(BigTagOn{}, BigTagOn{});
-    else main_loop(BigTagOn{}, BigTagOff{});
+  if constexpr (WLOADERS == WN * WM) {
+    if (active) {
+      if (late) main_loop(BigTagOn{}, BigTagOn{}, BigTagOn{});
+      else main_loop(BigTagOn{}, BigTagOff{}, BigTagOn{});
+    } else {
+      main_loop(BigTagOff{}, BigTagOff{}, BigTagOn{});
+    }
   } else {
-    main_loop(BigTagOff{}, BigTagOff{});
+    // narrow form: the wavefronts that convert weight pieces do so before their MFMAs, the others go straight to theirs
+    static_assert(WLOADERS == 4 && WN * WM == 8, "wavefronts 0-3 load weights, one per SIMD");
+    if (wave < WLOADERS) {
+      if (active) main_loop(BigTagOn{}, BigTagOn{}, BigTagOn{});
+      else main_loop(BigTagOff{}, BigTagOff{}, BigTagOn{});
+    } else {
+      if (active) main_loop(BigTagOn{}, BigTagOff{}, BigTagOff{});
+      else main_loop(BigTagOff{}, BigTagOff{}, BigTagOff{});
+    }
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------------
@@ -249,11 +277,11 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
     for (int tj = 0; tj < 4; ++tj) {
       const int r = wm * 64 + tj * 16 + n_in;
       if (r < rows_here) {
-        T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo + (int64_t)ntile * (BN / 2) + wn * 64 + 4 * g;
+        T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo + (int64_t)ntile * (BN / 2) + wn * (WROWS / 2) + 4 * g;
 #pragma unroll
-        for (int ti = 0; ti < 4; ++ti) {
+        for (int ti = 0; ti < TI / 2; ++ti) {
           const float gq[4] = {acc[ti][tj][0], acc[ti][tj][1], acc[ti][tj][2], acc[ti][tj][3]};
-          const float uq[4] = {acc[ti + 4][tj][0], acc[ti + 4][tj][1], acc[ti + 4][tj][2], acc[ti + 4][tj][3]};
+          const float uq[4] = {acc[ti + TI / 2][tj][0], acc[ti + TI / 2][tj][1], acc[ti + TI / 2][tj][2], acc[ti + TI / 2][tj][3]};
           *reinterpret_cast<uint2*>(orow + ti * 16) = gateup_quad<T, ACT>(gq, uq, fq);
         }
       }
@@ -269,20 +297,20 @@ grouped_mfma_big_kernel(GemmParams p, int n_tiles) {
       if (r < rows_here) {
         T* orow = reinterpret_cast<T*>(p.out) + out_row(p, row_begin + r) * p.ldo;
 #pragma unroll
-        for (int ti = 0; ti < 8; ++ti)
-          *reinterpret_cast<uint2*>(orow + (int64_t)ntile * BN + wn * 128 + ti * 16 + 4 * g) =
+        for (int ti = 0; ti < TI; ++ti)
+          *reinterpret_cast<uint2*>(orow + (int64_t)ntile * BN + wn * WROWS + ti * 16 + 4 * g) =
               make_uint2(pack2<T>(acc[ti][tj][0], acc[ti][tj][1]), pack2<T>(acc[ti][tj][2], acc[ti][tj][3]));
       }
     }
   }
 }
 
-template <typename T, int WF, int MODE, int WN, int WM, int STAGES>
+template <typename T, int WF, int MODE, int WN, int WM, int STAGES, int TI = 8>
 static int launch_big_m(const GemmParams& p, int64_t max_rows, hipStream_t st) {
-  constexpr int BN = 128 * WN, BM = 64 * WM;
+  constexpr int BN = 16 * TI * WN, BM = 64 * WM;
   constexpr size_t lds_bytes = (size_t)(2 * BN + 3 * BM) * BIG_LS * 2;
   static std::atomic<uint64_t> lds_ready{0};
-  auto kern = grouped_mfma_big_kernel<T, WF, MODE, WN, WM, STAGES>;
+  auto kern = grouped_mfma_big_kernel<T, WF, MODE, WN, WM, STAGES, TI>;
   if (int rc = reserve_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ready, "mfma big kernel")) return rc;
   const int n_tiles = (int)(MODE == MODE_GATEUP ? p.n_out / (BN / 2) : p.n_out / BN);
   const int experts = p.offsets ? p.E : 1;
@@ -322,6 +350,38 @@ int launch_mfma_big(int act_dtype, int wtag, int mode, const GemmParams& p, int6
   if (act_dtype == STMOE_F16) return launch_big_t<f16_t, WF_Q8_0_P>(mode, p, max_rows, st);
   if (act_dtype == STMOE_BF16) return launch_big_t<bf16_t, WF_Q8_0_P>(mode, p, max_rows, st);
   return set_error(STMOE_ERR_UNSUPPORTED, "mfma big kernel: activation dtype %d", act_dtype);
+}
+
+// The narrow form: 64 weight rows x 256 token rows per workgroup (see the kernel's head).
+#ifndef STMOE_NARROW_TI
+#define STMOE_NARROW_TI 2
+#endif
+template <typename T, int WF>
+static int launch_narrow_t(int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
+  if (mode == MODE_GATEUP) return launch_big_m<T, WF, MODE_GATEUP, 2, 4, 2, STMOE_NARROW_TI>(p, max_rows, st);
+  return launch_big_m<T, WF, MODE_DOWN, 2, 4, 2, STMOE_NARROW_TI>(p, max_rows, st);
+}
+
+int launch_mfma_narrow(int act_dtype, int wtag, int mode, const GemmParams& p, int64_t max_rows, hipStream_t st) {
+  if (max_rows == 0) return STMOE_OK;
+  if (p.offsets && p.E >= 64) return set_error(STMOE_ERR_UNSUPPORTED, "mfma narrow kernel: at most 63 experts");
+  if (p.kred % 256 != 0 || p.lda % 8 != 0 || p.ldo % 4 != 0 || p.n_out % (mode == MODE_GATEUP ? 16 * STMOE_NARROW_TI : 32 * STMOE_NARROW_TI) != 0)
+    return set_error(STMOE_ERR_UNSUPPORTED, "mfma narrow kernel: needs K %% 256 == 0 and output features in whole tiles");
+  {
+    const int64_t src_rows = p.perm ? (max_rows + p.k_top - 1) / p.k_top : max_rows;
+    if (src_rows * p.lda * 2 >= (int64_t)1 << 32)
+      return set_error(STMOE_ERR_UNSUPPORTED, "mfma narrow kernel: activations span 4 GB or more");
+  }
+  if (act_dtype == STMOE_F16) {
+    if (wtag == WF_Q8_0_P) return launch_narrow_t<f16_t, WF_Q8_0_P>(mode, p, max_rows, st);
+    if (wtag == WF_Q4_1_P) return launch_narrow_t<f16_t, WF_Q4_1_P>(mode, p, max_rows, st);
+    if (wtag == WF_FP8_F32D_P) return launch_narrow_t<f16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
+  } else if (act_dtype == STMOE_BF16) {
+    if (wtag == WF_Q8_0_P) return launch_narrow_t<bf16_t, WF_Q8_0_P>(mode, p, max_rows, st);
+    if (wtag == WF_Q4_1_P) return launch_narrow_t<bf16_t, WF_Q4_1_P>(mode, p, max_rows, st);
+    if (wtag == WF_FP8_F32D_P) return launch_narrow_t<bf16_t, WF_FP8_F32D_P>(mode, p, max_rows, st);
+  }
+  return set_error(STMOE_ERR_UNSUPPORTED, "mfma narrow kernel: packed Q8_0, Q4_1 or fp8 weights with fp16 or bf16 activations");
 }
 
 }  // namespace stmoe

@@ -28,6 +28,7 @@ _PACKED_OF = {W_Q8_0: W_Q8_0_PACKED, W_Q4_1: W_Q4_1_PACKED, W_FP8: W_FP8_PACKED}
 VARIANT_AUTO, VARIANT_GENERIC, VARIANT_MFMA_TILE, VARIANT_SKINNY, VARIANT_MFMA_BIG, VARIANT_FP8_MFMA, VARIANT_MFMA_WS = 0, 1, 2, 3, 4, 5, 6
 VARIANT_FP8_TILE = 7
 VARIANT_STEP_BY_STEP = 8  # automatic choice among the kernels that round where the reference rounds (never the fp8 matrix cores)
+VARIANT_MFMA_NARROW = 9  # 64 x 256 tiles: a single matrix with a few hundred rows (chosen automatically where it pays)
 
 _DTYPE_ENUM = {
     torch.float32: F32,

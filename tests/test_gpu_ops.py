@@ -120,15 +120,82 @@ def test_quantized_linear_few_hundred_rows_splits_the_reduction(device, fmt, dty
     assert need > 0 and int(lib.stmoe_mmt_workspace_bytes(32)) == 0
     ws = torch.full((need,), 0xA5, dtype=torch.uint8, device=device)  # stale contents must not matter
     tol = 1e-3 if dtype == torch.float16 else 8e-3
-    plain = _hip.mmt(x.to(device), dw, workspace=torch.empty(0, dtype=torch.uint8, device=device))
+    # (the 256 x 256 kernel is named: from 129 rows on the automatic choice takes this matrix to 64 x 256 tiles, which need
+    # no split; up to 128 rows it is the automatic choice)
+    ws_kernel = _hip.VARIANT_MFMA_WS if M > 128 else _hip.VARIANT_AUTO
+    plain = _hip.mmt(x.to(device), dw, workspace=torch.empty(0, dtype=torch.uint8, device=device), variant=ws_kernel)
     assert O.rel_l2(plain.cpu(), ref) < tol
-    first = _hip.mmt(x.to(device), dw, workspace=ws)
-    second = _hip.mmt(x.to(device), dw, workspace=ws)
+    first = _hip.mmt(x.to(device), dw, workspace=ws, variant=ws_kernel)
+    second = _hip.mmt(x.to(device), dw, workspace=ws, variant=ws_kernel)
     default = _hip.mmt(x.to(device), dw)
     assert O.rel_l2(first.cpu(), ref) < tol
     assert torch.equal(first.view(torch.int16), second.view(torch.int16))
-    assert torch.equal(first.view(torch.int16), default.view(torch.int16))
+    # the binding's own buffer: the split sums again, or (narrow tiles) one running sum per output like `plain`
+    assert torch.equal(default.view(torch.int16), (first if M <= 128 else plain).view(torch.int16))
     assert O.rel_l2(first.float().cpu(), plain.float().cpu()) < (5e-4 if dtype == torch.float16 else 4e-3)
+
+
+@pytest.mark.parametrize("fmt", ["q8_0", "q4_1", "fp8"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_quantized_linear_narrow_tiles(device, fmt, dtype):
+    """A single matrix with a few hundred rows runs on tiles of 64 output features x 256 rows (kernel variant 9): enough
+    tiles for the CUs without cutting the reduction.  Against the oracle's dense product, bit for bit against the
+    128 x 128 tile kernel (both keep one fp32 running sum per output, in the same order), and as the automatic choice from
+    129 rows on; ragged row counts on both sides of the 256-row tile; a matrix whose feature count is no multiple of 64
+    goes to the other kernels."""
+    import moe_cases as MC
+    from sharktank_amd import _hip
+    from sharktank_amd.ops import device_weight
+
+    K, N = 1024, 448  # 7 feature tiles
+    case = MC.build(MC.Case(T=4, K=K, N=N, E=1, k=1, fmt=fmt, dtype=dtype, seed=410))
+    dw = device_weight(MC.to_inference_tensor(fmt, case.planes["gate"], [1, N, K], "w", device), stacked=True, prepack=True)
+    wd = MC.dense_weights(case)[0][0].to(dtype)
+    tol = 1e-3 if dtype == torch.float16 else 8e-3
+    for M in (1, 64, 129, 200, 255, 256, 257, 300, 512, 700):
+        x = (torch.randn(M, K, generator=torch.Generator().manual_seed(M)) * 0.5).to(dtype)
+        ref = O.mmt(x, wd)
+        narrow = _hip.mmt(x.to(device), dw, variant=_hip.VARIANT_MFMA_NARROW)
+        tile = _hip.mmt(x.to(device), dw, variant=_hip.VARIANT_MFMA_TILE)
+        assert torch.isfinite(narrow.float()).all()
+        assert O.rel_l2(narrow.cpu(), ref) < tol, (M, O.rel_l2(narrow.cpu(), ref))
+        assert torch.equal(narrow.view(torch.int16), tile.view(torch.int16)), M
+        if M > 128:
+            assert torch.equal(_hip.mmt(x.to(device), dw).view(torch.int16), narrow.view(torch.int16)), M
+    # 96 output features: no whole 64-feature tiles, the request falls through to the kernels that take the shape
+    case = MC.build(MC.Case(T=4, K=K, N=96, E=1, k=1, fmt=fmt, dtype=dtype, seed=411))
+    dw = device_weight(MC.to_inference_tensor(fmt, case.planes["gate"], [1, 96, K], "w", device), stacked=True, prepack=True)
+    x = (torch.randn(200, K, generator=torch.Generator().manual_seed(5)) * 0.5).to(dtype)
+    got = _hip.mmt(x.to(device), dw, variant=_hip.VARIANT_MFMA_NARROW)
+    assert O.rel_l2(got.cpu(), O.mmt(x, MC.dense_weights(case)[0][0].to(dtype))) < tol
+
+
+@pytest.mark.parametrize("fmt,dtype", [("q8_0", torch.float16), ("q4_1", torch.bfloat16)])
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_gated_ffn_on_narrow_tiles(device, fmt, dtype, act):
+    """The gated form of the narrow tiles (32 gate + the same 32 up features x 256 rows, the gated product formed in
+    registers) and the down projection on them: one expert through the grouped FFN with kernel variant 9 named, against the
+    oracle's down(act(gate x) * up x) and against the 128 x 128 tile kernel."""
+    import moe_cases as MC
+    from sharktank_amd import _hip
+    from sharktank_amd.ops import device_weight
+
+    K, N = 512, 768
+    case = MC.build(MC.Case(T=4, K=K, N=N, E=1, k=1, fmt=fmt, dtype=dtype, act=act, seed=420))
+    dws = [device_weight(MC.to_inference_tensor(fmt, case.planes[n], shape, n, device), stacked=True, prepack=True)
+           for n, shape in (("gate", [1, N, K]), ("up", [1, N, K]), ("down", [1, K, N]))]
+    dense = MC.dense_weights(case)
+    wg, wu, wdn = (dense[i][0].to(dtype) for i in range(3))
+    fn = torch.nn.functional.silu if act == "silu" else torch.nn.functional.gelu
+    act_id = _hip.ACT_SILU if act == "silu" else _hip.ACT_GELU_ERF
+    for M in (130, 256, 300, 513):
+        x = (torch.randn(M, K, generator=torch.Generator().manual_seed(M))).to(dtype)
+        want = O._mm_rt(fn(O._mm_rt(x, wg)) * O._mm_rt(x, wu), wdn)
+        got = _hip.grouped_ffn(x.to(device), *dws, act_id, None, None, 1, variant=_hip.VARIANT_MFMA_NARROW)
+        tile = _hip.grouped_ffn(x.to(device), *dws, act_id, None, None, 1, variant=_hip.VARIANT_MFMA_TILE)
+        assert torch.isfinite(got.float()).all()
+        assert O.rel_l2(got.cpu(), want) < (1e-3 if dtype == torch.float16 else 8e-3), (M, O.rel_l2(got.cpu(), want))
+        assert O.rel_l2(got.float().cpu(), tile.float().cpu()) < (2e-4 if dtype == torch.float16 else 4e-3)
 
 
 def test_quantized_linear_split_reduction_under_hip_graph_capture(device):
